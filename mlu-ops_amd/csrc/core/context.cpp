@@ -1,0 +1,167 @@
+// Handle management: mluOpCreate / Destroy / SetQueue / GetQueue and the
+// small per-handle switches.  Behaviour follows reference
+// core/context.cpp:158-470; the MLU attribute reads become a read of the HIP
+// device properties and the queue is a hipStream_t.
+#include <cstdlib>
+#include <cstring>
+#include <new>
+
+#include "core/core.h"
+
+namespace {
+
+int parseGfxNumber(const char *name) {
+  // "gfx950:sramecc+:xnack-" -> 950 ; "gfx90a" -> 0x90a is not needed here,
+  // only gfx950 is a supported target, so a decimal parse is enough.
+  const char *p = strstr(name, "gfx");
+  if (p == nullptr) return 0;
+  return atoi(p + 3);
+}
+
+bool hostOnlyHandleRequested() {
+  const char *v = getenv("MLUOP_HOST_ONLY_HANDLE");
+  return v != nullptr && v[0] == '1';
+}
+
+}  // namespace
+
+extern "C" {
+
+mluOpStatus_t MLUOP_WIN_API mluOpCreate(mluOpHandle_t *handle) {
+  PARAM_CHECK("[mluOpCreate]", handle != NULL);
+  mluOpContext *ctx = new (std::nothrow) mluOpContext();
+  if (ctx == nullptr) return MLUOP_STATUS_ALLOC_FAILED;
+
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) {
+    (void)hipGetLastError();
+    if (hostOnlyHandleRequested()) {
+      // A handle for exercising descriptor logic and parameter checks on a
+      // machine without a GPU.  It reports the supported architecture so the
+      // checks behind the architecture gate can be reached; every operator
+      // returns EXECUTION_FAILED before it would launch anything.
+      ctx->device = -1;
+      ctx->arch = 950;
+      *handle = ctx;
+      return MLUOP_STATUS_SUCCESS;
+    }
+    MLUOP_LOG(ERROR) << "[mluOpCreate] no usable HIP device: " << hipGetErrorString(err);
+    delete ctx;
+    return MLUOP_STATUS_INTERNAL_ERROR;
+  }
+  hipDeviceProp_t prop;
+  err = hipGetDeviceProperties(&prop, dev);
+  if (err != hipSuccess) {
+    MLUOP_LOG(ERROR) << "[mluOpCreate] hipGetDeviceProperties failed: " << hipGetErrorString(err);
+    delete ctx;
+    return MLUOP_STATUS_INTERNAL_ERROR;
+  }
+  ctx->device = dev;
+  ctx->arch = parseGfxNumber(prop.gcnArchName);
+  ctx->cu_count = prop.multiProcessorCount;
+  ctx->lds_bytes = (int)prop.sharedMemPerBlock;
+  void *pinned = nullptr;
+  err = hipHostMalloc(&pinned, 64, hipHostMallocDefault);
+  if (err != hipSuccess) {
+    MLUOP_LOG(ERROR) << "[mluOpCreate] hipHostMalloc failed: " << hipGetErrorString(err);
+    delete ctx;
+    return MLUOP_STATUS_ALLOC_FAILED;
+  }
+  ctx->pinned_scalar = static_cast<int32_t *>(pinned);
+  *handle = ctx;
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpDestroy(mluOpHandle_t handle) {
+  PARAM_CHECK("[mluOpDestroy]", handle != NULL);
+  if (handle->pinned_scalar != nullptr) (void)hipHostFree(handle->pinned_scalar);
+  delete handle;
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpSetQueue(mluOpHandle_t handle, mluOpQueue_t queue) {
+  PARAM_CHECK("[mluOpSetQueue]", handle != NULL);
+  handle->queue = reinterpret_cast<hipStream_t>(queue);  // NULL is allowed
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpGetQueue(mluOpHandle_t handle, mluOpQueue_t *queue) {
+  PARAM_CHECK("[mluOpGetQueue]", handle != NULL);
+  PARAM_CHECK("[mluOpGetQueue]", queue != NULL);
+  *queue = reinterpret_cast<mluOpQueue_t>(handle->queue);
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpSetQuantizeRoundMode(mluOpHandle_t handle,
+                                                      mluOpQuantizeRoundMode_t round_mode) {
+  PARAM_CHECK("[mluOpSetQuantizeRoundMode]", handle != NULL);
+  PARAM_CHECK("[mluOpSetQuantizeRoundMode]", round_mode == MLUOP_ROUND_HALF_TO_EVEN ||
+                                                 round_mode == MLUOP_ROUND_HALF_OFF_ZERO ||
+                                                 round_mode == MLUOP_ROUND_HALF_UP);
+  handle->round_mode = round_mode;
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpGetQuantizeRoundMode(mluOpHandle_t handle,
+                                                      mluOpQuantizeRoundMode_t *round_mode) {
+  PARAM_CHECK("[mluOpGetQuantizeRoundMode]", handle != NULL);
+  PARAM_CHECK("[mluOpGetQuantizeRoundMode]", round_mode != NULL);
+  *round_mode = handle->round_mode;
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpSetAtomicsMode(mluOpHandle_t handle,
+                                                mluOpAtomicsMode_t atomics_mode) {
+  PARAM_CHECK("[mluOpSetAtomicsMode]", handle != NULL);
+  handle->atomics_mode = atomics_mode;
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpGetAtomicsMode(mluOpHandle_t handle,
+                                                mluOpAtomicsMode_t *atomics_mode) {
+  PARAM_CHECK("[mluOpGetAtomicsMode]", handle != NULL);
+  PARAM_CHECK("[mluOpGetAtomicsMode]", atomics_mode != NULL);
+  *atomics_mode = handle->atomics_mode;
+  return MLUOP_STATUS_SUCCESS;
+}
+
+void MLUOP_WIN_API mluOpGetLibVersion(int *major, int *minor, int *patch) {
+  if (major) *major = MLUOP_MAJOR;
+  if (minor) *minor = MLUOP_MINOR;
+  if (patch) *patch = MLUOP_PATCHLEVEL;
+}
+
+const char *MLUOP_WIN_API mluOpGetErrorString(mluOpStatus_t status) {
+  switch (status) {
+    case MLUOP_STATUS_SUCCESS: return "MLUOP_STATUS_SUCCESS";
+    case MLUOP_STATUS_NOT_INITIALIZED: return "MLUOP_STATUS_NOT_INITIALIZED";
+    case MLUOP_STATUS_ALLOC_FAILED: return "MLUOP_STATUS_ALLOC_FAILED";
+    case MLUOP_STATUS_BAD_PARAM: return "MLUOP_STATUS_BAD_PARAM";
+    case MLUOP_STATUS_INTERNAL_ERROR: return "MLUOP_STATUS_INTERNAL_ERROR";
+    case MLUOP_STATUS_ARCH_MISMATCH: return "MLUOP_STATUS_ARCH_MISMATCH";
+    case MLUOP_STATUS_EXECUTION_FAILED: return "MLUOP_STATUS_EXECUTION_FAILED";
+    case MLUOP_STATUS_NOT_SUPPORTED: return "MLUOP_STATUS_NOT_SUPPORTED";
+    case MLUOP_STATUS_NUMERICAL_OVERFLOW: return "MLUOP_STATUS_NUMERICAL_OVERFLOW";
+  }
+  return "MLUOP_STATUS_UNKNOWN";
+}
+
+}  // extern "C"
+
+namespace mluop {
+
+bool logEnabled() {
+  static const bool enabled = [] {
+    const char *v = getenv("MLUOP_LOG_PRINT");
+    return !(v != nullptr && v[0] == '0');
+  }();
+  return enabled;
+}
+
+void logLine(const char *level, const std::string &msg) {
+  if (!logEnabled()) return;
+  fprintf(stderr, "[mluop][%s] %s\n", level, msg.c_str());
+}
+
+}  // namespace mluop

@@ -1,0 +1,56 @@
+// Host-side interface of the indice-convolution kernel set (forward,
+// backward data, backward filter).
+#ifndef MLUOP_AMD_SPARSE_CONV_INDICE_CONV_H_
+#define MLUOP_AMD_SPARSE_CONV_INDICE_CONV_H_
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace mluop {
+namespace sparse_conv {
+
+enum class ElemType { kHalf, kBFloat16, kFloat };
+
+inline size_t elemSize(ElemType t) { return t == ElemType::kFloat ? 4 : 2; }
+
+// A filter tensor seen as W(k, ci, co) = base[k*stride_k + ci*stride_ci + co*stride_co]
+// (element strides), which covers every accepted filter layout without a
+// transposed copy.
+struct FilterView {
+  const void *base;
+  int64_t stride_k;
+  int64_t stride_ci;
+  int64_t stride_co;
+};
+
+struct ConvProblem {
+  ElemType dtype;
+  int K;          // kernel volume = indice_pairs.dim[0]
+  int L;          // indice_pairs.dim[2] = rows of the input-side tensor
+  int num_out;    // rows of the output-side tensor
+  int Ci;
+  int Co;
+  const int32_t *indice_pairs;  // device [K, 2, L]
+  const int64_t *indice_num;    // host [K]
+};
+
+// Which of the two gather-GEMM directions a launch computes.
+//   kForward:      rows = output rows,  gathered = features,    B = W[k]
+//   kBackwardData: rows = input rows,   gathered = output_grad, B = W[k]^T
+enum class GatherDirection { kForward, kBackwardData };
+
+size_t gatherConvWorkspaceBytes(const ConvProblem &p, GatherDirection dir);
+hipError_t launchGatherConv(hipStream_t stream, const ConvProblem &p, GatherDirection dir,
+                            const void *gathered, const FilterView &filters, void *workspace,
+                            void *result);
+
+size_t backwardFilterWorkspaceBytes(const ConvProblem &p);
+hipError_t launchBackwardFilter(hipStream_t stream, const ConvProblem &p, const void *features,
+                                const void *output_grad, void *workspace, void *filters_grad);
+
+}  // namespace sparse_conv
+}  // namespace mluop
+
+#endif  // MLUOP_AMD_SPARSE_CONV_INDICE_CONV_H_

@@ -1,0 +1,217 @@
+// mluOpIndiceConvolutionBackwardFilter and its workspace query.  Checks follow
+// the order and status codes of reference
+// kernels/sparse_conv/indice_convolution_backward_filter/
+// indice_convolution_backward_filter.cpp:100-258 and :536-620; bfloat16 is
+// accepted in addition to half and float.
+#include <string>
+
+#include "core/core.h"
+#include "sparse_conv/indice_conv.h"
+
+namespace {
+
+using mluop::sparse_conv::ConvProblem;
+using mluop::sparse_conv::ElemType;
+
+bool isFloatDtype(mluOpDataType_t t) {
+  return t == MLUOP_DTYPE_HALF || t == MLUOP_DTYPE_FLOAT || t == MLUOP_DTYPE_BFLOAT16;
+}
+
+ElemType toElemType(mluOpDataType_t t) {
+  return t == MLUOP_DTYPE_FLOAT ? ElemType::kFloat
+                                : (t == MLUOP_DTYPE_HALF ? ElemType::kHalf : ElemType::kBFloat16);
+}
+
+mluOpStatus_t dtypeValid(const std::string &api, const mluOpTensorDescriptor_t features_desc,
+                         const mluOpTensorDescriptor_t output_grad_desc,
+                         const mluOpTensorDescriptor_t indice_pairs_desc,
+                         const mluOpTensorDescriptor_t filters_grad_desc) {
+  const mluOpDataType_t input_dtype = features_desc->getDtype();
+  const mluOpDataType_t diffy_dtype = output_grad_desc->getDtype();
+  const mluOpDataType_t filters_grad_dtype = filters_grad_desc->getDtype();
+  const mluOpDataType_t pairs_dtype = indice_pairs_desc->getDtype();
+  if (pairs_dtype != MLUOP_DTYPE_INT32) {
+    MLUOP_LOG(ERROR) << api << " indice_pairs_desc only supports data type int32, now "
+                     << mluop::getNameOfDataType(pairs_dtype) << ".";
+    return MLUOP_STATUS_BAD_PARAM;
+  }
+  if (input_dtype != diffy_dtype || input_dtype != filters_grad_dtype ||
+      !isFloatDtype(input_dtype) || !isFloatDtype(diffy_dtype) ||
+      !isFloatDtype(filters_grad_dtype)) {
+    MLUOP_LOG(ERROR) << api << " The data type of features_desc, output_grad_desc and "
+                     << "filters_grad_desc should be the same floating-point type. Now "
+                     << mluop::getNameOfDataType(input_dtype) << "-"
+                     << mluop::getNameOfDataType(diffy_dtype) << "-"
+                     << mluop::getNameOfDataType(filters_grad_dtype) << ".";
+    return MLUOP_STATUS_BAD_PARAM;
+  }
+  const mluOpDataType_t input_on = features_desc->getOnchipDtype();
+  const mluOpDataType_t diffy_on = output_grad_desc->getOnchipDtype();
+  const mluOpDataType_t grad_on = filters_grad_desc->getOnchipDtype();
+  const mluOpDataType_t pairs_on = indice_pairs_desc->getOnchipDtype();
+  if ((input_on != MLUOP_DTYPE_INVALID && input_on != input_dtype) ||
+      (diffy_on != MLUOP_DTYPE_INVALID && diffy_on != diffy_dtype) ||
+      (pairs_on != MLUOP_DTYPE_INVALID && pairs_on != pairs_dtype)) {
+    MLUOP_LOG(ERROR) << api << " For features_desc, output_grad_desc and indice_pairs_desc the "
+                     << "on-chip data type, when set, must equal the off-chip data type.";
+    return MLUOP_STATUS_BAD_PARAM;
+  }
+  if ((grad_on != MLUOP_DTYPE_INVALID && !isFloatDtype(grad_on)) ||
+      (filters_grad_dtype == MLUOP_DTYPE_FLOAT && grad_on == MLUOP_DTYPE_HALF)) {
+    MLUOP_LOG(ERROR) << api << " The on-chip data type of filters_grad_desc, when set, must be a "
+                     << "floating-point type at least as wide as the off-chip data type.";
+    return MLUOP_STATUS_BAD_PARAM;
+  }
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t baseParamCheck(const std::string &api, mluOpHandle_t handle,
+                             const mluOpTensorDescriptor_t features_desc,
+                             const mluOpTensorDescriptor_t output_grad_desc,
+                             const mluOpTensorDescriptor_t indice_pairs_desc,
+                             const mluOpTensorDescriptor_t filters_grad_desc,
+                             const int64_t indice_num[], const int64_t inverse) {
+  PARAM_CHECK(api, handle != nullptr);
+  PARAM_CHECK(api, features_desc != nullptr);
+  PARAM_CHECK(api, output_grad_desc != nullptr);
+  PARAM_CHECK(api, indice_pairs_desc != nullptr);
+  PARAM_CHECK(api, filters_grad_desc != nullptr);
+  PARAM_CHECK(api, indice_num != nullptr);
+  PARAM_CHECK(api, inverse == 0);
+
+  STRIDE_TENSOR_CHECK(api, features_desc, "features_desc must be contiguous");
+  STRIDE_TENSOR_CHECK(api, output_grad_desc, "output_grad_desc must be contiguous");
+  STRIDE_TENSOR_CHECK(api, indice_pairs_desc, "indice_pairs_desc must be contiguous");
+  STRIDE_TENSOR_CHECK(api, filters_grad_desc, "filters_grad_desc must be contiguous");
+
+  if (handle->arch != 950) {
+    MLUOP_LOG(ERROR) << api << " Only gfx950 devices are supported.";
+    return MLUOP_STATUS_ARCH_MISMATCH;
+  }
+
+  mluOpStatus_t st =
+      dtypeValid(api, features_desc, output_grad_desc, indice_pairs_desc, filters_grad_desc);
+  if (st != MLUOP_STATUS_SUCCESS) return st;
+
+  if (mluOpGetTensorElementNum(features_desc) >= LARGE_TENSOR_NUM ||
+      mluOpGetTensorElementNum(output_grad_desc) >= LARGE_TENSOR_NUM ||
+      mluOpGetTensorElementNum(indice_pairs_desc) >= LARGE_TENSOR_NUM ||
+      mluOpGetTensorElementNum(filters_grad_desc) >= LARGE_TENSOR_NUM) {
+    MLUOP_LOG(ERROR) << api << " Overflow max tensor num: tensors must hold fewer than 2^31 "
+                     << "elements.";
+    return MLUOP_STATUS_NOT_SUPPORTED;
+  }
+  bool shape_check = true;
+  if (2 != features_desc->getDim() || 2 != output_grad_desc->getDim() ||
+      3 != indice_pairs_desc->getDim() ||
+      (4 != filters_grad_desc->getDim() && 5 != filters_grad_desc->getDim())) {
+    shape_check = false;
+  }
+  if (shape_check) {
+    // filters_grad is (kd,)kh,kw,Ci,Co positionally, whatever its layout tag.
+    const int n = filters_grad_desc->getDim();
+    const int64_t ci = filters_grad_desc->getDimIndex(n - 2);
+    const int64_t co = filters_grad_desc->getDimIndex(n - 1);
+    const int64_t kd = n == 4 ? 1 : filters_grad_desc->getDimIndex(0);
+    const int64_t kh = n == 4 ? filters_grad_desc->getDimIndex(0) : filters_grad_desc->getDimIndex(1);
+    const int64_t kw = n == 4 ? filters_grad_desc->getDimIndex(1) : filters_grad_desc->getDimIndex(2);
+    if (ci != features_desc->getDimIndex(1) || co != output_grad_desc->getDimIndex(1) ||
+        features_desc->getDimIndex(0) != indice_pairs_desc->getDimIndex(2) ||
+        2 != indice_pairs_desc->getDimIndex(1) ||
+        kd * kh * kw != indice_pairs_desc->getDimIndex(0)) {
+      shape_check = false;
+    }
+    PARAM_CHECK_LE(api, indice_pairs_desc->getDimIndex(2), INDICE_IN_LARGE_TENSOR_NUM);
+  }
+  if (!shape_check) {
+    MLUOP_LOG(ERROR) << api << " Shape check failed!";
+    return MLUOP_STATUS_BAD_PARAM;
+  }
+  return MLUOP_STATUS_SUCCESS;
+}
+
+bool anyZeroElement(const mluOpTensorDescriptor_t a, const mluOpTensorDescriptor_t b,
+                    const mluOpTensorDescriptor_t c, const mluOpTensorDescriptor_t d) {
+  return a->getTotalElementNum() == 0 || b->getTotalElementNum() == 0 ||
+         c->getTotalElementNum() == 0 || d->getTotalElementNum() == 0;
+}
+
+ConvProblem makeProblem(const mluOpTensorDescriptor_t features_desc,
+                        const mluOpTensorDescriptor_t output_grad_desc,
+                        const mluOpTensorDescriptor_t indice_pairs_desc,
+                        const int64_t indice_num[], const void *indice_pairs) {
+  ConvProblem p;
+  p.dtype = toElemType(features_desc->getDtype());
+  p.K = (int)indice_pairs_desc->getDimIndex(0);
+  p.L = (int)indice_pairs_desc->getDimIndex(2);
+  p.num_out = (int)output_grad_desc->getDimIndex(0);
+  p.Ci = (int)features_desc->getDimIndex(1);
+  p.Co = (int)output_grad_desc->getDimIndex(1);
+  p.indice_pairs = static_cast<const int32_t *>(indice_pairs);
+  p.indice_num = indice_num;
+  return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+mluOpStatus_t MLUOP_WIN_API mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize(
+    mluOpHandle_t handle, const mluOpTensorDescriptor_t features_desc,
+    const mluOpTensorDescriptor_t output_grad_desc,
+    const mluOpTensorDescriptor_t indice_pairs_desc,
+    const mluOpTensorDescriptor_t filters_grad_desc, const int64_t indice_num[],
+    const int64_t inverse, const int64_t subm, size_t *size) {
+  const std::string api = "[mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize]";
+  (void)subm;
+  PARAM_CHECK(api, size != nullptr);
+  mluOpStatus_t st = baseParamCheck(api, handle, features_desc, output_grad_desc,
+                                    indice_pairs_desc, filters_grad_desc, indice_num, inverse);
+  if (st != MLUOP_STATUS_SUCCESS) return st;
+  if (anyZeroElement(features_desc, output_grad_desc, indice_pairs_desc, filters_grad_desc)) {
+    return MLUOP_STATUS_SUCCESS;
+  }
+  const ConvProblem p =
+      makeProblem(features_desc, output_grad_desc, indice_pairs_desc, indice_num, nullptr);
+  *size = mluop::sparse_conv::backwardFilterWorkspaceBytes(p);
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardFilter(
+    mluOpHandle_t handle, const mluOpTensorDescriptor_t features_desc, const void *features,
+    const mluOpTensorDescriptor_t output_grad_desc, const void *output_grad,
+    const mluOpTensorDescriptor_t indice_pairs_desc, const void *indice_pairs,
+    const int64_t indice_num[], const int64_t inverse, const int64_t subm, void *workspace,
+    size_t workspace_size, const mluOpTensorDescriptor_t filters_grad_desc, void *filters_grad) {
+  const std::string api = "[mluOpIndiceConvolutionBackwardFilter]";
+  (void)subm;
+  mluOpStatus_t st = baseParamCheck(api, handle, features_desc, output_grad_desc,
+                                    indice_pairs_desc, filters_grad_desc, indice_num, inverse);
+  if (st != MLUOP_STATUS_SUCCESS) return st;
+  if (anyZeroElement(features_desc, output_grad_desc, indice_pairs_desc, filters_grad_desc)) {
+    return MLUOP_STATUS_SUCCESS;
+  }
+  PARAM_CHECK(api, features != nullptr);
+  PARAM_CHECK(api, output_grad != nullptr);
+  PARAM_CHECK(api, indice_pairs != nullptr);
+  PARAM_CHECK(api, filters_grad != nullptr);
+  if (workspace_size > 0) {
+    PARAM_CHECK(api, workspace != nullptr);
+  }
+  const ConvProblem p =
+      makeProblem(features_desc, output_grad_desc, indice_pairs_desc, indice_num, indice_pairs);
+  const size_t need = mluop::sparse_conv::backwardFilterWorkspaceBytes(p);
+  if (workspace_size < need || (need > 0 && workspace == nullptr)) {
+    MLUOP_LOG(ERROR) << api << " workspace of " << workspace_size
+                     << " bytes is smaller than the " << need
+                     << " bytes mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize reports.";
+    return MLUOP_STATUS_BAD_PARAM;
+  }
+  DEVICE_HANDLE_CHECK(api, handle);
+  HIP_CHECK_RETURN(api, mluop::sparse_conv::launchBackwardFilter(handle->queue, p, features,
+                                                                output_grad, workspace,
+                                                                filters_grad));
+  return MLUOP_STATUS_SUCCESS;
+}
+
+}  // extern "C"

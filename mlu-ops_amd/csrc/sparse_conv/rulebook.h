@@ -1,0 +1,47 @@
+// Host-side interface of the rulebook (indice pairs) kernel set.
+#ifndef MLUOP_AMD_SPARSE_CONV_RULEBOOK_H_
+#define MLUOP_AMD_SPARSE_CONV_RULEBOOK_H_
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace mluop {
+namespace sparse_conv {
+
+// Geometry of one sparse convolution, axes in (d, h, w) order.
+struct RulebookGeom {
+  int batch;
+  int in_space[3];
+  int out_space[3];
+  int ksize[3];
+  int pad[3];
+  int stride[3];
+  int dilation[3];
+  int K;         // kernel volume
+  int L;         // active input rows
+  int out_rows;  // rows of the caller's out_indices tensor (M)
+  bool sub_m;
+};
+
+// Bytes of device workspace the kernel set needs for this geometry.
+size_t rulebookWorkspaceBytes(const RulebookGeom &g);
+
+// Enqueues submanifold rulebook construction on `stream`.
+hipError_t launchSubmRulebook(hipStream_t stream, const RulebookGeom &g, const int32_t *indices,
+                              void *workspace, int32_t *indice_pairs, int32_t *out_indices,
+                              int32_t *indice_num);
+
+// Enqueues regular (strided / dilated) rulebook construction on `stream` and
+// an asynchronous copy of the number of active outputs into `host_num_act_out`
+// (pinned host memory).  The caller synchronises the stream before reading it.
+hipError_t launchRegularRulebook(hipStream_t stream, const RulebookGeom &g,
+                                 const int32_t *indices, void *workspace, int32_t *indice_pairs,
+                                 int32_t *out_indices, int32_t *indice_num,
+                                 int32_t *host_num_act_out);
+
+}  // namespace sparse_conv
+}  // namespace mluop
+
+#endif  // MLUOP_AMD_SPARSE_CONV_RULEBOOK_H_

@@ -1,0 +1,473 @@
+// Rulebook (indice pairs) construction for 3-D sparse convolution on gfx950.
+//
+// Contract (reference test/mlu_op_gtest/pb_gtest/src/zoo/get_indice_pairs/
+// get_indice_pairs.cpp:234-406): for input row j = (n, d, h, w) and kernel
+// offset k = (kd*KH + kh)*KW + kw the output coordinate along each axis is
+// o = (i + pad - k_axis*dilation) / stride, valid when the division is exact
+// and 0 <= o < O_axis.  Submanifold mode keeps a pair when some input row sits
+// at the output coordinate (output row = that input row, the highest row index
+// wins for duplicated coordinates); regular mode keeps every valid pair and
+// numbers the distinct output cells in ascending linear order.  Inside one
+// offset, pairs are listed by ascending input row; unused tails are -1.
+//
+// Kernel set
+//   submanifold:  clear hash -> insert rows -> probe (one wavefront per 64
+//                 rows, per-wave pair counts) -> scan counts per offset ->
+//                 emit (wave-ballot ranks, coalesced pair writes, -1 tails)
+//   regular:      clear bitmap -> mark output cells + record candidates ->
+//                 scan counts -> bitmap popcount scan (ranks, out_indices) ->
+//                 emit with rank lookup
+// The stable order needs no sort: rows are visited in ascending order by
+// construction (lane = row) and positions come from exclusive prefix sums.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "sparse_conv/rulebook.h"
+
+namespace mluop {
+namespace sparse_conv {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWave = 64;
+constexpr unsigned long long kEmptySlot = ~0ull;
+constexpr int kWordsPerBlock = 1024;  // bitmap words (64 cells each) per block
+
+struct GeomDev {
+  int batch;
+  int out[3];
+  int ks[3];
+  int pad[3];
+  int stride[3];
+  int dil[3];
+  int K;
+  int L;
+};
+
+__device__ __forceinline__ uint32_t hashCell(uint32_t key) {
+  uint32_t h = key * 0x9E3779B1u;
+  return h ^ (h >> 15);
+}
+
+__device__ __forceinline__ int4 loadCoord(const int32_t *indices, int j, bool aligned) {
+  if (aligned) return reinterpret_cast<const int4 *>(indices)[j];
+  const int32_t *p = indices + 4 * (size_t)j;
+  return make_int4(p[0], p[1], p[2], p[3]);
+}
+
+__device__ __forceinline__ void storeCoord(int32_t *dst, int j, int4 v, bool aligned) {
+  if (aligned) {
+    reinterpret_cast<int4 *>(dst)[j] = v;
+  } else {
+    int32_t *p = dst + 4 * (size_t)j;
+    p[0] = v.x; p[1] = v.y; p[2] = v.z; p[3] = v.w;
+  }
+}
+
+// Output coordinate along one axis; -1 when this (input, offset) has none.
+__device__ __forceinline__ int axisOut(int i, int pad, int kk, int dil, int stride, int osize) {
+  int num = i + pad - kk * dil;
+  if (num < 0) return -1;
+  int o = num;
+  if (stride != 1) {
+    o = num / stride;
+    if (o * stride != num) return -1;
+  }
+  return o < osize ? o : -1;
+}
+
+__global__ __launch_bounds__(kBlock) void rbFill64(unsigned long long *dst, size_t n,
+                                                   unsigned long long value) {
+  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * kBlock;
+  for (; i < n; i += stride) dst[i] = value;
+}
+
+// Inserts every row's linear cell index into the open-addressing table (slot =
+// cell << 32 | row; 64-bit max keeps the highest row for a duplicated cell) and
+// copies indices to out_indices, padding rows beyond L with -1.
+__global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t *indices,
+                                                       bool aligned, unsigned long long *table,
+                                                       uint32_t mask, int32_t *out_indices,
+                                                       int out_rows) {
+  int j = blockIdx.x * kBlock + threadIdx.x;
+  if (j < g.L) {
+    int4 c = loadCoord(indices, j, aligned);
+    if (j < out_rows) storeCoord(out_indices, j, c, aligned);
+    bool in_range = (unsigned)c.x < (unsigned)g.batch && (unsigned)c.y < (unsigned)g.out[0] &&
+                    (unsigned)c.z < (unsigned)g.out[1] && (unsigned)c.w < (unsigned)g.out[2];
+    if (in_range) {
+      uint32_t cell = (uint32_t)(((c.x * g.out[0] + c.y) * g.out[1] + c.z) * g.out[2] + c.w);
+      unsigned long long packed = ((unsigned long long)cell << 32) | (uint32_t)j;
+      uint32_t slot = hashCell(cell) & mask;
+      while (true) {
+        unsigned long long old = atomicCAS(&table[slot], kEmptySlot, packed);
+        if (old == kEmptySlot) break;
+        if ((uint32_t)(old >> 32) == cell) {
+          atomicMax(&table[slot], packed);
+          break;
+        }
+        slot = (slot + 1) & mask;
+      }
+    }
+  } else if (j < out_rows) {
+    storeCoord(out_indices, j, make_int4(-1, -1, -1, -1), aligned);
+  }
+}
+
+__device__ __forceinline__ int tableLookup(const unsigned long long *table, uint32_t mask,
+                                           uint32_t cell) {
+  uint32_t slot = hashCell(cell) & mask;
+  while (true) {
+    unsigned long long e = table[slot];
+    if (e == kEmptySlot) return -1;
+    if ((uint32_t)(e >> 32) == cell) return (int)(uint32_t)e;
+    slot = (slot + 1) & mask;
+  }
+}
+
+// One wavefront per 64 consecutive rows.  For every offset: resolve the pair
+// (submanifold: table lookup -> output row; regular: output cell, marked in the
+// bitmap), store it as a candidate at [k][row] and record how many lanes of the
+// wave produced one.
+template <bool SUBM>
+__global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, const int32_t *indices,
+                                                       bool aligned,
+                                                       const unsigned long long *table,
+                                                       uint32_t mask, unsigned long long *bitmap,
+                                                       int32_t *cand, int32_t *counts, int n_wave) {
+  const int j = blockIdx.x * kBlock + threadIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wt = j >> 6;
+  if (wt >= n_wave) return;  // whole wave beyond the last row
+  const bool active = j < g.L;
+  int4 c = make_int4(-1, 0, 0, 0);
+  if (active) c = loadCoord(indices, j, aligned);
+  const bool n_ok = active && (unsigned)c.x < (unsigned)g.batch;
+  int k = 0;
+  for (int kd = 0; kd < g.ks[0]; ++kd) {
+    const int od = axisOut(c.y, g.pad[0], kd, g.dil[0], g.stride[0], g.out[0]);
+    for (int kh = 0; kh < g.ks[1]; ++kh) {
+      const int oh = axisOut(c.z, g.pad[1], kh, g.dil[1], g.stride[1], g.out[1]);
+      for (int kw = 0; kw < g.ks[2]; ++kw, ++k) {
+        const int ow = axisOut(c.w, g.pad[2], kw, g.dil[2], g.stride[2], g.out[2]);
+        int r = -1;
+        if (n_ok && (od | oh | ow) >= 0) {
+          const uint32_t cell =
+              (uint32_t)(((c.x * g.out[0] + od) * g.out[1] + oh) * g.out[2] + ow);
+          if (SUBM) {
+            r = tableLookup(table, mask, cell);
+          } else {
+            r = (int)cell;
+            const unsigned long long bit = 1ull << (cell & 63);
+            unsigned long long *word = bitmap + (cell >> 6);
+            if ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & bit) == 0)
+              atomicOr(word, bit);
+          }
+        }
+        if (active) cand[(size_t)k * g.L + j] = r;
+        const unsigned long long b = __ballot(r >= 0);
+        if (lane == 0) counts[(size_t)k * n_wave + wt] = __popcll(b);
+      }
+    }
+  }
+}
+
+// Exclusive prefix sum over `n` ints per row of `data` (one block per row), the
+// row total goes to totals[row].
+__global__ __launch_bounds__(kBlock) void rbScanRows(int32_t *data, int n, int32_t *totals) {
+  __shared__ int s_wsum[kBlock / kWave];
+  int32_t *row = data + (size_t)blockIdx.x * n;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  int carry = 0;
+  for (int base = 0; base < n; base += kBlock) {
+    const int i = base + threadIdx.x;
+    const int v = i < n ? row[i] : 0;
+    int incl = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      int t = __shfl_up(incl, off, kWave);
+      if (lane >= off) incl += t;
+    }
+    if (lane == kWave - 1) s_wsum[wave] = incl;
+    __syncthreads();
+    int woff = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / kWave; ++w) {
+      if (w < wave) woff += s_wsum[w];
+      total += s_wsum[w];
+    }
+    if (i < n) row[i] = carry + woff + incl - v;
+    carry += total;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) totals[blockIdx.x] = carry;
+}
+
+// Compacts the candidates of every offset in row order: position = exclusive
+// wave prefix + rank of the lane among the wave's hits.  Lane j also owns
+// position j of every offset's tail and writes -1 there when j >= indice_num[k].
+template <bool SUBM>
+__global__ __launch_bounds__(kBlock) void rbEmitPairs(int L, int K, const int32_t *cand,
+                                                      const int32_t *wave_offs, int n_wave,
+                                                      const int32_t *indice_num,
+                                                      const unsigned long long *bitmap,
+                                                      const uint32_t *word_rank,
+                                                      int32_t *pairs) {
+  const int j = blockIdx.x * kBlock + threadIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wt = j >> 6;
+  if (wt >= n_wave) return;
+  const bool active = j < L;
+  const unsigned long long lt_mask = (1ull << lane) - 1ull;
+  for (int k = 0; k < K; ++k) {
+    int r = active ? cand[(size_t)k * L + j] : -1;
+    if (!SUBM && r >= 0) {
+      const unsigned long long below = bitmap[r >> 6] & ((1ull << (r & 63)) - 1ull);
+      r = (int)(word_rank[r >> 6] + (uint32_t)__popcll(below));
+    }
+    const unsigned long long b = __ballot(r >= 0);
+    int32_t *in_col = pairs + (size_t)k * 2 * L;
+    int32_t *out_col = in_col + L;
+    if (r >= 0) {
+      const int pos = wave_offs[(size_t)k * n_wave + wt] + __popcll(b & lt_mask);
+      in_col[pos] = j;
+      out_col[pos] = r;
+    }
+    if (active && j >= indice_num[k]) {
+      in_col[j] = -1;
+      out_col[j] = -1;
+    }
+  }
+}
+
+// ---- regular mode: ranks of marked cells -----------------------------------
+
+__global__ __launch_bounds__(kBlock) void rbBitmapBlockSum(const unsigned long long *bitmap,
+                                                           size_t n_words, int32_t *block_sum) {
+  __shared__ int s_wsum[kBlock / kWave];
+  const size_t base = (size_t)blockIdx.x * kWordsPerBlock;
+  int cnt = 0;
+#pragma unroll
+  for (int i = 0; i < kWordsPerBlock / kBlock; ++i) {
+    size_t w = base + (size_t)i * kBlock + threadIdx.x;
+    if (w < n_words) cnt += __popcll(bitmap[w]);
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) cnt += __shfl_down(cnt, off, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0) s_wsum[threadIdx.x >> 6] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int t = 0;
+    for (int w = 0; w < kBlock / kWave; ++w) t += s_wsum[w];
+    block_sum[blockIdx.x] = t;
+  }
+}
+
+// Per bitmap word: number of marked cells before it (word_rank).  Every marked
+// cell is decoded to (n, d, h, w) and written at its rank; rows from
+// num_act_out up to out_rows are set to -1.
+__global__ __launch_bounds__(kBlock) void rbRankAndDecode(GeomDev g,
+                                                          const unsigned long long *bitmap,
+                                                          size_t n_words,
+                                                          const int32_t *block_excl,
+                                                          const int32_t *num_act_out,
+                                                          uint32_t *word_rank,
+                                                          int32_t *out_indices, bool aligned,
+                                                          int out_rows) {
+  __shared__ int s_wsum[kBlock / kWave];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const size_t base = (size_t)blockIdx.x * kWordsPerBlock;
+  int carry = block_excl[blockIdx.x];
+  const int hw = g.out[1] * g.out[2];
+  const int vol = g.out[0] * hw;
+  for (int i = 0; i < kWordsPerBlock / kBlock; ++i) {
+    const size_t w = base + (size_t)i * kBlock + threadIdx.x;
+    unsigned long long bits = w < n_words ? bitmap[w] : 0ull;
+    const int v = __popcll(bits);
+    int incl = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      int t = __shfl_up(incl, off, kWave);
+      if (lane >= off) incl += t;
+    }
+    if (lane == kWave - 1) s_wsum[wave] = incl;
+    __syncthreads();
+    int woff = 0, total = 0;
+#pragma unroll
+    for (int x = 0; x < kBlock / kWave; ++x) {
+      if (x < wave) woff += s_wsum[x];
+      total += s_wsum[x];
+    }
+    int rank = carry + woff + incl - v;
+    if (w < n_words) word_rank[w] = (uint32_t)rank;
+    while (bits) {
+      const int bit = __ffsll((long long)bits) - 1;
+      bits &= bits - 1;
+      if (rank < out_rows) {
+        int cell = (int)(w * 64 + bit);
+        int4 o;
+        o.x = cell / vol;
+        cell -= o.x * vol;
+        o.y = cell / hw;
+        cell -= o.y * hw;
+        o.z = cell / g.out[2];
+        o.w = cell - o.z * g.out[2];
+        storeCoord(out_indices, rank, o, aligned);
+      }
+      ++rank;
+    }
+    carry += total;
+    __syncthreads();
+  }
+  const int n_out = *num_act_out;
+  const size_t gstride = (size_t)gridDim.x * kBlock;
+  for (size_t r = (size_t)n_out + (size_t)blockIdx.x * kBlock + threadIdx.x; r < (size_t)out_rows;
+       r += gstride) {
+    storeCoord(out_indices, (int)r, make_int4(-1, -1, -1, -1), aligned);
+  }
+}
+
+// ---- host side ---------------------------------------------------------------
+
+inline size_t alignUp(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
+
+inline uint32_t tableCapacity(int L) {
+  uint32_t cap = 64;
+  while (cap < 2u * (uint32_t)L) cap <<= 1;
+  return cap;
+}
+
+struct Workspace {
+  // submanifold
+  unsigned long long *table = nullptr;
+  uint32_t table_cap = 0;
+  // regular
+  unsigned long long *bitmap = nullptr;
+  uint32_t *word_rank = nullptr;
+  int32_t *block_sum = nullptr;
+  int32_t *num_act_out = nullptr;
+  size_t n_words = 0;
+  int n_bitmap_blocks = 0;
+  // both
+  int32_t *cand = nullptr;
+  int32_t *counts = nullptr;
+  int n_wave = 0;
+  size_t bytes = 0;
+};
+
+Workspace carve(const RulebookGeom &g, void *base) {
+  Workspace ws;
+  // Blocks are carved from the caller's pointer rounded up to 256 bytes; the
+  // reported size includes that slack.
+  char *p = base ? reinterpret_cast<char *>(alignUp(reinterpret_cast<uintptr_t>(base))) : nullptr;
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    char *r = p ? p + off : nullptr;
+    off += alignUp(bytes);
+    return r;
+  };
+  ws.n_wave = (g.L + kWave - 1) / kWave;
+  if (g.sub_m) {
+    ws.table_cap = tableCapacity(g.L);
+    ws.table = reinterpret_cast<unsigned long long *>(take((size_t)ws.table_cap * 8));
+  } else {
+    const size_t cells = (size_t)g.batch * g.out_space[0] * g.out_space[1] * g.out_space[2];
+    ws.n_words = (cells + 63) / 64;
+    ws.n_bitmap_blocks = (int)((ws.n_words + kWordsPerBlock - 1) / kWordsPerBlock);
+    ws.bitmap = reinterpret_cast<unsigned long long *>(take(ws.n_words * 8));
+    ws.word_rank = reinterpret_cast<uint32_t *>(take(ws.n_words * 4));
+    ws.block_sum = reinterpret_cast<int32_t *>(take((size_t)ws.n_bitmap_blocks * 4));
+    ws.num_act_out = reinterpret_cast<int32_t *>(take(4));
+  }
+  ws.cand = reinterpret_cast<int32_t *>(take((size_t)g.K * g.L * 4));
+  ws.counts = reinterpret_cast<int32_t *>(take((size_t)g.K * ws.n_wave * 4));
+  ws.bytes = off + 256;
+  return ws;
+}
+
+GeomDev toDev(const RulebookGeom &g) {
+  GeomDev d;
+  d.batch = g.batch;
+  for (int a = 0; a < 3; ++a) {
+    d.out[a] = g.out_space[a];
+    d.ks[a] = g.ksize[a];
+    d.pad[a] = g.pad[a];
+    d.stride[a] = g.stride[a];
+    d.dil[a] = g.dilation[a];
+  }
+  d.K = g.K;
+  d.L = g.L;
+  return d;
+}
+
+inline bool aligned16(const void *a, const void *b) {
+  return (((uintptr_t)a | (uintptr_t)b) & 15u) == 0;
+}
+
+inline int fillBlocks(size_t n) {
+  size_t b = (n + kBlock - 1) / kBlock;
+  return (int)(b < 1 ? 1 : (b > 4096 ? 4096 : b));
+}
+
+}  // namespace
+
+size_t rulebookWorkspaceBytes(const RulebookGeom &g) { return carve(g, nullptr).bytes; }
+
+hipError_t launchSubmRulebook(hipStream_t stream, const RulebookGeom &g, const int32_t *indices,
+                              void *workspace, int32_t *indice_pairs, int32_t *out_indices,
+                              int32_t *indice_num) {
+  const Workspace ws = carve(g, workspace);
+  const GeomDev d = toDev(g);
+  const bool al = aligned16(indices, out_indices);
+  const uint32_t mask = ws.table_cap - 1;
+  const int rows = g.L > g.out_rows ? g.L : g.out_rows;
+  const int row_blocks = (rows + kBlock - 1) / kBlock;
+  const int l_blocks = (g.L + kBlock - 1) / kBlock;
+
+  rbFill64<<<fillBlocks(ws.table_cap), kBlock, 0, stream>>>(ws.table, ws.table_cap, kEmptySlot);
+  rbSubmInsert<<<row_blocks, kBlock, 0, stream>>>(d, indices, al, ws.table, mask, out_indices,
+                                                  g.out_rows);
+  rbProbeCount<true><<<l_blocks, kBlock, 0, stream>>>(d, indices, al, ws.table, mask, nullptr,
+                                                      ws.cand, ws.counts, ws.n_wave);
+  rbScanRows<<<g.K, kBlock, 0, stream>>>(ws.counts, ws.n_wave, indice_num);
+  rbEmitPairs<true><<<l_blocks, kBlock, 0, stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
+                                                     indice_num, nullptr, nullptr, indice_pairs);
+  return hipGetLastError();
+}
+
+hipError_t launchRegularRulebook(hipStream_t stream, const RulebookGeom &g,
+                                 const int32_t *indices, void *workspace, int32_t *indice_pairs,
+                                 int32_t *out_indices, int32_t *indice_num,
+                                 int32_t *host_num_act_out) {
+  const Workspace ws = carve(g, workspace);
+  const GeomDev d = toDev(g);
+  const bool al_in = aligned16(indices, indices);
+  const bool al_out = aligned16(out_indices, out_indices);
+  const int l_blocks = (g.L + kBlock - 1) / kBlock;
+
+  rbFill64<<<fillBlocks(ws.n_words), kBlock, 0, stream>>>(ws.bitmap, ws.n_words, 0ull);
+  rbProbeCount<false><<<l_blocks, kBlock, 0, stream>>>(d, indices, al_in, nullptr, 0, ws.bitmap,
+                                                       ws.cand, ws.counts, ws.n_wave);
+  rbScanRows<<<g.K, kBlock, 0, stream>>>(ws.counts, ws.n_wave, indice_num);
+  rbBitmapBlockSum<<<ws.n_bitmap_blocks, kBlock, 0, stream>>>(ws.bitmap, ws.n_words,
+                                                              ws.block_sum);
+  rbScanRows<<<1, kBlock, 0, stream>>>(ws.block_sum, ws.n_bitmap_blocks, ws.num_act_out);
+  hipError_t err = hipMemcpyAsync(host_num_act_out, ws.num_act_out, sizeof(int32_t),
+                                  hipMemcpyDeviceToHost, stream);
+  if (err != hipSuccess) return err;
+  rbRankAndDecode<<<ws.n_bitmap_blocks, kBlock, 0, stream>>>(d, ws.bitmap, ws.n_words,
+                                                             ws.block_sum, ws.num_act_out,
+                                                             ws.word_rank, out_indices, al_out,
+                                                             g.out_rows);
+  rbEmitPairs<false><<<l_blocks, kBlock, 0, stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
+                                                      indice_num, ws.bitmap, ws.word_rank,
+                                                      indice_pairs);
+  return hipGetLastError();
+}
+
+}  // namespace sparse_conv
+}  // namespace mluop

@@ -1,0 +1,372 @@
+"""ctypes binding of libmluops.so, the MI355X sparse-convolution library.
+
+The module mirrors the C API of ``include/mlu_op.h`` one to one (``lib()`` returns
+the loaded library with argument types set) and adds a thin convenience layer
+(`Handle`, `TensorDescriptor`, `SparseConvDescriptor`, `get_indice_pairs`,
+`indice_conv_forward`, ...) that follows the call sequence a framework uses:
+create descriptor -> query workspace -> run op -> read num_act_out -> copy
+indice_num to the host -> convolution ops.
+
+Device buffers are torch tensors; torch supplies memory and the stream, every
+computation runs in the library's own HIP kernels.  There is no CPU fallback: a
+missing library raises at import of the first symbol.
+"""
+import ctypes
+import os
+
+from . import datagen  # noqa: F401
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "..", "lib", "libmluops.so"))
+
+# mluOpStatus_t
+STATUS_SUCCESS = 0
+STATUS_NOT_INITIALIZED = 1
+STATUS_ALLOC_FAILED = 2
+STATUS_BAD_PARAM = 3
+STATUS_INTERNAL_ERROR = 4
+STATUS_ARCH_MISMATCH = 5
+STATUS_EXECUTION_FAILED = 6
+STATUS_NOT_SUPPORTED = 7
+STATUS_NUMERICAL_OVERFLOW = 8
+
+# mluOpTensorLayout_t
+LAYOUT_NCHW, LAYOUT_NHWC, LAYOUT_HWCN, LAYOUT_NDHWC, LAYOUT_ARRAY, LAYOUT_NCDHW = 0, 1, 2, 3, 4, 5
+LAYOUT_TNC, LAYOUT_NTC, LAYOUT_NC, LAYOUT_NLC, LAYOUT_NCL = 6, 7, 8, 9, 10
+
+# mluOpDataType_t
+DTYPE_INVALID, DTYPE_HALF, DTYPE_FLOAT, DTYPE_INT8, DTYPE_INT16, DTYPE_INT31 = 0, 1, 2, 3, 4, 5
+DTYPE_INT32, DTYPE_UINT8, DTYPE_BOOL, DTYPE_INT64 = 6, 7, 8, 9
+DTYPE_UINT32, DTYPE_UINT64, DTYPE_UINT16, DTYPE_DOUBLE = 11, 12, 13, 14
+DTYPE_COMPLEX_HALF, DTYPE_COMPLEX_FLOAT, DTYPE_BFLOAT16 = 15, 16, 17
+
+ATOMICS_NOT_ALLOWED, ATOMICS_ALLOWED = 1, 2
+POINTER_MODE_HOST, POINTER_MODE_DEVICE = 0, 1
+
+_vp = ctypes.c_void_p
+_ip = ctypes.POINTER(ctypes.c_int)
+_i64p = ctypes.POINTER(ctypes.c_int64)
+_szp = ctypes.POINTER(ctypes.c_size_t)
+
+# name -> (restype, argtypes); every symbol declared in include/mlu_op.h.
+SIGNATURES = {
+    "mluOpCreate": (ctypes.c_int, [ctypes.POINTER(_vp)]),
+    "mluOpDestroy": (ctypes.c_int, [_vp]),
+    "mluOpSetQueue": (ctypes.c_int, [_vp, _vp]),
+    "mluOpGetQueue": (ctypes.c_int, [_vp, ctypes.POINTER(_vp)]),
+    "mluOpGetErrorString": (ctypes.c_char_p, [ctypes.c_int]),
+    "mluOpGetSizeOfDataType": (ctypes.c_int, [ctypes.c_int, _szp]),
+    "mluOpGetLibVersion": (None, [_ip, _ip, _ip]),
+    "mluOpSetQuantizeRoundMode": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "mluOpGetQuantizeRoundMode": (ctypes.c_int, [_vp, _ip]),
+    "mluOpSetAtomicsMode": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "mluOpGetAtomicsMode": (ctypes.c_int, [_vp, _ip]),
+    "mluOpCreateTensorDescriptor": (ctypes.c_int, [ctypes.POINTER(_vp)]),
+    "mluOpSetTensorDescriptor": (ctypes.c_int, [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _ip]),
+    "mluOpSetTensorDescriptor_v2": (ctypes.c_int, [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _i64p]),
+    "mluOpSetTensorDescriptorEx": (ctypes.c_int, [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _ip, _ip]),
+    "mluOpSetTensorDescriptorEx_v2": (ctypes.c_int, [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _i64p, _i64p]),
+    "mluOpSetTensorDescriptorPointerMode": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "mluOpGetTensorDescriptorPointerMode": (ctypes.c_int, [_vp, _ip]),
+    "mluOpSetTensorDescriptorOnchipDataType": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "mluOpGetTensorDescriptorOnchipDataType": (ctypes.c_int, [_vp, _ip]),
+    "mluOpGetTensorDescriptor": (ctypes.c_int, [_vp, _ip, _ip, _ip, _ip]),
+    "mluOpGetTensorDescriptor_v2": (ctypes.c_int, [_vp, _ip, _ip, _ip, _i64p]),
+    "mluOpGetTensorDescriptorEx": (ctypes.c_int, [_vp, _ip, _ip, _ip, _ip, _ip]),
+    "mluOpGetTensorDescriptorEx_v2": (ctypes.c_int, [_vp, _ip, _ip, _ip, _i64p, _i64p]),
+    "mluOpGetTensorElementNum": (ctypes.c_size_t, [_vp]),
+    "mluOpResetTensorDescriptor": (ctypes.c_int, [_vp]),
+    "mluOpDestroyTensorDescriptor": (ctypes.c_int, [_vp]),
+    "mluOpCreateSparseConvolutionDescriptor": (ctypes.c_int, [ctypes.POINTER(_vp)]),
+    "mluOpDestroySparseConvolutionDescriptor": (ctypes.c_int, [_vp]),
+    "mluOpSetSparseConvolutionDescriptor": (
+        ctypes.c_int, [_vp, ctypes.c_int, ctypes.c_int, _ip, _ip, _ip, _ip, _ip, _ip,
+                       ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mluOpGetSparseConvolutionNumActOut": (ctypes.c_int, [_vp, _ip]),
+    "mluOpGetIndicePairs": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_size_t, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "mluOpGetIndicePairsWorkspaceSize": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _szp]),
+    "mluOpGetIndiceConvolutionForwardWorkspaceSize": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i64p, ctypes.c_int64, ctypes.c_int64,
+                       ctypes.c_int64, _szp]),
+    "mluOpIndiceConvolutionForward": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64p, ctypes.c_int64, ctypes.c_int64,
+                       ctypes.c_int64, _vp, ctypes.c_size_t, _vp, _vp]),
+    "mluOpGetIndiceConvolutionBackwardDataWorkspaceSize": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i64p, ctypes.c_int64, _szp]),
+    "mluOpIndiceConvolutionBackwardData": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64p, ctypes.c_int64, ctypes.c_int64,
+                       _vp, ctypes.c_size_t, _vp, _vp]),
+    "mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i64p, ctypes.c_int64, ctypes.c_int64, _szp]),
+    "mluOpIndiceConvolutionBackwardFilter": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64p, ctypes.c_int64, ctypes.c_int64,
+                       _vp, ctypes.c_size_t, _vp, _vp]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libmluops.so is missing (%s): build it with `make -C mlu-ops_amd` or "
+                "__graft_entry__.build(); there is no fallback path." % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+class MluOpError(RuntimeError):
+    def __init__(self, status, what):
+        self.status = status
+        name = lib().mluOpGetErrorString(status).decode()
+        super().__init__("%s returned %s" % (what, name))
+
+
+def check(status, what="mluOp call"):
+    if status != STATUS_SUCCESS:
+        raise MluOpError(status, what)
+
+
+def _int_array(values, ctype=ctypes.c_int):
+    values = [int(v) for v in values]
+    return (ctype * max(len(values), 1))(*values)
+
+
+class Handle:
+    """mluOpHandle_t bound to the current device; `queue` is a raw hipStream_t."""
+
+    def __init__(self, queue=None):
+        self.ptr = _vp()
+        check(lib().mluOpCreate(ctypes.byref(self.ptr)), "mluOpCreate")
+        if queue is not None:
+            self.set_queue(queue)
+
+    def set_queue(self, queue):
+        check(lib().mluOpSetQueue(self.ptr, _vp(queue)), "mluOpSetQueue")
+
+    def close(self):
+        if self.ptr:
+            lib().mluOpDestroy(self.ptr)
+            self.ptr = _vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class TensorDescriptor:
+    def __init__(self, layout, dtype, dims, onchip_dtype=None):
+        self.ptr = _vp()
+        check(lib().mluOpCreateTensorDescriptor(ctypes.byref(self.ptr)))
+        dims = list(dims)
+        check(lib().mluOpSetTensorDescriptor(self.ptr, layout, dtype, len(dims), _int_array(dims)),
+              "mluOpSetTensorDescriptor")
+        if onchip_dtype is not None:
+            check(lib().mluOpSetTensorDescriptorOnchipDataType(self.ptr, onchip_dtype))
+        self.dims = dims
+        self.dtype = dtype
+        self.layout = layout
+
+    def close(self):
+        if self.ptr:
+            lib().mluOpDestroyTensorDescriptor(self.ptr)
+            self.ptr = _vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class SparseConvDescriptor:
+    def __init__(self, batch, pad, stride, dilation, input_space, filter_space, output_space,
+                 sub_m, transpose=0, inverse=0, dim_nb=5):
+        self.ptr = _vp()
+        check(lib().mluOpCreateSparseConvolutionDescriptor(ctypes.byref(self.ptr)))
+        check(lib().mluOpSetSparseConvolutionDescriptor(
+            self.ptr, dim_nb, batch, _int_array(pad), _int_array(stride), _int_array(dilation),
+            _int_array(input_space), _int_array(filter_space), _int_array(output_space),
+            int(sub_m), int(transpose), int(inverse)), "mluOpSetSparseConvolutionDescriptor")
+
+    def num_act_out(self):
+        n = ctypes.c_int(0)
+        check(lib().mluOpGetSparseConvolutionNumActOut(self.ptr, ctypes.byref(n)))
+        return n.value
+
+    def close(self):
+        if self.ptr:
+            lib().mluOpDestroySparseConvolutionDescriptor(self.ptr)
+            self.ptr = _vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def regular_output_space(input_space, filter_space, pad, stride, dilation):
+    """Output extent of a regular convolution per axis (the caller supplies it to the API)."""
+    return [(i + 2 * p - d * (k - 1) - 1) // s + 1
+            for i, k, p, s, d in zip(input_space, filter_space, pad, stride, dilation)]
+
+
+# ---------------------------------------------------------------------------
+# torch-facing convenience layer (device memory and stream only)
+# ---------------------------------------------------------------------------
+
+def _torch():
+    import torch
+    return torch
+
+
+def torch_dtype_code(dtype):
+    torch = _torch()
+    return {torch.float16: DTYPE_HALF, torch.float32: DTYPE_FLOAT, torch.bfloat16: DTYPE_BFLOAT16,
+            torch.int32: DTYPE_INT32}[dtype]
+
+
+def make_handle_on_current_stream():
+    torch = _torch()
+    return Handle(queue=torch.cuda.current_stream().cuda_stream)
+
+
+def _workspace(nbytes, device):
+    torch = _torch()
+    return torch.empty((max(int(nbytes), 1),), dtype=torch.uint8, device=device)
+
+
+def get_indice_pairs(handle, indices, batch, input_space, filter_space, output_space, pad, stride,
+                     dilation, sub_m, out_rows=None):
+    """Builds the rulebook for `indices` (int32 [L, 4] device tensor).
+
+    Returns (indice_pairs [K,2,L], out_indices [out_rows,4], indice_num [K] device int32,
+    num_act_out).  In submanifold mode num_act_out is L."""
+    torch = _torch()
+    L = indices.shape[0]
+    K = 1
+    for k in filter_space:
+        K *= int(k)
+    if out_rows is None:
+        if sub_m:
+            out_rows = L
+        else:
+            vol = batch
+            for o in output_space:
+                vol *= int(o)
+            out_rows = min(vol, K * L)
+    dev = indices.device
+    pairs = torch.empty((K, 2, L), dtype=torch.int32, device=dev)
+    out_indices = torch.empty((out_rows, 4), dtype=torch.int32, device=dev)
+    indice_num = torch.empty((K,), dtype=torch.int32, device=dev)
+    desc = SparseConvDescriptor(batch, pad, stride, dilation, input_space, filter_space,
+                                output_space, sub_m)
+    d_in = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [L, 4])
+    d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+    d_out = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [out_rows, 4])
+    d_num = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K])
+    size = ctypes.c_size_t(0)
+    check(lib().mluOpGetIndicePairsWorkspaceSize(handle.ptr, desc.ptr, d_in.ptr, d_pairs.ptr,
+                                                 d_out.ptr, d_num.ptr, ctypes.byref(size)),
+          "mluOpGetIndicePairsWorkspaceSize")
+    ws = _workspace(size.value, dev)
+    check(lib().mluOpGetIndicePairs(handle.ptr, desc.ptr, d_in.ptr, indices.data_ptr(),
+                                    ws.data_ptr(), size.value, d_pairs.ptr, pairs.data_ptr(),
+                                    d_out.ptr, out_indices.data_ptr(), d_num.ptr,
+                                    indice_num.data_ptr()), "mluOpGetIndicePairs")
+    num_act_out = L if sub_m else desc.num_act_out()
+    return pairs, out_indices, indice_num, num_act_out
+
+
+def _host_counts(indice_num):
+    vals = [int(v) for v in indice_num]
+    return (ctypes.c_int64 * max(len(vals), 1))(*vals)
+
+
+def indice_conv_forward(handle, features, filters, filters_layout, indice_pairs, indice_num_host,
+                        num_act_out, sub_m, inverse=0):
+    """features [L,Ci], filters 5-D in `filters_layout`, indice_num_host: K python ints."""
+    torch = _torch()
+    code = torch_dtype_code(features.dtype)
+    K, _, L = indice_pairs.shape
+    if filters_layout == LAYOUT_ARRAY:
+        co = filters.shape[4]
+    else:
+        co = filters.shape[0]
+    out = torch.empty((num_act_out, co), dtype=features.dtype, device=features.device)
+    d_feat = TensorDescriptor(LAYOUT_ARRAY, code, list(features.shape))
+    d_filt = TensorDescriptor(filters_layout, code, list(filters.shape))
+    d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+    d_out = TensorDescriptor(LAYOUT_ARRAY, code, [num_act_out, co])
+    counts = _host_counts(indice_num_host)
+    size = ctypes.c_size_t(0)
+    check(lib().mluOpGetIndiceConvolutionForwardWorkspaceSize(
+        handle.ptr, d_feat.ptr, d_filt.ptr, d_pairs.ptr, d_out.ptr, counts, num_act_out, inverse,
+        int(sub_m), ctypes.byref(size)), "mluOpGetIndiceConvolutionForwardWorkspaceSize")
+    ws = _workspace(size.value, features.device)
+    check(lib().mluOpIndiceConvolutionForward(
+        handle.ptr, d_feat.ptr, features.data_ptr(), d_filt.ptr, filters.data_ptr(), d_pairs.ptr,
+        indice_pairs.data_ptr(), counts, num_act_out, inverse, int(sub_m), ws.data_ptr(),
+        size.value, d_out.ptr, out.data_ptr()), "mluOpIndiceConvolutionForward")
+    return out
+
+
+def indice_conv_backward_data(handle, output_grad, filters, filters_layout, indice_pairs,
+                              indice_num_host, sub_m, ci, inverse=0):
+    torch = _torch()
+    code = torch_dtype_code(output_grad.dtype)
+    K, _, L = indice_pairs.shape
+    dx = torch.empty((L, ci), dtype=output_grad.dtype, device=output_grad.device)
+    d_dy = TensorDescriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
+    d_filt = TensorDescriptor(filters_layout, code, list(filters.shape))
+    d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+    d_dx = TensorDescriptor(LAYOUT_ARRAY, code, [L, ci])
+    counts = _host_counts(indice_num_host)
+    size = ctypes.c_size_t(0)
+    check(lib().mluOpGetIndiceConvolutionBackwardDataWorkspaceSize(
+        handle.ptr, d_dy.ptr, d_filt.ptr, d_pairs.ptr, d_dx.ptr, counts, inverse,
+        ctypes.byref(size)), "mluOpGetIndiceConvolutionBackwardDataWorkspaceSize")
+    ws = _workspace(size.value, output_grad.device)
+    check(lib().mluOpIndiceConvolutionBackwardData(
+        handle.ptr, d_dy.ptr, output_grad.data_ptr(), d_filt.ptr, filters.data_ptr(), d_pairs.ptr,
+        indice_pairs.data_ptr(), counts, inverse, int(sub_m), ws.data_ptr(), size.value, d_dx.ptr,
+        dx.data_ptr()), "mluOpIndiceConvolutionBackwardData")
+    return dx
+
+
+def indice_conv_backward_filter(handle, features, output_grad, indice_pairs, indice_num_host,
+                                filter_space, sub_m, inverse=0, onchip_float=True):
+    """Returns filters_grad laid out [kd, kh, kw, Ci, Co]."""
+    torch = _torch()
+    code = torch_dtype_code(features.dtype)
+    K, _, L = indice_pairs.shape
+    ci, co = features.shape[1], output_grad.shape[1]
+    dw = torch.empty(tuple(filter_space) + (ci, co), dtype=features.dtype, device=features.device)
+    d_x = TensorDescriptor(LAYOUT_ARRAY, code, list(features.shape))
+    d_dy = TensorDescriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
+    d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+    d_dw = TensorDescriptor(LAYOUT_ARRAY, code, list(dw.shape),
+                            onchip_dtype=DTYPE_FLOAT if onchip_float else None)
+    counts = _host_counts(indice_num_host)
+    size = ctypes.c_size_t(0)
+    check(lib().mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize(
+        handle.ptr, d_x.ptr, d_dy.ptr, d_pairs.ptr, d_dw.ptr, counts, inverse, int(sub_m),
+        ctypes.byref(size)), "mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize")
+    ws = _workspace(size.value, features.device)
+    check(lib().mluOpIndiceConvolutionBackwardFilter(
+        handle.ptr, d_x.ptr, features.data_ptr(), d_dy.ptr, output_grad.data_ptr(), d_pairs.ptr,
+        indice_pairs.data_ptr(), counts, inverse, int(sub_m), ws.data_ptr(), size.value, d_dw.ptr,
+        dw.data_ptr()), "mluOpIndiceConvolutionBackwardFilter")
+    return dw

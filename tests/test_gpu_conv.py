@@ -1,0 +1,214 @@
+"""GPU parity of the three indice-convolution operators against the CPU oracle.
+
+Inputs are seeded fp32 values rounded through the tensor dtype (so device and oracle see the
+same numbers), the oracle accumulates in fp32 and its result is rounded through the output
+dtype, then diff1/diff2 are graded at the reference's thresholds (spconv_cases.THRESH)."""
+import os
+
+import numpy as np
+import pytest
+
+import sparse_conv_oracle as oracle
+from spconv_cases import check_close, from_torch, out_space, random_voxels, round_to, to_torch
+
+pytestmark = pytest.mark.gpu
+
+
+def build_rulebook(idx, batch, space, ks, pad, stride, dil, sub_m):
+    ospace = list(space) if sub_m else out_space(space, ks, pad, stride, dil)
+    pairs, out_idx, num, n_out = oracle.get_indice_pairs(idx, batch, pad, stride, dil, ks, ospace, sub_m,
+                                                         exact_count=True)
+    return pairs, num, n_out
+
+
+def conv_case(seed, batch, space, L, ks, ci, co, sub_m, stride=(1, 1, 1)):
+    rng = np.random.default_rng(seed)
+    idx = random_voxels(rng, batch, space, L)
+    pad = [k // 2 for k in ks]
+    pairs, num, n_out = build_rulebook(idx, batch, space, ks, pad, list(stride), [1, 1, 1], sub_m)
+    K = int(np.prod(ks))
+    feats = rng.standard_normal((idx.shape[0], ci)).astype(np.float32)
+    b = 1.0 / np.sqrt(K * ci)
+    w = rng.uniform(-b, b, size=tuple(ks) + (ci, co)).astype(np.float32)
+    dy = (rng.standard_normal((n_out, co)) * 1e-1).astype(np.float32)
+    return dict(idx=idx, pairs=pairs, num=num, n_out=n_out, feats=feats, w=w, dy=dy, K=K, ks=ks,
+                ci=ci, co=co, sub_m=sub_m)
+
+
+def run_all_ops(handle, c, dtype_name, force_simt=False, check=("fwd", "bwd_data", "bwd_filter")):
+    import torch
+    import mluop_hip
+    if force_simt:
+        os.environ["MLUOP_SPCONV_FORCE_SIMT"] = "1"
+    else:
+        os.environ.pop("MLUOP_SPCONV_FORCE_SIMT", None)
+    try:
+        dev = "cuda"
+        feats_r = round_to(c["feats"], dtype_name)
+        w_r = round_to(c["w"], dtype_name)
+        dy_r = round_to(c["dy"], dtype_name)
+        w_k = w_r.reshape(c["K"], c["ci"], c["co"])
+        pairs_t = torch.from_numpy(c["pairs"]).cuda()
+        num_host = [int(v) for v in c["num"]]
+        feats_t = to_torch(feats_r, dtype_name, dev)
+        w_t = to_torch(w_r, dtype_name, dev)
+        dy_t = to_torch(dy_r, dtype_name, dev)
+        res = {}
+        if "fwd" in check:
+            out = mluop_hip.indice_conv_forward(handle, feats_t, w_t, mluop_hip.LAYOUT_ARRAY, pairs_t, num_host,
+                                                c["n_out"], c["sub_m"])
+            torch.cuda.synchronize()
+            ref = oracle.forward(feats_r, w_k, c["pairs"], c["num"], c["n_out"])
+            res["fwd"] = check_close(from_torch(out), ref, dtype_name, "forward")
+        if "bwd_data" in check:
+            dx = mluop_hip.indice_conv_backward_data(handle, dy_t, w_t, mluop_hip.LAYOUT_ARRAY, pairs_t, num_host,
+                                                     c["sub_m"], c["ci"])
+            torch.cuda.synchronize()
+            ref = oracle.backward_data(dy_r, w_k, c["pairs"], c["num"])
+            res["bwd_data"] = check_close(from_torch(dx), ref, dtype_name, "backward_data")
+        if "bwd_filter" in check:
+            dw = mluop_hip.indice_conv_backward_filter(handle, feats_t, dy_t, pairs_t, num_host, c["ks"],
+                                                       c["sub_m"])
+            torch.cuda.synchronize()
+            ref = oracle.backward_filter(feats_r, dy_r, c["pairs"], c["num"], fast=True)
+            res["bwd_filter"] = check_close(from_torch(dw).reshape(ref.shape), ref, dtype_name,
+                                            "backward_filter")
+        return res
+    finally:
+        os.environ.pop("MLUOP_SPCONV_FORCE_SIMT", None)
+
+
+SHAPES = [
+    # (batch, space, L, ks, ci, co, sub_m, stride)
+    (1, (6, 6, 6), 50, (3, 3, 3), 16, 16, True, (1, 1, 1)),
+    (2, (8, 9, 10), 400, (3, 3, 3), 32, 32, True, (1, 1, 1)),
+    (1, (10, 12, 12), 900, (3, 3, 3), 64, 64, True, (1, 1, 1)),
+    (2, (8, 10, 10), 500, (3, 3, 3), 64, 32, False, (2, 2, 2)),
+    (1, (8, 8, 8), 300, (3, 3, 3), 32, 128, True, (1, 1, 1)),
+    (1, (8, 8, 8), 300, (3, 3, 3), 128, 64, False, (1, 1, 1)),
+    (1, (6, 6, 6), 100, (3, 3, 3), 21, 10, True, (1, 1, 1)),   # odd channel counts -> SIMT
+    (1, (6, 6, 6), 100, (1, 3, 3), 13, 70, False, (1, 2, 1)),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("dtype_name", ["float32", "float16", "bfloat16"])
+def test_conv_ops_match_oracle(gpu_handle, shape, dtype_name):
+    batch, space, L, ks, ci, co, sub_m, stride = shape
+    print("conv case", shape, dtype_name, flush=True)
+    c = conv_case(11, batch, space, L, ks, ci, co, sub_m, stride)
+    run_all_ops(gpu_handle, c, dtype_name)
+
+
+@pytest.mark.parametrize("dtype_name", ["float16", "bfloat16"])
+def test_simt_path_matches_oracle_on_mfma_shapes(gpu_handle, dtype_name):
+    c = conv_case(12, 2, (8, 9, 10), 400, (3, 3, 3), 64, 64, True)
+    run_all_ops(gpu_handle, c, dtype_name, force_simt=True, check=("fwd", "bwd_data"))
+
+
+@pytest.mark.parametrize("layout_name", ["NDHWC", "NCDHW", "ARRAY"])
+@pytest.mark.parametrize("dtype_name", ["float32", "float16"])
+def test_forward_filter_layouts(gpu_handle, layout_name, dtype_name):
+    import torch
+    import mluop_hip
+    c = conv_case(13, 1, (8, 8, 8), 300, (3, 3, 3), 32, 64, True)
+    feats_r = round_to(c["feats"], dtype_name)
+    w_r = round_to(c["w"], dtype_name)  # [kd,kh,kw,ci,co]
+    if layout_name == "NDHWC":
+        w_l, code = np.transpose(w_r, (4, 0, 1, 2, 3)), mluop_hip.LAYOUT_NDHWC
+    elif layout_name == "NCDHW":
+        w_l, code = np.transpose(w_r, (4, 3, 0, 1, 2)), mluop_hip.LAYOUT_NCDHW
+    else:
+        w_l, code = w_r, mluop_hip.LAYOUT_ARRAY
+    w_l = np.ascontiguousarray(w_l)
+    # the oracle's own layout transpose must land on the [K, Ci, Co] tensor
+    w_k = oracle.filters_to_kcico(w_l, code, c["K"], c["ci"], c["co"])
+    assert np.array_equal(w_k, w_r.reshape(c["K"], c["ci"], c["co"]))
+    pairs_t = torch.from_numpy(c["pairs"]).cuda()
+    num_host = [int(v) for v in c["num"]]
+    out = mluop_hip.indice_conv_forward(gpu_handle, to_torch(feats_r, dtype_name, "cuda"),
+                                        to_torch(w_l, dtype_name, "cuda"), code, pairs_t, num_host, c["n_out"], True)
+    dx = mluop_hip.indice_conv_backward_data(gpu_handle, to_torch(round_to(c["dy"], dtype_name), dtype_name, "cuda"),
+                                             to_torch(w_l, dtype_name, "cuda"), code, pairs_t, num_host, True, c["ci"])
+    torch.cuda.synchronize()
+    check_close(from_torch(out), oracle.forward(feats_r, w_k, c["pairs"], c["num"], c["n_out"]), dtype_name,
+                "forward " + layout_name)
+    check_close(from_torch(dx), oracle.backward_data(round_to(c["dy"], dtype_name), w_k, c["pairs"], c["num"]),
+                dtype_name, "backward_data " + layout_name)
+
+
+def test_reference_case0_shape_backward_data(gpu_handle):
+    """Shapes of the reference's only in-tree case (zoo/indice_convolution_backward_data/test_case/
+    case_0.prototxt): L=10, 3x3 HWCN filter, Ci=210... here Ci=21, Co=10 4-D filter, identity pairs."""
+    import torch
+    import mluop_hip
+    rng = np.random.default_rng(3)
+    L, K, ci, co = 10, 9, 21, 10
+    pairs = np.full((K, 2, L), -1, dtype=np.int32)
+    for k in range(K):
+        pairs[k, 0, :] = np.arange(L)
+        pairs[k, 1, :] = np.arange(L)
+    num = [L] * K
+    dy = rng.standard_normal((L, co)).astype(np.float32)
+    w = rng.standard_normal((3, 3, ci, co)).astype(np.float32)
+    handle = gpu_handle
+    lib = mluop_hip.lib()
+    import ctypes
+    d_dy = mluop_hip.TensorDescriptor(mluop_hip.LAYOUT_ARRAY, mluop_hip.DTYPE_FLOAT, [L, co])
+    d_w = mluop_hip.TensorDescriptor(mluop_hip.LAYOUT_HWCN, mluop_hip.DTYPE_FLOAT, [3, 3, ci, co])
+    d_p = mluop_hip.TensorDescriptor(mluop_hip.LAYOUT_ARRAY, mluop_hip.DTYPE_INT32, [K, 2, L])
+    d_dx = mluop_hip.TensorDescriptor(mluop_hip.LAYOUT_ARRAY, mluop_hip.DTYPE_FLOAT, [L, ci])
+    counts = (ctypes.c_int64 * K)(*num)
+    size = ctypes.c_size_t(0)
+    mluop_hip.check(lib.mluOpGetIndiceConvolutionBackwardDataWorkspaceSize(
+        handle.ptr, d_dy.ptr, d_w.ptr, d_p.ptr, d_dx.ptr, counts, 0, ctypes.byref(size)))
+    ws = torch.empty(max(size.value, 1), dtype=torch.uint8, device="cuda")
+    t_dy, t_w, t_p = torch.from_numpy(dy).cuda(), torch.from_numpy(w).cuda(), torch.from_numpy(pairs).cuda()
+    t_dx = torch.empty((L, ci), dtype=torch.float32, device="cuda")
+    mluop_hip.check(lib.mluOpIndiceConvolutionBackwardData(
+        handle.ptr, d_dy.ptr, t_dy.data_ptr(), d_w.ptr, t_w.data_ptr(), d_p.ptr, t_p.data_ptr(), counts, 0, 0,
+        ws.data_ptr(), size.value, d_dx.ptr, t_dx.data_ptr()))
+    torch.cuda.synchronize()
+    ref = oracle.backward_data(dy, w.reshape(K, ci, co), pairs, num)
+    check_close(t_dx.cpu().numpy(), ref, "float32", "case_0 shape")
+
+
+def test_config1_forward_full_size(gpu_handle):
+    """BASELINE config 1: 20 000 uniform voxels, Ci=Co=16 fp32, subm 3x3x3, rulebook built on the GPU."""
+    import torch
+    import mluop_hip
+    idx = mluop_hip.datagen.uniform_voxels((1, 40, 400, 352), 20000, seed=1)
+    rng = np.random.default_rng(1)
+    feats = rng.standard_normal((20000, 16)).astype(np.float32)
+    w = mluop_hip.datagen.kaiming_uniform_filters((3, 3, 3), 16, 16, seed=1)
+    t_idx = torch.from_numpy(idx).cuda()
+    pairs, out_idx, num, n_out = mluop_hip.get_indice_pairs(gpu_handle, t_idx, 1, (40, 400, 352), (3, 3, 3),
+                                                           (40, 400, 352), [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+    num_host = num.cpu().tolist()
+    out = mluop_hip.indice_conv_forward(gpu_handle, torch.from_numpy(feats).cuda(), torch.from_numpy(w).cuda(),
+                                        mluop_hip.LAYOUT_ARRAY, pairs, num_host, n_out, True)
+    torch.cuda.synchronize()
+    ref = oracle.forward(feats, w.reshape(27, 16, 16), pairs.cpu().numpy(), num_host, n_out)
+    check_close(out.cpu().numpy(), ref, "float32", "config1 forward")
+
+
+def test_config4_all_ops_full_size(gpu_handle):
+    """BASELINE config 4 (headline): 120 000 clustered voxels, Ci=Co=64 fp16, subm 3x3x3: forward,
+    backward data and backward filter (dY ~ N(0, 1e-2), filter gradient accumulated in fp32)."""
+    import torch
+    import mluop_hip
+    L = 120000
+    idx = mluop_hip.datagen.clustered_voxels((1, 41, 1600, 1408), L, seed=4)
+    rng = np.random.default_rng(4)
+    feats = round_to(rng.standard_normal((L, 64)).astype(np.float32), "float16")
+    w = round_to(mluop_hip.datagen.kaiming_uniform_filters((3, 3, 3), 64, 64, seed=4), "float16")
+    dy = round_to((rng.standard_normal((L, 64)) * 1e-1).astype(np.float32), "float16")
+    t_idx = torch.from_numpy(idx).cuda()
+    pairs, out_idx, num, n_out = mluop_hip.get_indice_pairs(gpu_handle, t_idx, 1, (41, 1600, 1408), (3, 3, 3),
+                                                           (41, 1600, 1408), [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+    num_host = num.cpu().tolist()
+    pairs_np = pairs.cpu().numpy()
+    c = dict(pairs=pairs_np, num=np.array(num_host), n_out=n_out, feats=feats, w=w, dy=dy, K=27, ks=(3, 3, 3),
+             ci=64, co=64, sub_m=True)
+    print("config4 ops", flush=True)
+    run_all_ops(gpu_handle, c, "float16")

@@ -1,0 +1,124 @@
+"""GPU parity of mluOpGetIndicePairs against the CPU oracle: every output tensor must be
+bit-exact (reference accuracy rule: diff3 == 0 for indice_pairs, out_indices, indice_num)."""
+import numpy as np
+import pytest
+
+import sparse_conv_oracle as oracle
+from spconv_cases import out_space, random_voxels
+
+pytestmark = pytest.mark.gpu
+
+
+def run_gpu(handle, idx, batch, space, ks, ospace, pad, stride, dil, sub_m, out_rows=None):
+    import torch
+    import mluop_hip
+    t = torch.from_numpy(idx).cuda()
+    pairs, out_idx, num, n_out = mluop_hip.get_indice_pairs(
+        handle, t, batch, space, ks, ospace, pad, stride, dil, sub_m, out_rows=out_rows)
+    torch.cuda.synchronize()
+    return pairs.cpu().numpy(), out_idx.cpu().numpy(), num.cpu().numpy(), n_out
+
+
+def compare(handle, idx, batch, space, ks, pad, stride, dil, sub_m, out_rows=None):
+    ospace = list(space) if sub_m else out_space(space, ks, pad, stride, dil)
+    p, o, n, n_out = run_gpu(handle, idx, batch, space, ks, ospace, pad, stride, dil, sub_m, out_rows)
+    rows = o.shape[0]
+    rp, ro, rn, rn_out = oracle.get_indice_pairs(idx, batch, pad, stride, dil, ks, ospace, sub_m,
+                                                 out_rows=rows, exact_count=True)
+    assert np.array_equal(n, rn), "indice_num"
+    assert np.array_equal(p, rp), "indice_pairs"
+    assert np.array_equal(o, ro), "out_indices"
+    assert n_out == rn_out
+    return p, o, n, n_out
+
+
+SUBM_CASES = [
+    # (batch, space, L, ks, shuffle, duplicates, seed)
+    (1, (4, 5, 6), 1, (3, 3, 3), True, 0, 0),
+    (1, (4, 5, 6), 60, (3, 3, 3), True, 0, 1),
+    (2, (6, 7, 9), 300, (3, 3, 3), True, 0, 2),
+    (2, (6, 7, 9), 300, (3, 3, 3), False, 0, 3),
+    (3, (8, 8, 8), 700, (3, 3, 3), True, 40, 4),
+    (1, (10, 12, 14), 1000, (5, 5, 5), True, 0, 5),
+    (1, (9, 9, 9), 400, (1, 3, 5), True, 0, 6),
+    (1, (16, 32, 32), 5000, (3, 3, 3), True, 0, 7),
+    (1, (5, 5, 5), 125, (3, 3, 3), False, 0, 8),  # full block
+    (1, (3, 70, 70), 257, (3, 3, 3), True, 0, 9),
+]
+
+
+@pytest.mark.parametrize("case", SUBM_CASES)
+def test_subm_rulebook_matches_oracle(gpu_handle, case):
+    batch, space, L, ks, shuffle, dup, seed = case
+    rng = np.random.default_rng(seed)
+    idx = random_voxels(rng, batch, space, L, shuffle=shuffle, duplicates=dup)
+    pad = [k // 2 for k in ks]
+    print("subm case", case, flush=True)
+    p, o, n, n_out = compare(gpu_handle, idx, batch, space, ks, pad, [1, 1, 1], [1, 1, 1], True)
+    K = int(np.prod(ks))
+    if dup == 0:
+        assert n[K // 2] == idx.shape[0]
+        assert np.array_equal(n, n[::-1])
+
+
+REGULAR_CASES = [
+    # (batch, space, L, ks, pad, stride, dil, seed)
+    (1, (6, 6, 6), 40, (3, 3, 3), (1, 1, 1), (2, 2, 2), (1, 1, 1), 0),
+    (2, (9, 10, 11), 300, (3, 3, 3), (1, 1, 1), (2, 2, 2), (1, 1, 1), 1),
+    (2, (9, 10, 11), 300, (3, 3, 3), (0, 1, 1), (2, 1, 2), (1, 1, 1), 2),
+    (1, (12, 12, 12), 500, (3, 3, 3), (2, 2, 2), (1, 1, 1), (2, 2, 2), 3),
+    (1, (12, 12, 12), 500, (2, 2, 2), (0, 0, 0), (2, 2, 2), (1, 1, 1), 4),
+    (3, (8, 16, 16), 1500, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 5),
+    (1, (7, 9, 13), 200, (1, 3, 2), (0, 1, 0), (1, 3, 2), (1, 1, 1), 6),
+    (1, (16, 40, 40), 6000, (3, 3, 3), (1, 1, 1), (2, 2, 2), (1, 1, 1), 7),
+    (1, (10, 10, 10), 300, (3, 1, 3), (1, 0, 2), (1, 2, 1), (1, 1, 2), 8),
+]
+
+
+@pytest.mark.parametrize("case", REGULAR_CASES)
+def test_regular_rulebook_matches_oracle(gpu_handle, case):
+    batch, space, L, ks, pad, stride, dil, seed = case
+    rng = np.random.default_rng(100 + seed)
+    idx = random_voxels(rng, batch, space, L, shuffle=True)
+    print("regular case", case, flush=True)
+    p, o, n, n_out = compare(gpu_handle, idx, batch, space, ks, list(pad), list(stride), list(dil), False)
+    K = int(np.prod(ks))
+    assert n.sum() < K * idx.shape[0]  # at least one invalid (input, offset): oracle count quirk not hit
+    lin_space = out_space(space, ks, pad, stride, dil)
+    lin = ((o[:n_out, 0] * lin_space[0] + o[:n_out, 1]) * lin_space[1] + o[:n_out, 2]) * lin_space[2] + o[:n_out, 3]
+    assert np.all(np.diff(lin) > 0)
+
+
+def test_regular_out_indices_smaller_tensor_is_rejected_cleanly(gpu_handle):
+    """A caller-supplied out_indices with fewer rows than active outputs must not be overrun."""
+    import mluop_hip
+    rng = np.random.default_rng(5)
+    idx = random_voxels(rng, 1, (8, 8, 8), 200)
+    ospace = out_space((8, 8, 8), (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1))
+    with pytest.raises(mluop_hip.MluOpError) as e:
+        run_gpu(gpu_handle, idx, 1, (8, 8, 8), (3, 3, 3), ospace, [1, 1, 1], [1, 1, 1], [1, 1, 1], False,
+                out_rows=10)
+    assert e.value.status == mluop_hip.STATUS_BAD_PARAM
+
+
+def test_config1_subm_rulebook_full_size(gpu_handle):
+    """BASELINE config 1: 20 000 uniform voxels in 1x40x400x352, subm 3x3x3."""
+    import mluop_hip
+    idx = mluop_hip.datagen.uniform_voxels((1, 40, 400, 352), 20000, seed=1)
+    compare(gpu_handle, idx, 1, (40, 400, 352), (3, 3, 3), [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+
+
+def test_config4_subm_rulebook_full_size(gpu_handle):
+    """BASELINE config 4 (headline): 120 000 clustered voxels in 1x41x1600x1408, sorted and shuffled."""
+    import mluop_hip
+    for shuffle in (False, True):
+        idx = mluop_hip.datagen.clustered_voxels((1, 41, 1600, 1408), 120000, seed=4, shuffle=shuffle)
+        print("config4 shuffle", shuffle, flush=True)
+        compare(gpu_handle, idx, 1, (41, 1600, 1408), (3, 3, 3), [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+
+
+def test_config3_regular_rulebook_full_size(gpu_handle):
+    """BASELINE config 3: 4 x 30 000 clustered voxels in 4x41x1600x1408, 3x3x3 stride 2 pad 1."""
+    import mluop_hip
+    idx = mluop_hip.datagen.clustered_voxels((4, 41, 1600, 1408), 30000, seed=3)
+    compare(gpu_handle, idx, 4, (41, 1600, 1408), (3, 3, 3), [1, 1, 1], [2, 2, 2], [1, 1, 1], False)
