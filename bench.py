@@ -1,0 +1,312 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-convolution hot path on one MI355X.
+
+A step is one pass of the path over one synthetic voxel set already resident in HBM:
+mluOpGetIndicePairs (rulebook) followed by mluOpIndiceConvolutionForward, called through the
+library's C ABI with descriptors and workspaces prepared once.  The default workload is BASELINE
+configuration 4 (submanifold 3x3x3, 120 000 clustered voxels in 1x41x1600x1408, Ci=Co=64 fp16).
+
+Prints one JSON line: `value` is the forward operator's algorithmic TFLOP/s (2*P*Ci*Co per call
+over its device time), `rulebook_mvoxels_per_s` the second half of the metric, `roofline`
+describes the kernel that takes the most time in a step, `cpu_baseline` times the CPU oracle on
+the same workload on one host core.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (os.path.join(ROOT, "mlu-ops_amd", "python"), os.path.join(ROOT, "oracle")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+METRIC = "indice_conv fwd TFLOP/s + get_indice_pairs Mvoxels/s, 120k voxels Ci=Co=64"
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+WORKLOADS = {
+    # name: (grid N,D,H,W, voxels per batch, generator, seed, Ci, Co, dtype, kernel)
+    "config4": dict(grid=(1, 41, 1600, 1408), per_batch=120000, gen="clustered", seed=4, ci=64, co=64,
+                    dtype="float16", ks=(3, 3, 3),
+                    text="BASELINE config 4: subm 3x3x3, 120000 clustered voxels in 1x41x1600x1408, "
+                         "Ci=Co=64 fp16, rows sorted by linear cell index"),
+    "config2": dict(grid=(2, 41, 1600, 1408), per_batch=60000, gen="clustered", seed=2, ci=32, co=32,
+                    dtype="float16", ks=(3, 3, 3),
+                    text="BASELINE config 2: subm 3x3x3, 2x60000 clustered voxels in 2x41x1600x1408, "
+                         "Ci=Co=32 fp16"),
+    "config1": dict(grid=(1, 40, 400, 352), per_batch=20000, gen="uniform", seed=1, ci=16, co=16,
+                    dtype="float32", ks=(3, 3, 3),
+                    text="BASELINE config 1: subm 3x3x3, 20000 uniform voxels in 1x40x400x352, Ci=Co=16 fp32"),
+}
+
+
+class Step:
+    """Descriptors, buffers and workspaces of one submanifold layer, built once."""
+
+    def __init__(self, handle, wl):
+        import numpy as np
+        import torch
+        import mluop_hip as m
+        self.m, self.torch, self.handle, self.wl = m, torch, handle, wl
+        grid = wl["grid"]
+        if wl["gen"] == "clustered":
+            idx = m.datagen.clustered_voxels(grid, wl["per_batch"], wl["seed"])
+        else:
+            idx = m.datagen.uniform_voxels(grid, wl["per_batch"] * grid[0], wl["seed"])
+        self.idx_np = idx
+        L = idx.shape[0]
+        ks = wl["ks"]
+        K = ks[0] * ks[1] * ks[2]
+        ci, co = wl["ci"], wl["co"]
+        self.L, self.K, self.ci, self.co = L, K, ci, co
+        tdt = getattr(torch, wl["dtype"])
+        self.elem = 4 if wl["dtype"] == "float32" else 2
+        rng = np.random.default_rng(wl["seed"])
+        self.feats_np = rng.standard_normal((L, ci)).astype(np.float32)
+        self.w_np = m.datagen.kaiming_uniform_filters(ks, ci, co, wl["seed"])
+        self.dy_np = (rng.standard_normal((L, co)) * 0.1).astype(np.float32)
+        dev = "cuda"
+        self.indices = torch.from_numpy(idx).to(dev)
+        self.features = torch.from_numpy(self.feats_np).to(dev, tdt)
+        self.filters = torch.from_numpy(self.w_np).to(dev, tdt)
+        self.dy = torch.from_numpy(self.dy_np).to(dev, tdt)
+        self.pairs = torch.empty((K, 2, L), dtype=torch.int32, device=dev)
+        self.out_indices = torch.empty((L, 4), dtype=torch.int32, device=dev)
+        self.indice_num = torch.empty((K,), dtype=torch.int32, device=dev)
+        self.out = torch.empty((L, co), dtype=tdt, device=dev)
+        self.dx = torch.empty((L, ci), dtype=tdt, device=dev)
+        self.dw = torch.empty(tuple(ks) + (ci, co), dtype=tdt, device=dev)
+        space = list(grid[1:])
+        pad = [k // 2 for k in ks]
+        code = m.torch_dtype_code(tdt)
+        self.sdesc = m.SparseConvDescriptor(grid[0], pad, [1, 1, 1], [1, 1, 1], space, list(ks), space, 1)
+        self.d_idx = m.TensorDescriptor(m.LAYOUT_ARRAY, m.DTYPE_INT32, [L, 4])
+        self.d_pairs = m.TensorDescriptor(m.LAYOUT_ARRAY, m.DTYPE_INT32, [K, 2, L])
+        self.d_oidx = m.TensorDescriptor(m.LAYOUT_ARRAY, m.DTYPE_INT32, [L, 4])
+        self.d_num = m.TensorDescriptor(m.LAYOUT_ARRAY, m.DTYPE_INT32, [K])
+        self.d_feat = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [L, ci])
+        self.d_filt = m.TensorDescriptor(m.LAYOUT_ARRAY, code, list(ks) + [ci, co])
+        self.d_out = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [L, co])
+        self.d_dy = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [L, co])
+        self.d_dx = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [L, ci])
+        self.d_dw = m.TensorDescriptor(m.LAYOUT_ARRAY, code, list(ks) + [ci, co], onchip_dtype=m.DTYPE_FLOAT)
+        lib = m.lib()
+        size = ctypes.c_size_t(0)
+        m.check(lib.mluOpGetIndicePairsWorkspaceSize(handle.ptr, self.sdesc.ptr, self.d_idx.ptr, self.d_pairs.ptr,
+                                                     self.d_oidx.ptr, self.d_num.ptr, ctypes.byref(size)))
+        self.ws_rb_size = size.value
+        self.ws_rb = torch.empty(max(size.value, 1), dtype=torch.uint8, device=dev)
+        # one rulebook build to learn indice_num (the host-side hand-off a framework does once per layer)
+        self.rulebook()
+        torch.cuda.synchronize()
+        self.num_host = self.indice_num.cpu().tolist()
+        self.P = int(sum(self.num_host))
+        self.counts = (ctypes.c_int64 * K)(*self.num_host)
+        m.check(lib.mluOpGetIndiceConvolutionForwardWorkspaceSize(
+            handle.ptr, self.d_feat.ptr, self.d_filt.ptr, self.d_pairs.ptr, self.d_out.ptr, self.counts, L, 0, 1,
+            ctypes.byref(size)))
+        self.ws_fwd_size = size.value
+        self.ws_fwd = torch.empty(max(size.value, 1), dtype=torch.uint8, device=dev)
+        m.check(lib.mluOpGetIndiceConvolutionBackwardDataWorkspaceSize(
+            handle.ptr, self.d_dy.ptr, self.d_filt.ptr, self.d_pairs.ptr, self.d_dx.ptr, self.counts, 0,
+            ctypes.byref(size)))
+        self.ws_bd_size = size.value
+        self.ws_bd = torch.empty(max(size.value, 1), dtype=torch.uint8, device=dev)
+        m.check(lib.mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize(
+            handle.ptr, self.d_feat.ptr, self.d_dy.ptr, self.d_pairs.ptr, self.d_dw.ptr, self.counts, 0, 1,
+            ctypes.byref(size)))
+        self.ws_bf_size = size.value
+        self.ws_bf = torch.empty(max(size.value, 1), dtype=torch.uint8, device=dev)
+
+    def rulebook(self):
+        m = self.m
+        m.check(m.lib().mluOpGetIndicePairs(
+            self.handle.ptr, self.sdesc.ptr, self.d_idx.ptr, self.indices.data_ptr(), self.ws_rb.data_ptr(),
+            self.ws_rb_size, self.d_pairs.ptr, self.pairs.data_ptr(), self.d_oidx.ptr, self.out_indices.data_ptr(),
+            self.d_num.ptr, self.indice_num.data_ptr()), "mluOpGetIndicePairs")
+
+    def forward(self):
+        m = self.m
+        m.check(m.lib().mluOpIndiceConvolutionForward(
+            self.handle.ptr, self.d_feat.ptr, self.features.data_ptr(), self.d_filt.ptr, self.filters.data_ptr(),
+            self.d_pairs.ptr, self.pairs.data_ptr(), self.counts, self.L, 0, 1, self.ws_fwd.data_ptr(),
+            self.ws_fwd_size, self.d_out.ptr, self.out.data_ptr()), "mluOpIndiceConvolutionForward")
+
+    def backward_data(self):
+        m = self.m
+        m.check(m.lib().mluOpIndiceConvolutionBackwardData(
+            self.handle.ptr, self.d_dy.ptr, self.dy.data_ptr(), self.d_filt.ptr, self.filters.data_ptr(),
+            self.d_pairs.ptr, self.pairs.data_ptr(), self.counts, 0, 1, self.ws_bd.data_ptr(), self.ws_bd_size,
+            self.d_dx.ptr, self.dx.data_ptr()), "mluOpIndiceConvolutionBackwardData")
+
+    def backward_filter(self):
+        m = self.m
+        m.check(m.lib().mluOpIndiceConvolutionBackwardFilter(
+            self.handle.ptr, self.d_feat.ptr, self.features.data_ptr(), self.d_dy.ptr, self.dy.data_ptr(),
+            self.d_pairs.ptr, self.pairs.data_ptr(), self.counts, 0, 1, self.ws_bf.data_ptr(), self.ws_bf_size,
+            self.d_dw.ptr, self.dw.data_ptr()), "mluOpIndiceConvolutionBackwardFilter")
+
+    # algorithmic work (per call)
+    def conv_flops(self):
+        return 2.0 * self.P * self.ci * self.co
+
+    def rulebook_bytes(self):
+        return 16.0 * self.L + 8.0 * self.K * self.L + 4.0 * self.K + 16.0 * self.L
+
+    def forward_bytes(self):
+        s = self.elem
+        return self.L * self.ci * s + self.L * self.co * s + self.K * self.ci * self.co * s + 8.0 * self.P
+
+
+def median(v):
+    v = sorted(v)
+    return v[len(v) // 2]
+
+
+def time_ops(torch, ops, steps):
+    """Runs every op of `ops` once per step, with events between them on the current stream.
+    Returns (wall seconds, {name: [ms per step]})."""
+    names = [n for n, _ in ops]
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(ops) + 1)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(steps):
+        ev[s][0].record()
+        for i, (_, fn) in enumerate(ops):
+            fn()
+            ev[s][i + 1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = {n: [ev[s][i].elapsed_time(ev[s][i + 1]) for s in range(steps)] for i, n in enumerate(names)}
+    return wall, per
+
+
+def cpu_baseline(step, reps=3):
+    """The CPU oracle (plain-C restatement of the reference's cpuCompute) on the same workload,
+    one thread: rulebook, then forward on the device-rounded inputs."""
+    import numpy as np
+    import sparse_conv_oracle as oracle
+    wl = step.wl
+    space = list(wl["grid"][1:])
+    ks = list(wl["ks"])
+    pad = [k // 2 for k in ks]
+    rnd = oracle.round_through_half if wl["dtype"] == "float16" else (lambda a: a)
+    feats, w = rnd(step.feats_np), rnd(step.w_np).reshape(step.K, step.ci, step.co)
+    t_rb, t_fw = [], []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        pairs, oidx, num, n_out = oracle.get_indice_pairs(step.idx_np, wl["grid"][0], pad, [1, 1, 1], [1, 1, 1],
+                                                          ks, space, True)
+        t1 = time.perf_counter()
+        oracle.forward(feats, w, pairs, num, n_out)
+        t2 = time.perf_counter()
+        t_rb.append(t1 - t0)
+        t_fw.append(t2 - t1)
+    P = int(np.sum(num))
+    fw, rb = median(t_fw), median(t_rb)
+    return {"value": 2.0 * P * step.ci * step.co / fw / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": "full workload (%d voxels, %d pairs), median of %d runs, gcc -O2 single thread, "
+                      "host has %d logical cores" % (step.L, P, reps, os.cpu_count()),
+            "forward_ms": fw * 1e3, "rulebook_ms": rb * 1e3,
+            "rulebook_mvoxels_per_s": step.L / rb / 1e6}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="config4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only-step", action="store_true",
+                    help="run just warmup + timed steps (for profiler runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the rulebook and the "
+              "convolutions shard by batch index without communication); run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import mluop_hip as m
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    handle = m.make_handle_on_current_stream()
+    wl = WORKLOADS[args.workload]
+    step = Step(handle, wl)
+    step_ops = [("get_indice_pairs", step.rulebook), ("forward", step.forward)]
+
+    for _ in range(args.warmup):
+        for _, fn in step_ops:
+            fn()
+    torch.cuda.synchronize()
+
+    # timed region: exactly --steps steps
+    wall, per = time_ops(torch, step_ops, args.steps)
+    ms_per_step = wall * 1e3 / args.steps
+    fwd_ms = sum(per["forward"]) / args.steps
+    rb_ms = sum(per["get_indice_pairs"]) / args.steps
+    result = {
+        "metric": METRIC, "value": step.conv_flops() / (fwd_ms * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if wl["dtype"] == "float32" else "f16", "data": "synthetic",
+        "config": {"workload": wl["text"] + "; step = get_indice_pairs + indice_convolution_forward",
+                   "voxels": step.L, "pairs": step.P, "Ci": step.ci, "Co": step.co, "kernel_volume": step.K},
+        "rulebook_mvoxels_per_s": step.L / (rb_ms * 1e-3) / 1e6,
+        "forward_ms": fwd_ms, "forward_ms_min": min(per["forward"]),
+        "rulebook_ms": rb_ms, "rulebook_ms_min": min(per["get_indice_pairs"]),
+    }
+    if args.only_step:
+        print(json.dumps(result))
+        return
+
+    # the same steps again with the library's per-kernel event timing switched on
+    handle.set_kernel_timing(True)
+    for _ in range(args.steps):
+        for _, fn in step_ops:
+            fn()
+    records = handle.kernel_timings()
+    handle.set_kernel_timing(False)
+    agg = {}
+    for name, ms in records:
+        tot, cnt = agg.get(name, (0.0, 0))
+        agg[name] = (tot + ms, cnt + 1)
+    kernels = {n: {"avg_us": t / c * 1e3, "launches_per_step": c / args.steps} for n, (t, c) in agg.items()}
+    result["kernels"] = kernels
+    dominant = max(agg, key=lambda n: agg[n][0])
+    dom_ms = agg[dominant][0] / agg[dominant][1]
+    if dominant.startswith("rb"):
+        alg_bytes, what = step.rulebook_bytes(), "rulebook bytes 16L + 8KL + 4K + 16N_out"
+    else:
+        alg_bytes, what = step.forward_bytes(), "forward bytes L*Ci*s + N*Co*s + K*Ci*Co*s + 8P"
+    achieved = alg_bytes / (dom_ms * 1e-3) / 1e9
+    result["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": dominant,
+                          "kernel_avg_us": dom_ms * 1e3, "algorithmic_bytes": alg_bytes, "bytes_model": what}
+    if "gatherConvMfma" in agg:
+        g_ms = agg["gatherConvMfma"][0] / agg["gatherConvMfma"][1]
+        result["forward_kernel"] = {
+            "kernel": "gatherConvMfma", "avg_us": g_ms * 1e3,
+            "hbm_frac": step.forward_bytes() / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "mfma_frac": step.conv_flops() / (g_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS}
+
+    # the two backward operators of the same layer, reported beside the metric
+    _, per_b = time_ops(torch, [("backward_data", step.backward_data), ("backward_filter", step.backward_filter)],
+                        max(args.steps // 4, 5))
+    result["backward_data_ms"] = median(per_b["backward_data"])
+    result["backward_filter_ms"] = median(per_b["backward_filter"])
+    result["backward_data_tflops"] = step.conv_flops() / (result["backward_data_ms"] * 1e-3) / 1e12
+    result["backward_filter_tflops"] = step.conv_flops() / (result["backward_filter_ms"] * 1e-3) / 1e12
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(step)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -7,6 +7,7 @@
 #include <new>
 
 #include "core/core.h"
+#include "mlu_op_ext.h"
 
 namespace {
 
@@ -76,6 +77,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpCreate(mluOpHandle_t *handle) {
 mluOpStatus_t MLUOP_WIN_API mluOpDestroy(mluOpHandle_t handle) {
   PARAM_CHECK("[mluOpDestroy]", handle != NULL);
   if (handle->pinned_scalar != nullptr) (void)hipHostFree(handle->pinned_scalar);
+  handle->timer.destroy();
   delete handle;
   return MLUOP_STATUS_SUCCESS;
 }
@@ -123,6 +125,37 @@ mluOpStatus_t MLUOP_WIN_API mluOpGetAtomicsMode(mluOpHandle_t handle,
   PARAM_CHECK("[mluOpGetAtomicsMode]", handle != NULL);
   PARAM_CHECK("[mluOpGetAtomicsMode]", atomics_mode != NULL);
   *atomics_mode = handle->atomics_mode;
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelTiming(mluOpHandle_t handle, int enable) {
+  PARAM_CHECK("[mluOpExtSetKernelTiming]", handle != NULL);
+  if (handle->device >= 0) (void)hipStreamSynchronize(handle->queue);
+  handle->timer.clear();
+  handle->timer.enabled = enable != 0 && handle->device >= 0;
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpExtGetKernelTimingCount(mluOpHandle_t handle, int *count) {
+  PARAM_CHECK("[mluOpExtGetKernelTimingCount]", handle != NULL);
+  PARAM_CHECK("[mluOpExtGetKernelTimingCount]", count != NULL);
+  if (handle->device >= 0) {
+    HIP_CHECK_RETURN("[mluOpExtGetKernelTimingCount]", hipStreamSynchronize(handle->queue));
+  }
+  *count = (int)handle->timer.records.size();
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpExtGetKernelTiming(mluOpHandle_t handle, int index,
+                                                    const char **name, float *milliseconds) {
+  const char *api = "[mluOpExtGetKernelTiming]";
+  PARAM_CHECK(api, handle != NULL);
+  PARAM_CHECK(api, name != NULL);
+  PARAM_CHECK(api, milliseconds != NULL);
+  PARAM_CHECK(api, index >= 0 && index < (int)handle->timer.records.size());
+  const mluop::KernelTimingRecord &r = handle->timer.records[index];
+  *name = r.name;
+  HIP_CHECK_RETURN(api, hipEventElapsedTime(milliseconds, r.start, r.stop));
   return MLUOP_STATUS_SUCCESS;
 }
 

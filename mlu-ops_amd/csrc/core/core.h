@@ -10,7 +10,9 @@
 #include <cstdio>
 #include <sstream>
 #include <string>
+#include <vector>
 
+#include "core/launch.h"
 #include "mlu_op.h"
 
 // reference core/logging.h:37, get_indice_pairs_structs.h:36
@@ -31,6 +33,10 @@ struct mluOpContext {
   mluOpQuantizeRoundMode_t round_mode = MLUOP_ROUND_HALF_TO_EVEN;
   mluOpAtomicsMode_t atomics_mode = MLUOP_ATOMICS_NOT_ALLOWED;
   int32_t *pinned_scalar = nullptr;  // 64-byte pinned host slot for read-backs
+  mluop::KernelTimer timer;          // per-kernel event timing, off by default
+
+  // What the kernel launchers need: the stream, and the timer while it is on.
+  mluop::LaunchCtx launchCtx() { return mluop::LaunchCtx(queue, timer.enabled ? &timer : nullptr); }
 };
 
 // ---------------------------------------------------------------------------

@@ -156,7 +156,7 @@ mluOpStatus_t internalGetIndicePairs(mluOpHandle_t handle, const std::string &ap
 
   if (g.sub_m) {
     HIP_CHECK_RETURN(api, mluop::sparse_conv::launchSubmRulebook(
-                              handle->queue, g, static_cast<const int32_t *>(indices), workspace,
+                              handle->launchCtx(), g, static_cast<const int32_t *>(indices), workspace,
                               static_cast<int32_t *>(indice_pairs),
                               static_cast<int32_t *>(out_indices),
                               static_cast<int32_t *>(indice_num)));
@@ -166,7 +166,7 @@ mluOpStatus_t internalGetIndicePairs(mluOpHandle_t handle, const std::string &ap
   }
 
   HIP_CHECK_RETURN(api, mluop::sparse_conv::launchRegularRulebook(
-                            handle->queue, g, static_cast<const int32_t *>(indices), workspace,
+                            handle->launchCtx(), g, static_cast<const int32_t *>(indices), workspace,
                             static_cast<int32_t *>(indice_pairs),
                             static_cast<int32_t *>(out_indices),
                             static_cast<int32_t *>(indice_num), handle->pinned_scalar));

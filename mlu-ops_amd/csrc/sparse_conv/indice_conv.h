@@ -8,6 +8,8 @@
 #include <cstddef>
 #include <cstdint>
 
+#include "core/launch.h"
+
 namespace mluop {
 namespace sparse_conv {
 
@@ -42,12 +44,12 @@ struct ConvProblem {
 enum class GatherDirection { kForward, kBackwardData };
 
 size_t gatherConvWorkspaceBytes(const ConvProblem &p, GatherDirection dir);
-hipError_t launchGatherConv(hipStream_t stream, const ConvProblem &p, GatherDirection dir,
+hipError_t launchGatherConv(const LaunchCtx &lc, const ConvProblem &p, GatherDirection dir,
                             const void *gathered, const FilterView &filters, void *workspace,
                             void *result);
 
 size_t backwardFilterWorkspaceBytes(const ConvProblem &p);
-hipError_t launchBackwardFilter(hipStream_t stream, const ConvProblem &p, const void *features,
+hipError_t launchBackwardFilter(const LaunchCtx &lc, const ConvProblem &p, const void *features,
                                 const void *output_grad, void *workspace, void *filters_grad);
 
 }  // namespace sparse_conv

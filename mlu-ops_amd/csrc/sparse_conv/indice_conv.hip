@@ -519,7 +519,7 @@ GatherWorkspace carveGather(const ConvProblem &p, const GatherDims &d, void *bas
 
 // Fills the by-value counts (K <= kMaxInlineK) or uploads them.  The int32
 // staging vector is consumed by a synchronous-with-host pageable copy.
-hipError_t prepareCounts(hipStream_t stream, const ConvProblem &p, OffsetCounts *inl,
+hipError_t prepareCounts(const LaunchCtx &lc, const ConvProblem &p, OffsetCounts *inl,
                          int32_t *dev_counts, int *max_count) {
   int mx = 0;
   for (int k = 0; k < p.K; ++k) {
@@ -543,52 +543,54 @@ hipError_t prepareCounts(hipStream_t stream, const ConvProblem &p, OffsetCounts 
     int64_t n = p.indice_num[k];
     tmp[k] = (int)(n < 0 ? 0 : (n > p.L ? p.L : n));
   }
-  hipError_t err = hipMemcpyAsync(dev_counts, tmp, (size_t)p.K * 4, hipMemcpyHostToDevice, stream);
-  if (err == hipSuccess) err = hipStreamSynchronize(stream);
+  hipError_t err = hipMemcpyAsync(dev_counts, tmp, (size_t)p.K * 4, hipMemcpyHostToDevice, lc.stream);
+  if (err == hipSuccess) err = hipStreamSynchronize(lc.stream);
   free(tmp);
   return err;
 }
 
 template <typename E, int Q, int C>
-void launchMfmaInstance(hipStream_t stream, const void *A, const void *packed,
+void launchMfmaInstance(const LaunchCtx &lc, const void *A, const void *packed,
                         const int32_t *map, int R, int K, const OffsetCounts &inl,
                         const int32_t *dev_counts, void *result) {
   constexpr int NT = 64 * (C / 16 / mfmaColBlocksPerWave(C));
   constexpr int TR = mfmaTileRows(C);
   const int blocks = (R + TR - 1) / TR;
-  gatherConvMfma<E, Q, C><<<blocks, NT, 0, stream>>>(
+  lc.begin("gatherConvMfma");
+  gatherConvMfma<E, Q, C><<<blocks, NT, 0, lc.stream>>>(
       static_cast<const typename E::storage *>(A),
       static_cast<const typename E::storage *>(packed), map, R, K, inl, dev_counts,
       static_cast<typename E::storage *>(result));
+  lc.end();
 }
 
 template <typename E, int Q>
-void launchMfmaByC(hipStream_t stream, int C, const void *A, const void *packed,
+void launchMfmaByC(const LaunchCtx &lc, int C, const void *A, const void *packed,
                    const int32_t *map, int R, int K, const OffsetCounts &inl,
                    const int32_t *dev_counts, void *result) {
   switch (C) {
-    case 16: launchMfmaInstance<E, Q, 16>(stream, A, packed, map, R, K, inl, dev_counts, result); break;
-    case 32: launchMfmaInstance<E, Q, 32>(stream, A, packed, map, R, K, inl, dev_counts, result); break;
-    case 64: launchMfmaInstance<E, Q, 64>(stream, A, packed, map, R, K, inl, dev_counts, result); break;
-    case 128: launchMfmaInstance<E, Q, 128>(stream, A, packed, map, R, K, inl, dev_counts, result); break;
+    case 16: launchMfmaInstance<E, Q, 16>(lc, A, packed, map, R, K, inl, dev_counts, result); break;
+    case 32: launchMfmaInstance<E, Q, 32>(lc, A, packed, map, R, K, inl, dev_counts, result); break;
+    case 64: launchMfmaInstance<E, Q, 64>(lc, A, packed, map, R, K, inl, dev_counts, result); break;
+    case 128: launchMfmaInstance<E, Q, 128>(lc, A, packed, map, R, K, inl, dev_counts, result); break;
     default: break;
   }
 }
 
 template <typename E>
-void launchMfma(hipStream_t stream, int Q, int C, const void *A, const void *packed,
+void launchMfma(const LaunchCtx &lc, int Q, int C, const void *A, const void *packed,
                 const int32_t *map, int R, int K, const OffsetCounts &inl,
                 const int32_t *dev_counts, void *result) {
   switch (Q) {
-    case 32: launchMfmaByC<E, 32>(stream, C, A, packed, map, R, K, inl, dev_counts, result); break;
-    case 64: launchMfmaByC<E, 64>(stream, C, A, packed, map, R, K, inl, dev_counts, result); break;
-    case 128: launchMfmaByC<E, 128>(stream, C, A, packed, map, R, K, inl, dev_counts, result); break;
+    case 32: launchMfmaByC<E, 32>(lc, C, A, packed, map, R, K, inl, dev_counts, result); break;
+    case 64: launchMfmaByC<E, 64>(lc, C, A, packed, map, R, K, inl, dev_counts, result); break;
+    case 128: launchMfmaByC<E, 128>(lc, C, A, packed, map, R, K, inl, dev_counts, result); break;
     default: break;
   }
 }
 
 template <typename E>
-void launchGatherTyped(hipStream_t stream, const ConvProblem &p, const GatherDims &d,
+void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d,
                        const GatherWorkspace &ws, const OffsetCounts &inl, const void *gathered,
                        const FilterView &f, bool use_mfma, void *result) {
   typedef typename E::storage S;
@@ -598,19 +600,23 @@ void launchGatherTyped(hipStream_t stream, const ConvProblem &p, const GatherDim
   if (use_mfma) {
     if constexpr (!std::is_same<E, FloatElem>::value) {
       const size_t frags = (size_t)p.K * (d.C / 16) * (d.Q / 32) * 64;
-      packFilterFragments<E><<<gridFor(frags), 256, 0, stream>>>(
+      lc.begin("packFilterFragments");
+      packFilterFragments<E><<<gridFor(frags), 256, 0, lc.stream>>>(
           static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K, d.Q, d.C,
           static_cast<S *>(ws.packed));
-      launchMfma<E>(stream, d.Q, d.C, gathered, ws.packed, ws.map, d.R, p.K, inl, ws.dev_counts,
+      lc.end();
+      launchMfma<E>(lc, d.Q, d.C, gathered, ws.packed, ws.map, d.R, p.K, inl, ws.dev_counts,
                     result);
     }
     return;
   }
   dim3 grid((d.R + 31) / 32, (d.C + 63) / 64);
-  gatherConvSimt<E><<<grid, 256, 0, stream>>>(static_cast<const S *>(gathered), d.Q,
+  lc.begin("gatherConvSimt");
+  gatherConvSimt<E><<<grid, 256, 0, lc.stream>>>(static_cast<const S *>(gathered), d.Q,
                                               static_cast<const S *>(f.base), f.stride_k, sQ, sC,
                                               ws.map, d.R, p.K, inl, ws.dev_counts, d.C,
                                               static_cast<S *>(result));
+  lc.end();
 }
 
 struct FilterGradWorkspace {
@@ -647,20 +653,24 @@ FilterGradWorkspace carveFilterGrad(const ConvProblem &p, void *base) {
 }
 
 template <typename E>
-void launchFilterGradTyped(hipStream_t stream, const ConvProblem &p,
+void launchFilterGradTyped(const LaunchCtx &lc, const ConvProblem &p,
                            const FilterGradWorkspace &ws, const OffsetCounts &inl,
                            const void *features, const void *output_grad, void *filters_grad) {
   typedef typename E::storage S;
   const int tiles = ((p.Ci + 31) / 32) * ((p.Co + 63) / 64);
   dim3 grid(tiles, p.K, ws.splits);
-  backwardFilterSimt<E><<<grid, 256, 0, stream>>>(
+  lc.begin("backwardFilterSimt");
+  backwardFilterSimt<E><<<grid, 256, 0, lc.stream>>>(
       static_cast<const S *>(features), static_cast<const S *>(output_grad), p.indice_pairs, p.L,
       p.L, p.num_out, p.Ci, p.Co, inl, ws.dev_counts, ws.splits, ws.partial,
       static_cast<S *>(filters_grad));
+  lc.end();
   if (ws.splits > 1) {
     const size_t n = (size_t)p.K * p.Ci * p.Co;
-    reduceFilterPartials<E><<<gridFor(n), 256, 0, stream>>>(ws.partial, n, ws.splits,
+    lc.begin("reduceFilterPartials");
+    reduceFilterPartials<E><<<gridFor(n), 256, 0, lc.stream>>>(ws.partial, n, ws.splits,
                                                             static_cast<S *>(filters_grad));
+    lc.end();
   }
 }
 
@@ -670,22 +680,26 @@ size_t gatherConvWorkspaceBytes(const ConvProblem &p, GatherDirection dir) {
   return carveGather(p, gatherDims(p, dir), nullptr).bytes;
 }
 
-hipError_t launchGatherConv(hipStream_t stream, const ConvProblem &p, GatherDirection dir,
+hipError_t launchGatherConv(const LaunchCtx &lc, const ConvProblem &p, GatherDirection dir,
                             const void *gathered, const FilterView &filters, void *workspace,
                             void *result) {
   const GatherDims d = gatherDims(p, dir);
   const GatherWorkspace ws = carveGather(p, d, workspace);
   OffsetCounts inl;
   int max_count = 0;
-  hipError_t err = prepareCounts(stream, p, &inl, ws.dev_counts, &max_count);
+  hipError_t err = prepareCounts(lc, p, &inl, ws.dev_counts, &max_count);
   if (err != hipSuccess) return err;
 
   const size_t map_elems = (size_t)p.K * d.R;
-  fillInt32<<<gridFor(map_elems), 256, 0, stream>>>(ws.map, map_elems, -1);
+  lc.begin("fillInt32");
+  fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems, -1);
+  lc.end();
   if (max_count > 0) {
     dim3 grid((max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256, p.K);
-    scatterRowMap<<<grid, 256, 0, stream>>>(p.indice_pairs, p.L, inl, ws.dev_counts, d.row_col,
+    lc.begin("scatterRowMap");
+    scatterRowMap<<<grid, 256, 0, lc.stream>>>(p.indice_pairs, p.L, inl, ws.dev_counts, d.row_col,
                                             d.src_col, d.R, d.n_src, ws.map);
+    lc.end();
   }
   // The MFMA kernel moves rows with 16-byte accesses.
   const bool ptr_ok =
@@ -693,13 +707,13 @@ hipError_t launchGatherConv(hipStream_t stream, const ConvProblem &p, GatherDire
   const bool use_mfma = mfmaShapeOk(p.dtype, d.Q, d.C) && ptr_ok && !forceSimt();
   switch (p.dtype) {
     case ElemType::kHalf:
-      launchGatherTyped<HalfElem>(stream, p, d, ws, inl, gathered, filters, use_mfma, result);
+      launchGatherTyped<HalfElem>(lc, p, d, ws, inl, gathered, filters, use_mfma, result);
       break;
     case ElemType::kBFloat16:
-      launchGatherTyped<BFloat16Elem>(stream, p, d, ws, inl, gathered, filters, use_mfma, result);
+      launchGatherTyped<BFloat16Elem>(lc, p, d, ws, inl, gathered, filters, use_mfma, result);
       break;
     case ElemType::kFloat:
-      launchGatherTyped<FloatElem>(stream, p, d, ws, inl, gathered, filters, false, result);
+      launchGatherTyped<FloatElem>(lc, p, d, ws, inl, gathered, filters, false, result);
       break;
   }
   return hipGetLastError();
@@ -709,23 +723,23 @@ size_t backwardFilterWorkspaceBytes(const ConvProblem &p) {
   return carveFilterGrad(p, nullptr).bytes;
 }
 
-hipError_t launchBackwardFilter(hipStream_t stream, const ConvProblem &p, const void *features,
+hipError_t launchBackwardFilter(const LaunchCtx &lc, const ConvProblem &p, const void *features,
                                 const void *output_grad, void *workspace, void *filters_grad) {
   const FilterGradWorkspace ws = carveFilterGrad(p, workspace);
   OffsetCounts inl;
   int max_count = 0;
-  hipError_t err = prepareCounts(stream, p, &inl, ws.dev_counts, &max_count);
+  hipError_t err = prepareCounts(lc, p, &inl, ws.dev_counts, &max_count);
   if (err != hipSuccess) return err;
   switch (p.dtype) {
     case ElemType::kHalf:
-      launchFilterGradTyped<HalfElem>(stream, p, ws, inl, features, output_grad, filters_grad);
+      launchFilterGradTyped<HalfElem>(lc, p, ws, inl, features, output_grad, filters_grad);
       break;
     case ElemType::kBFloat16:
-      launchFilterGradTyped<BFloat16Elem>(stream, p, ws, inl, features, output_grad,
+      launchFilterGradTyped<BFloat16Elem>(lc, p, ws, inl, features, output_grad,
                                           filters_grad);
       break;
     case ElemType::kFloat:
-      launchFilterGradTyped<FloatElem>(stream, p, ws, inl, features, output_grad, filters_grad);
+      launchFilterGradTyped<FloatElem>(lc, p, ws, inl, features, output_grad, filters_grad);
       break;
   }
   return hipGetLastError();

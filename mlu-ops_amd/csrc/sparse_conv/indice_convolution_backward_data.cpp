@@ -294,7 +294,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardData(
   DEVICE_HANDLE_CHECK(api, handle);
   const FilterView f = filterView(filters_desc, filters, p);
   HIP_CHECK_RETURN(api, mluop::sparse_conv::launchGatherConv(
-                            handle->queue, p, GatherDirection::kBackwardData, output_grad, f,
+                            handle->launchCtx(), p, GatherDirection::kBackwardData, output_grad, f,
                             workspace, input_grad));
   return MLUOP_STATUS_SUCCESS;
 }

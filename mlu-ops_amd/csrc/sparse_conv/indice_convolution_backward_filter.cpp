@@ -208,7 +208,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardFilter(
     return MLUOP_STATUS_BAD_PARAM;
   }
   DEVICE_HANDLE_CHECK(api, handle);
-  HIP_CHECK_RETURN(api, mluop::sparse_conv::launchBackwardFilter(handle->queue, p, features,
+  HIP_CHECK_RETURN(api, mluop::sparse_conv::launchBackwardFilter(handle->launchCtx(), p, features,
                                                                 output_grad, workspace,
                                                                 filters_grad));
   return MLUOP_STATUS_SUCCESS;

@@ -235,7 +235,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionForward(
   }
   DEVICE_HANDLE_CHECK(api, handle);
   const FilterView f = forwardFilterView(filters_desc, filters, p);
-  HIP_CHECK_RETURN(api, mluop::sparse_conv::launchGatherConv(handle->queue, p,
+  HIP_CHECK_RETURN(api, mluop::sparse_conv::launchGatherConv(handle->launchCtx(), p,
                                                             GatherDirection::kForward, features,
                                                             f, workspace, features_out));
   return MLUOP_STATUS_SUCCESS;

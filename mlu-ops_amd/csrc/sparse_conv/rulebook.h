@@ -7,6 +7,8 @@
 #include <cstddef>
 #include <cstdint>
 
+#include "core/launch.h"
+
 namespace mluop {
 namespace sparse_conv {
 
@@ -28,15 +30,15 @@ struct RulebookGeom {
 // Bytes of device workspace the kernel set needs for this geometry.
 size_t rulebookWorkspaceBytes(const RulebookGeom &g);
 
-// Enqueues submanifold rulebook construction on `stream`.
-hipError_t launchSubmRulebook(hipStream_t stream, const RulebookGeom &g, const int32_t *indices,
+// Enqueues submanifold rulebook construction on the context's stream.
+hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const int32_t *indices,
                               void *workspace, int32_t *indice_pairs, int32_t *out_indices,
                               int32_t *indice_num);
 
-// Enqueues regular (strided / dilated) rulebook construction on `stream` and
+// Enqueues regular (strided / dilated) rulebook construction and
 // an asynchronous copy of the number of active outputs into `host_num_act_out`
 // (pinned host memory).  The caller synchronises the stream before reading it.
-hipError_t launchRegularRulebook(hipStream_t stream, const RulebookGeom &g,
+hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                  const int32_t *indices, void *workspace, int32_t *indice_pairs,
                                  int32_t *out_indices, int32_t *indice_num,
                                  int32_t *host_num_act_out);

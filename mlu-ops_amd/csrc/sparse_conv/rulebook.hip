@@ -417,7 +417,7 @@ inline int fillBlocks(size_t n) {
 
 size_t rulebookWorkspaceBytes(const RulebookGeom &g) { return carve(g, nullptr).bytes; }
 
-hipError_t launchSubmRulebook(hipStream_t stream, const RulebookGeom &g, const int32_t *indices,
+hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const int32_t *indices,
                               void *workspace, int32_t *indice_pairs, int32_t *out_indices,
                               int32_t *indice_num) {
   const Workspace ws = carve(g, workspace);
@@ -428,18 +428,28 @@ hipError_t launchSubmRulebook(hipStream_t stream, const RulebookGeom &g, const i
   const int row_blocks = (rows + kBlock - 1) / kBlock;
   const int l_blocks = (g.L + kBlock - 1) / kBlock;
 
-  rbFill64<<<fillBlocks(ws.table_cap), kBlock, 0, stream>>>(ws.table, ws.table_cap, kEmptySlot);
-  rbSubmInsert<<<row_blocks, kBlock, 0, stream>>>(d, indices, al, ws.table, mask, out_indices,
+  lc.begin("rbFill64");
+  rbFill64<<<fillBlocks(ws.table_cap), kBlock, 0, lc.stream>>>(ws.table, ws.table_cap, kEmptySlot);
+  lc.end();
+  lc.begin("rbSubmInsert");
+  rbSubmInsert<<<row_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.table, mask, out_indices,
                                                   g.out_rows);
-  rbProbeCount<true><<<l_blocks, kBlock, 0, stream>>>(d, indices, al, ws.table, mask, nullptr,
+  lc.end();
+  lc.begin("rbProbeCount");
+  rbProbeCount<true><<<l_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.table, mask, nullptr,
                                                       ws.cand, ws.counts, ws.n_wave);
-  rbScanRows<<<g.K, kBlock, 0, stream>>>(ws.counts, ws.n_wave, indice_num);
-  rbEmitPairs<true><<<l_blocks, kBlock, 0, stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
+  lc.end();
+  lc.begin("rbScanRows");
+  rbScanRows<<<g.K, kBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
+  lc.end();
+  lc.begin("rbEmitPairs");
+  rbEmitPairs<true><<<l_blocks, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
                                                      indice_num, nullptr, nullptr, indice_pairs);
+  lc.end();
   return hipGetLastError();
 }
 
-hipError_t launchRegularRulebook(hipStream_t stream, const RulebookGeom &g,
+hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                  const int32_t *indices, void *workspace, int32_t *indice_pairs,
                                  int32_t *out_indices, int32_t *indice_num,
                                  int32_t *host_num_act_out) {
@@ -449,23 +459,37 @@ hipError_t launchRegularRulebook(hipStream_t stream, const RulebookGeom &g,
   const bool al_out = aligned16(out_indices, out_indices);
   const int l_blocks = (g.L + kBlock - 1) / kBlock;
 
-  rbFill64<<<fillBlocks(ws.n_words), kBlock, 0, stream>>>(ws.bitmap, ws.n_words, 0ull);
-  rbProbeCount<false><<<l_blocks, kBlock, 0, stream>>>(d, indices, al_in, nullptr, 0, ws.bitmap,
+  lc.begin("rbFill64");
+  rbFill64<<<fillBlocks(ws.n_words), kBlock, 0, lc.stream>>>(ws.bitmap, ws.n_words, 0ull);
+  lc.end();
+  lc.begin("rbProbeCount");
+  rbProbeCount<false><<<l_blocks, kBlock, 0, lc.stream>>>(d, indices, al_in, nullptr, 0, ws.bitmap,
                                                        ws.cand, ws.counts, ws.n_wave);
-  rbScanRows<<<g.K, kBlock, 0, stream>>>(ws.counts, ws.n_wave, indice_num);
-  rbBitmapBlockSum<<<ws.n_bitmap_blocks, kBlock, 0, stream>>>(ws.bitmap, ws.n_words,
+  lc.end();
+  lc.begin("rbScanRows");
+  rbScanRows<<<g.K, kBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
+  lc.end();
+  lc.begin("rbBitmapBlockSum");
+  rbBitmapBlockSum<<<ws.n_bitmap_blocks, kBlock, 0, lc.stream>>>(ws.bitmap, ws.n_words,
                                                               ws.block_sum);
-  rbScanRows<<<1, kBlock, 0, stream>>>(ws.block_sum, ws.n_bitmap_blocks, ws.num_act_out);
+  lc.end();
+  lc.begin("rbScanRows");
+  rbScanRows<<<1, kBlock, 0, lc.stream>>>(ws.block_sum, ws.n_bitmap_blocks, ws.num_act_out);
+  lc.end();
   hipError_t err = hipMemcpyAsync(host_num_act_out, ws.num_act_out, sizeof(int32_t),
-                                  hipMemcpyDeviceToHost, stream);
+                                  hipMemcpyDeviceToHost, lc.stream);
   if (err != hipSuccess) return err;
-  rbRankAndDecode<<<ws.n_bitmap_blocks, kBlock, 0, stream>>>(d, ws.bitmap, ws.n_words,
+  lc.begin("rbRankAndDecode");
+  rbRankAndDecode<<<ws.n_bitmap_blocks, kBlock, 0, lc.stream>>>(d, ws.bitmap, ws.n_words,
                                                              ws.block_sum, ws.num_act_out,
                                                              ws.word_rank, out_indices, al_out,
                                                              g.out_rows);
-  rbEmitPairs<false><<<l_blocks, kBlock, 0, stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
+  lc.end();
+  lc.begin("rbEmitPairs");
+  rbEmitPairs<false><<<l_blocks, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
                                                       indice_num, ws.bitmap, ws.word_rank,
                                                       indice_pairs);
+  lc.end();
   return hipGetLastError();
 }
 

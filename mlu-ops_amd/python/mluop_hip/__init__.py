@@ -102,6 +102,11 @@ SIGNATURES = {
     "mluOpIndiceConvolutionBackwardFilter": (
         ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64p, ctypes.c_int64, ctypes.c_int64,
                        _vp, ctypes.c_size_t, _vp, _vp]),
+    # mlu_op_ext.h
+    "mluOpExtSetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "mluOpExtGetKernelTimingCount": (ctypes.c_int, [_vp, _ip]),
+    "mluOpExtGetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int, ctypes.POINTER(ctypes.c_char_p),
+                                               ctypes.POINTER(ctypes.c_float)]),
 }
 
 _lib = None
@@ -152,6 +157,21 @@ class Handle:
 
     def set_queue(self, queue):
         check(lib().mluOpSetQueue(self.ptr, _vp(queue)), "mluOpSetQueue")
+
+    def set_kernel_timing(self, enable):
+        check(lib().mluOpExtSetKernelTiming(self.ptr, 1 if enable else 0))
+
+    def kernel_timings(self):
+        """[(kernel name, milliseconds)] per launch since timing was enabled (waits for the queue)."""
+        n = ctypes.c_int(0)
+        check(lib().mluOpExtGetKernelTimingCount(self.ptr, ctypes.byref(n)))
+        out = []
+        name = ctypes.c_char_p()
+        ms = ctypes.c_float(0)
+        for i in range(n.value):
+            check(lib().mluOpExtGetKernelTiming(self.ptr, i, ctypes.byref(name), ctypes.byref(ms)))
+            out.append((name.value.decode(), ms.value))
+        return out
 
     def close(self):
         if self.ptr:
