@@ -209,29 +209,36 @@ __global__ __launch_bounds__(256) void packFilterFragments(const typename E::sto
   }
 }
 
-// Position of the n-th (0-based) set bit of m; m must have more than n bits set.
-__device__ __forceinline__ int nthSetBit(unsigned long long m, int n) {
-  int pos = 0;
-#pragma unroll
-  for (int width = 32; width >= 1; width >>= 1) {
-    const unsigned long long low = (m >> pos) & ((1ull << width) - 1ull);
-    const int c = __popcll(low);
-    if (n >= c) {
-      n -= c;
-      pos += width;
-    }
-  }
-  return pos;
-}
-
 constexpr int mfmaTileRows(int C) {
-  // fp32 accumulator tile of at most 48 KiB, a multiple of 64 rows, at most 256.
-  return (12288 / C) >= 256 ? 256 : ((12288 / C) / 64 * 64 < 64 ? 64 : (12288 / C) / 64 * 64);
+  // fp32 accumulator tile of at most 32 KiB: four workgroups share a CU's LDS.
+  return C <= 32 ? 256 : (C <= 64 ? 128 : 64);
 }
 constexpr int mfmaColBlocksPerWave(int C) { return C >= 128 ? 2 : 1; }
+constexpr int mfmaBlocksInFlight(int Q, int C) {
+  // Register budget: each block in flight holds Q/32 A fragments and
+  // Q/32 * column-blocks B fragments (4 VGPRs each).
+  return (Q / 32) * (1 + mfmaColBlocksPerWave(C)) <= 4 ? 4 : 2;
+}
 
-constexpr int kMaskChunk = 128;  // offsets whose ballot masks are resident in LDS at once
+constexpr int kOffsetChunk = 9;  // offsets whose pair lists are resident in LDS at once
 
+// Workgroup = TR result rows x all C columns; wave w owns columns
+// [w*16*NB, (w+1)*16*NB) of the fp32 accumulator tile in LDS, so no two waves
+// ever touch the same accumulator element and every element sees its
+// contributions in ascending offset order.
+//
+// Per chunk of kOffsetChunk offsets:
+//   A   lanes hold map[k][row] for all offsets of the chunk (loaded while the
+//       previous chunk was being multiplied), ballot which rows have a partner
+//       and compact the (row, partner) entries of every offset into LDS lists;
+//       one wave turns the list lengths into a flat list of 16-entry blocks;
+//   B   every wave walks the block list, several blocks in flight: gather 16
+//       partner rows as the MFMA A operand (zero rows pad a short block),
+//       multiply by its B fragments of W[k], add the 16 x 16*NB result into
+//       the accumulator rows of the entries.
+// The accumulator tile is stored with its 16-column groups XOR-swizzled by the
+// row index so that the four rows a wave updates at once fall into different
+// LDS banks more often than not.
 template <typename E, int Q, int C>
 __global__ __launch_bounds__(64 * (C / 16 / mfmaColBlocksPerWave(C)))
 void gatherConvMfma(const typename E::storage *A, const typename E::storage *packedW,
@@ -243,102 +250,189 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   constexpr int NT = 64 * WAVES;
   constexpr int TR = mfmaTileRows(C);
   constexpr int NSEG = TR / 64;
+  constexpr int SEG_ITERS = (NSEG + WAVES - 1) / WAVES;  // segments a wave scans
   constexpr int KB = Q / 32;
+  constexpr int KC = kOffsetChunk;
+  constexpr int D = mfmaBlocksInFlight(Q, C);
+  constexpr int GROUPS = C / 16;  // 16-column groups per accumulator row (power of two)
+  constexpr int MAX_BLOCKS = KC * (TR / 16);
 
   __shared__ float s_acc[TR * C];
-  __shared__ unsigned long long s_mask[kMaskChunk][NSEG];
+  __shared__ int32_t s_src[KC][TR];
+  __shared__ __attribute__((aligned(4))) uint8_t s_row[KC][TR];
+  __shared__ int s_cnt[KC][NSEG];
+  __shared__ int s_tot[KC];
+  __shared__ uint16_t s_blk[MAX_BLOCKS];
+  __shared__ int s_nblk;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int r0 = blockIdx.x * TR;
-  const int col0 = wave * 16 * NB;
+  const int grp0 = wave * NB;  // first 16-column group of this wave
+  const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
   for (int i = tid; i < TR * C; i += NT) s_acc[i] = 0.f;
 
-  for (int kc = 0; kc < K; kc += kMaskChunk) {
-    const int kn = (K - kc) < kMaskChunk ? (K - kc) : kMaskChunk;
-    __syncthreads();
-    // Phase A: which rows of the tile have a partner at offset k.
-    for (int kk = 0; kk < kn; ++kk) {
-      const int k = kc + kk;
-      const bool live = offsetCount(inl, dev_counts, k) > 0;
-      for (int seg = wave; seg < NSEG; seg += WAVES) {
-        const int r = r0 + seg * 64 + lane;
-        int idx = -1;
-        if (live && r < R) idx = map[(size_t)k * R + r];
-        const unsigned long long b = __ballot(idx >= 0);
-        if (lane == 0) s_mask[kk][seg] = b;
+  // map entries of the chunk being prepared, per segment this wave scans
+  int idx[SEG_ITERS][KC];
+  auto load_chunk = [&](int kc) {
+#pragma unroll
+    for (int it = 0; it < SEG_ITERS; ++it) {
+      const int seg = wave + it * WAVES;
+      const int r = r0 + seg * 64 + lane;
+#pragma unroll
+      for (int kk = 0; kk < KC; ++kk) {
+        // Unconditional loads from clamped addresses keep all of them in flight;
+        // offsets without pairs hold -1 everywhere in the map.
+        const bool ok = seg < NSEG && kc + kk < K && r < R;
+        const int k_safe = kc + kk < K ? kc + kk : K - 1;
+        const int r_safe = (seg < NSEG && r < R) ? r : R - 1;
+        const int v = map[(size_t)k_safe * R + r_safe];
+        idx[it][kk] = ok ? v : -1;
+      }
+    }
+  };
+  load_chunk(0);
+
+  for (int kc = 0; kc < K; kc += KC) {
+    const int kn = (K - kc) < KC ? (K - kc) : KC;
+    // A: per-segment hit counts, then compaction into the per-offset lists.
+#pragma unroll
+    for (int it = 0; it < SEG_ITERS; ++it) {
+      const int seg = wave + it * WAVES;
+      if (seg < NSEG) {
+#pragma unroll
+        for (int kk = 0; kk < KC; ++kk) {
+          const unsigned long long b = __ballot(idx[it][kk] >= 0);
+          if (lane == 0) s_cnt[kk][seg] = __popcll(b);
+        }
       }
     }
     __syncthreads();
-    // Phase B: every wave walks all blocks of all offsets for its column slice.
-    for (int kk = 0; kk < kn; ++kk) {
-      const int k = kc + kk;
-      unsigned long long m[NSEG];
-      int cnt = 0;
 #pragma unroll
-      for (int s = 0; s < NSEG; ++s) {
-        m[s] = s_mask[kk][s];
-        cnt += __popcll(m[s]);
-      }
-      if (cnt == 0) continue;
-      vec8 bfr[KB][NB];
+    for (int it = 0; it < SEG_ITERS; ++it) {
+      const int seg = wave + it * WAVES;
+      if (seg < NSEG) {
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
+        for (int kk = 0; kk < KC; ++kk) {
+          const unsigned long long b = __ballot(idx[it][kk] >= 0);
+          if (idx[it][kk] >= 0) {
+            int slot = __popcll(b & lt_mask);
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-          const size_t frag = ((size_t)k * (C / 16) + (col0 / 16 + nb)) * KB + kb;
-          bfr[kb][nb] = *reinterpret_cast<const vec8 *>(packedW + (frag * 64 + lane) * 8);
-        }
-      }
-      for (int b0 = 0; b0 < cnt; b0 += 16) {
-        const int g = b0 + (lane & 15);
-        int row = -1;
-        if (g < cnt) {
-          int base = 0;
-#pragma unroll
-          for (int s = 0; s < NSEG; ++s) {
-            const int c = __popcll(m[s]);
-            if (row < 0 && g < base + c) row = s * 64 + nthSetBit(m[s], g - base);
-            base += c;
+            for (int s = 0; s < NSEG; ++s)
+              if (s < seg) slot += s_cnt[kk][s];
+            s_row[kk][slot] = (uint8_t)(seg * 64 + lane);
+            s_src[kk][slot] = idx[it][kk];
           }
         }
-        int src = -1;
-        if (row >= 0) src = map[(size_t)k * R + r0 + row];
-        vec8 afr[KB];
-        const vec8 zero = {};
+      }
+    }
+    if (wave == 0) {
+      // list lengths -> flat list of blocks (offset-in-chunk << 8 | block number)
+      int tot = 0;
+      if (lane < kn) {
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-          afr[kb] = zero;
-          if (src >= 0)
-            afr[kb] = *reinterpret_cast<const vec8 *>(A + (size_t)src * Q + kb * 32 +
-                                                      (lane >> 4) * 8);
+        for (int s = 0; s < NSEG; ++s) tot += s_cnt[lane][s];
+      }
+      if (lane < KC) s_tot[lane] = tot;
+      const int nb = (tot + 15) >> 4;
+      int incl = nb;
+#pragma unroll
+      for (int off = 1; off < 32; off <<= 1) {
+        const int t = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += t;
+      }
+      const int first = incl - nb;
+      for (int b = 0; b < nb; ++b) s_blk[first + b] = (uint16_t)((lane << 8) | b);
+      if (lane == KC - 1) s_nblk = incl;
+    }
+    __syncthreads();
+    // next chunk's map entries travel while this chunk is multiplied
+    if (kc + KC < K) load_chunk(kc + KC);
+
+    // B: blocks of 16 entries, D blocks in flight per wave.
+    const int nblk = s_nblk;
+    for (int i0 = 0; i0 < nblk; i0 += D) {
+      int blk_kk[D], blk_left[D];
+      uint32_t blk_rows[D];
+      vec8 afr[D][KB];
+      vec8 bfr[D][KB][NB];
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        blk_kk[d] = -1;
+        if (i0 + d < nblk) {
+          const int e = s_blk[i0 + d];
+          blk_kk[d] = e >> 8;
+          const int b0 = (e & 0xff) << 4;
+          blk_left[d] = s_tot[blk_kk[d]] - b0;  // entries from b0 on (>= 1)
+          const int slot = b0 + (lane & 15);
+          int src = -1;
+          if ((lane & 15) < blk_left[d]) src = s_src[blk_kk[d]][slot];
+          blk_rows[d] = *reinterpret_cast<const uint32_t *>(&s_row[blk_kk[d]][b0 + 4 * (lane >> 4)]);
+          const vec8 zero = {};
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) {
+            afr[d][kb] = zero;
+            if (src >= 0)
+              afr[d][kb] = *reinterpret_cast<const vec8 *>(A + (size_t)src * Q + kb * 32 +
+                                                           (lane >> 4) * 8);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+              const size_t frag =
+                  ((size_t)(kc + blk_kk[d]) * GROUPS + (grp0 + nb)) * KB + kb;
+              bfr[d][kb][nb] = *reinterpret_cast<const vec8 *>(packedW + (frag * 64 + lane) * 8);
+            }
+          }
         }
-        int out_row[4];
+      }
 #pragma unroll
-        for (int v = 0; v < 4; ++v) out_row[v] = __shfl(row, (lane >> 4) * 4 + v, kWave);
+      for (int d = 0; d < D; ++d) {
+        if (blk_kk[d] < 0) continue;
+        float4v acc[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-          float4v acc = {0.f, 0.f, 0.f, 0.f};
+          acc[nb] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int kb = 0; kb < KB; ++kb) acc = E::mfma(afr[kb], bfr[kb][nb], acc);
+          for (int kb = 0; kb < KB; ++kb) acc[nb] = E::mfma(afr[d][kb], bfr[d][kb][nb], acc[nb]);
+        }
+        // lane holds result rows 4*(lane/16)+v (v = 0..3) of the block, column lane%16
+        float *cell[NB][4];
+        float old[NB][4];
 #pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            if (out_row[v] >= 0) s_acc[out_row[v] * C + col0 + nb * 16 + (lane & 15)] += acc[v];
+        for (int v = 0; v < 4; ++v) {
+          const int row = (blk_rows[d] >> (8 * v)) & 0xff;
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            const int grp = (grp0 + nb) ^ (row & (GROUPS - 1));
+            cell[nb][v] = &s_acc[row * C + grp * 16 + (lane & 15)];
           }
+        }
+        const int live = blk_left[d] - 4 * (lane >> 4);  // rows v < live exist
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) old[nb][v] = v < live ? *cell[nb][v] : 0.f;
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb)
+            if (v < live) *cell[nb][v] = old[nb][v] + acc[nb][v];
         }
       }
     }
+    __syncthreads();  // lists are rewritten by the next chunk
   }
-  __syncthreads();
   for (int i = tid; i < TR * C / 8; i += NT) {
     const int r = i / (C / 8);
     const int c8 = (i % (C / 8)) * 8;
     if (r0 + r >= R) break;
+    const int grp = (c8 >> 4) ^ (r & (GROUPS - 1));
+    const float *src_row = &s_acc[r * C + grp * 16 + (c8 & 15)];
     typename E::storage tmp[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) E::store(&tmp[e], s_acc[r * C + c8 + e]);
+    for (int e = 0; e < 8; ++e) E::store(&tmp[e], src_row[e]);
     *reinterpret_cast<uint4 *>(result + (size_t)(r0 + r) * C + c8) =
         *reinterpret_cast<const uint4 *>(tmp);
   }

@@ -31,7 +31,9 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kWave = 64;
-constexpr unsigned long long kEmptySlot = ~0ull;
+constexpr uint32_t kEmptyKey = 0xffffffffu;  // no cell index reaches 2^31
+constexpr int kGroup = 16;                   // offsets resolved together per lane
+constexpr int kMaxInlineOffsets = 128;       // kernel volumes with an in-argument offset table
 constexpr int kWordsPerBlock = 1024;  // bitmap words (64 cells each) per block
 
 struct GeomDev {
@@ -77,20 +79,45 @@ __device__ __forceinline__ int axisOut(int i, int pad, int kk, int dil, int stri
   return o < osize ? o : -1;
 }
 
-__global__ __launch_bounds__(kBlock) void rbFill64(unsigned long long *dst, size_t n,
-                                                   unsigned long long value) {
+__global__ __launch_bounds__(kBlock) void rbFill32(uint32_t *dst, size_t n, uint32_t value) {
+  // 16-byte stores; n is a multiple of 4 and dst is 16-byte aligned (workspace blocks are).
+  uint4 *d4 = reinterpret_cast<uint4 *>(dst);
+  const size_t n4 = n / 4;
   size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-  size_t stride = (size_t)gridDim.x * kBlock;
-  for (; i < n; i += stride) dst[i] = value;
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  const uint4 v = make_uint4(value, value, value, value);
+  for (; i < n4; i += stride) d4[i] = v;
 }
 
-// Inserts every row's linear cell index into the open-addressing table (slot =
-// cell << 32 | row; 64-bit max keeps the highest row for a duplicated cell) and
-// copies indices to out_indices, padding rows beyond L with -1.
+// Kernel offsets (kd, kh, kw) of offset index k.  Small kernel volumes carry a
+// table in the kernel arguments; larger ones are decoded by division.
+struct OffsetTable {
+  uint32_t packed[kMaxInlineOffsets];  // kd | kh << 8 | kw << 16
+};
+
+__device__ __forceinline__ void decodeOffset(const OffsetTable &tab, const GeomDev &g, int k,
+                                             int *kd, int *kh, int *kw) {
+  if (g.K <= kMaxInlineOffsets) {
+    const uint32_t p = tab.packed[k];
+    *kd = p & 0xff;
+    *kh = (p >> 8) & 0xff;
+    *kw = p >> 16;
+  } else {
+    const int hw = g.ks[1] * g.ks[2];
+    *kd = k / hw;
+    const int rem = k - *kd * hw;
+    *kh = rem / g.ks[2];
+    *kw = rem - *kh * g.ks[2];
+  }
+}
+
+// Open-addressing table over linear cell indices: keys[] holds the cell (or
+// kEmptyKey), vals[] the highest row index stored for that cell.  32-bit
+// atomics only: a 64-bit compare-and-swap costs several times more here.
 __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t *indices,
-                                                       bool aligned, unsigned long long *table,
-                                                       uint32_t mask, int32_t *out_indices,
-                                                       int out_rows) {
+                                                       bool aligned, uint32_t *keys,
+                                                       int32_t *vals, uint32_t mask,
+                                                       int32_t *out_indices, int out_rows) {
   int j = blockIdx.x * kBlock + threadIdx.x;
   if (j < g.L) {
     int4 c = loadCoord(indices, j, aligned);
@@ -98,14 +125,13 @@ __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t 
     bool in_range = (unsigned)c.x < (unsigned)g.batch && (unsigned)c.y < (unsigned)g.out[0] &&
                     (unsigned)c.z < (unsigned)g.out[1] && (unsigned)c.w < (unsigned)g.out[2];
     if (in_range) {
-      uint32_t cell = (uint32_t)(((c.x * g.out[0] + c.y) * g.out[1] + c.z) * g.out[2] + c.w);
-      unsigned long long packed = ((unsigned long long)cell << 32) | (uint32_t)j;
+      const uint32_t cell =
+          (uint32_t)(((c.x * g.out[0] + c.y) * g.out[1] + c.z) * g.out[2] + c.w);
       uint32_t slot = hashCell(cell) & mask;
       while (true) {
-        unsigned long long old = atomicCAS(&table[slot], kEmptySlot, packed);
-        if (old == kEmptySlot) break;
-        if ((uint32_t)(old >> 32) == cell) {
-          atomicMax(&table[slot], packed);
+        const uint32_t old = atomicCAS(&keys[slot], kEmptyKey, cell);
+        if (old == kEmptyKey || old == cell) {
+          atomicMax(&vals[slot], j);
           break;
         }
         slot = (slot + 1) & mask;
@@ -116,27 +142,18 @@ __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t 
   }
 }
 
-__device__ __forceinline__ int tableLookup(const unsigned long long *table, uint32_t mask,
-                                           uint32_t cell) {
-  uint32_t slot = hashCell(cell) & mask;
-  while (true) {
-    unsigned long long e = table[slot];
-    if (e == kEmptySlot) return -1;
-    if ((uint32_t)(e >> 32) == cell) return (int)(uint32_t)e;
-    slot = (slot + 1) & mask;
-  }
-}
-
-// One wavefront per 64 consecutive rows.  For every offset: resolve the pair
-// (submanifold: table lookup -> output row; regular: output cell, marked in the
-// bitmap), store it as a candidate at [k][row] and record how many lanes of the
-// wave produced one.
+// One wavefront per 64 consecutive rows, offsets in groups of kGroup so that a
+// lane keeps kGroup independent table probes in flight.  For every offset:
+// resolve the pair (submanifold: table lookup -> output row; regular: output
+// cell, marked in the bitmap), store it as a candidate at [k][row] and record
+// how many lanes of the wave produced one.
 template <bool SUBM>
-__global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, const int32_t *indices,
-                                                       bool aligned,
-                                                       const unsigned long long *table,
+__global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable tab,
+                                                       const int32_t *indices, bool aligned,
+                                                       const uint32_t *keys, const int32_t *vals,
                                                        uint32_t mask, unsigned long long *bitmap,
-                                                       int32_t *cand, int32_t *counts, int n_wave) {
+                                                       int32_t *cand, int32_t *counts,
+                                                       int n_wave) {
   const int j = blockIdx.x * kBlock + threadIdx.x;
   const int lane = threadIdx.x & (kWave - 1);
   const int wt = j >> 6;
@@ -145,29 +162,77 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, const int32_t 
   int4 c = make_int4(-1, 0, 0, 0);
   if (active) c = loadCoord(indices, j, aligned);
   const bool n_ok = active && (unsigned)c.x < (unsigned)g.batch;
-  int k = 0;
-  for (int kd = 0; kd < g.ks[0]; ++kd) {
-    const int od = axisOut(c.y, g.pad[0], kd, g.dil[0], g.stride[0], g.out[0]);
-    for (int kh = 0; kh < g.ks[1]; ++kh) {
-      const int oh = axisOut(c.z, g.pad[1], kh, g.dil[1], g.stride[1], g.out[1]);
-      for (int kw = 0; kw < g.ks[2]; ++kw, ++k) {
+  for (int k0 = 0; k0 < g.K; k0 += kGroup) {
+    uint32_t cell[kGroup];
+    int res[kGroup];
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      cell[u] = kEmptyKey;
+      res[u] = -1;
+      const int k = k0 + u;
+      if (k < g.K) {
+        int kd, kh, kw;
+        decodeOffset(tab, g, k, &kd, &kh, &kw);
+        const int od = axisOut(c.y, g.pad[0], kd, g.dil[0], g.stride[0], g.out[0]);
+        const int oh = axisOut(c.z, g.pad[1], kh, g.dil[1], g.stride[1], g.out[1]);
         const int ow = axisOut(c.w, g.pad[2], kw, g.dil[2], g.stride[2], g.out[2]);
-        int r = -1;
-        if (n_ok && (od | oh | ow) >= 0) {
-          const uint32_t cell =
-              (uint32_t)(((c.x * g.out[0] + od) * g.out[1] + oh) * g.out[2] + ow);
-          if (SUBM) {
-            r = tableLookup(table, mask, cell);
-          } else {
-            r = (int)cell;
-            const unsigned long long bit = 1ull << (cell & 63);
-            unsigned long long *word = bitmap + (cell >> 6);
-            if ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & bit) == 0)
-              atomicOr(word, bit);
+        if (n_ok && (od | oh | ow) >= 0)
+          cell[u] = (uint32_t)(((c.x * g.out[0] + od) * g.out[1] + oh) * g.out[2] + ow);
+      }
+    }
+    if (SUBM) {
+      uint32_t slot[kGroup];
+      uint32_t pending = 0, hit = 0;
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        slot[u] = hashCell(cell[u]) & mask;
+        if (cell[u] != kEmptyKey) pending |= 1u << u;
+      }
+      // Every round issues one load per unresolved probe of the lane, all
+      // independent; the wave leaves when its longest probe sequence ends.
+      while (__any(pending != 0)) {
+        uint32_t key[kGroup];
+#pragma unroll
+        for (int u = 0; u < kGroup; ++u) {
+          key[u] = kEmptyKey;
+          if (pending & (1u << u)) key[u] = keys[slot[u]];
+        }
+#pragma unroll
+        for (int u = 0; u < kGroup; ++u) {
+          if (pending & (1u << u)) {
+            if (key[u] == kEmptyKey) {
+              pending &= ~(1u << u);
+            } else if (key[u] == cell[u]) {
+              pending &= ~(1u << u);
+              hit |= 1u << u;
+            } else {
+              slot[u] = (slot[u] + 1) & mask;
+            }
           }
         }
-        if (active) cand[(size_t)k * g.L + j] = r;
-        const unsigned long long b = __ballot(r >= 0);
+      }
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        if (hit & (1u << u)) res[u] = vals[slot[u]];
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        if (cell[u] != kEmptyKey) {
+          res[u] = (int)cell[u];
+          const unsigned long long bit = 1ull << (cell[u] & 63);
+          unsigned long long *word = bitmap + (cell[u] >> 6);
+          if ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & bit) == 0)
+            atomicOr(word, bit);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      const int k = k0 + u;
+      if (k < g.K) {
+        if (active) cand[(size_t)k * g.L + j] = res[u];
+        const unsigned long long b = __ballot(res[u] >= 0);
         if (lane == 0) counts[(size_t)k * n_wave + wt] = __popcll(b);
       }
     }
@@ -222,23 +287,46 @@ __global__ __launch_bounds__(kBlock) void rbEmitPairs(int L, int K, const int32_
   if (wt >= n_wave) return;
   const bool active = j < L;
   const unsigned long long lt_mask = (1ull << lane) - 1ull;
-  for (int k = 0; k < K; ++k) {
-    int r = active ? cand[(size_t)k * L + j] : -1;
-    if (!SUBM && r >= 0) {
-      const unsigned long long below = bitmap[r >> 6] & ((1ull << (r & 63)) - 1ull);
-      r = (int)(word_rank[r >> 6] + (uint32_t)__popcll(below));
+  for (int k0 = 0; k0 < K; k0 += kGroup) {
+    int r[kGroup], base[kGroup], total[kGroup];
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      const int k = k0 + u;
+      r[u] = -1;
+      base[u] = 0;
+      total[u] = 0;
+      if (k < K) {
+        if (active) r[u] = cand[(size_t)k * L + j];
+        base[u] = wave_offs[(size_t)k * n_wave + wt];
+        total[u] = indice_num[k];
+      }
     }
-    const unsigned long long b = __ballot(r >= 0);
-    int32_t *in_col = pairs + (size_t)k * 2 * L;
-    int32_t *out_col = in_col + L;
-    if (r >= 0) {
-      const int pos = wave_offs[(size_t)k * n_wave + wt] + __popcll(b & lt_mask);
-      in_col[pos] = j;
-      out_col[pos] = r;
+    if (!SUBM) {
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        if (r[u] >= 0) {
+          const unsigned long long below = bitmap[r[u] >> 6] & ((1ull << (r[u] & 63)) - 1ull);
+          r[u] = (int)(word_rank[r[u] >> 6] + (uint32_t)__popcll(below));
+        }
+      }
     }
-    if (active && j >= indice_num[k]) {
-      in_col[j] = -1;
-      out_col[j] = -1;
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      const int k = k0 + u;
+      if (k < K) {
+        const unsigned long long b = __ballot(r[u] >= 0);
+        int32_t *in_col = pairs + (size_t)k * 2 * L;
+        int32_t *out_col = in_col + L;
+        if (r[u] >= 0) {
+          const int pos = base[u] + __popcll(b & lt_mask);
+          in_col[pos] = j;
+          out_col[pos] = r[u];
+        }
+        if (active && j >= total[u]) {
+          in_col[j] = -1;
+          out_col[j] = -1;
+        }
+      }
     }
   }
 }
@@ -335,15 +423,31 @@ __global__ __launch_bounds__(kBlock) void rbRankAndDecode(GeomDev g,
 
 inline size_t alignUp(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
+// Load factor of at most 1/4: an unsuccessful lookup (most of them are) then
+// ends after about 1.4 probes on average.
 inline uint32_t tableCapacity(int L) {
   uint32_t cap = 64;
-  while (cap < 2u * (uint32_t)L) cap <<= 1;
+  while (cap < 4u * (uint32_t)L) cap <<= 1;
   return cap;
+}
+
+OffsetTable makeOffsetTable(const RulebookGeom &g) {
+  OffsetTable t;
+  for (int k = 0; k < kMaxInlineOffsets; ++k) t.packed[k] = 0;
+  if (g.K <= kMaxInlineOffsets) {
+    int k = 0;
+    for (int kd = 0; kd < g.ksize[0]; ++kd)
+      for (int kh = 0; kh < g.ksize[1]; ++kh)
+        for (int kw = 0; kw < g.ksize[2]; ++kw, ++k)
+          t.packed[k] = (uint32_t)kd | ((uint32_t)kh << 8) | ((uint32_t)kw << 16);
+  }
+  return t;
 }
 
 struct Workspace {
   // submanifold
-  unsigned long long *table = nullptr;
+  uint32_t *keys = nullptr;  // keys[table_cap] immediately followed by vals[table_cap]
+  int32_t *vals = nullptr;
   uint32_t table_cap = 0;
   // regular
   unsigned long long *bitmap = nullptr;
@@ -351,6 +455,7 @@ struct Workspace {
   int32_t *block_sum = nullptr;
   int32_t *num_act_out = nullptr;
   size_t n_words = 0;
+  size_t bitmap_fill_words = 0;  // 32-bit words to clear, rounded up to a multiple of 4
   int n_bitmap_blocks = 0;
   // both
   int32_t *cand = nullptr;
@@ -373,12 +478,14 @@ Workspace carve(const RulebookGeom &g, void *base) {
   ws.n_wave = (g.L + kWave - 1) / kWave;
   if (g.sub_m) {
     ws.table_cap = tableCapacity(g.L);
-    ws.table = reinterpret_cast<unsigned long long *>(take((size_t)ws.table_cap * 8));
+    ws.keys = reinterpret_cast<uint32_t *>(take((size_t)ws.table_cap * 8));
+    ws.vals = ws.keys ? reinterpret_cast<int32_t *>(ws.keys + ws.table_cap) : nullptr;
   } else {
     const size_t cells = (size_t)g.batch * g.out_space[0] * g.out_space[1] * g.out_space[2];
     ws.n_words = (cells + 63) / 64;
     ws.n_bitmap_blocks = (int)((ws.n_words + kWordsPerBlock - 1) / kWordsPerBlock);
-    ws.bitmap = reinterpret_cast<unsigned long long *>(take(ws.n_words * 8));
+    ws.bitmap_fill_words = (ws.n_words * 2 + 3) / 4 * 4;
+    ws.bitmap = reinterpret_cast<unsigned long long *>(take(ws.bitmap_fill_words * 4));
     ws.word_rank = reinterpret_cast<uint32_t *>(take(ws.n_words * 4));
     ws.block_sum = reinterpret_cast<int32_t *>(take((size_t)ws.n_bitmap_blocks * 4));
     ws.num_act_out = reinterpret_cast<int32_t *>(take(4));
@@ -428,16 +535,20 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
   const int row_blocks = (rows + kBlock - 1) / kBlock;
   const int l_blocks = (g.L + kBlock - 1) / kBlock;
 
-  lc.begin("rbFill64");
-  rbFill64<<<fillBlocks(ws.table_cap), kBlock, 0, lc.stream>>>(ws.table, ws.table_cap, kEmptySlot);
+  const OffsetTable tab = makeOffsetTable(g);
+  // keys become kEmptyKey and vals -1 with the same all-ones pattern
+  lc.begin("rbFill32");
+  rbFill32<<<fillBlocks((size_t)ws.table_cap / 2), kBlock, 0, lc.stream>>>(
+      ws.keys, (size_t)ws.table_cap * 2, kEmptyKey);
   lc.end();
   lc.begin("rbSubmInsert");
-  rbSubmInsert<<<row_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.table, mask, out_indices,
-                                                  g.out_rows);
+  rbSubmInsert<<<row_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.keys, ws.vals, mask,
+                                                     out_indices, g.out_rows);
   lc.end();
   lc.begin("rbProbeCount");
-  rbProbeCount<true><<<l_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.table, mask, nullptr,
-                                                      ws.cand, ws.counts, ws.n_wave);
+  rbProbeCount<true><<<l_blocks, kBlock, 0, lc.stream>>>(d, tab, indices, al, ws.keys, ws.vals,
+                                                         mask, nullptr, ws.cand, ws.counts,
+                                                         ws.n_wave);
   lc.end();
   lc.begin("rbScanRows");
   rbScanRows<<<g.K, kBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
@@ -459,12 +570,15 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
   const bool al_out = aligned16(out_indices, out_indices);
   const int l_blocks = (g.L + kBlock - 1) / kBlock;
 
-  lc.begin("rbFill64");
-  rbFill64<<<fillBlocks(ws.n_words), kBlock, 0, lc.stream>>>(ws.bitmap, ws.n_words, 0ull);
+  const OffsetTable tab = makeOffsetTable(g);
+  lc.begin("rbFill32");
+  rbFill32<<<fillBlocks(ws.n_words / 2 + 1), kBlock, 0, lc.stream>>>(
+      reinterpret_cast<uint32_t *>(ws.bitmap), ws.bitmap_fill_words, 0u);
   lc.end();
   lc.begin("rbProbeCount");
-  rbProbeCount<false><<<l_blocks, kBlock, 0, lc.stream>>>(d, indices, al_in, nullptr, 0, ws.bitmap,
-                                                       ws.cand, ws.counts, ws.n_wave);
+  rbProbeCount<false><<<l_blocks, kBlock, 0, lc.stream>>>(d, tab, indices, al_in, nullptr,
+                                                          nullptr, 0, ws.bitmap, ws.cand,
+                                                          ws.counts, ws.n_wave);
   lc.end();
   lc.begin("rbScanRows");
   rbScanRows<<<g.K, kBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
