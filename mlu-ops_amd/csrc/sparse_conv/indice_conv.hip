@@ -39,6 +39,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef unsigned short u16;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
 constexpr int kMaxInlineK = 128;
@@ -210,230 +211,297 @@ __global__ __launch_bounds__(256) void packFilterFragments(const typename E::sto
 }
 
 constexpr int mfmaTileRows(int C) {
-  // fp32 accumulator tile of at most 32 KiB: four workgroups share a CU's LDS.
-  return C <= 32 ? 256 : (C <= 64 ? 128 : 64);
+  // fp32 accumulator tile of about 34 KiB
+  return C <= 64 ? 128 : 64;
 }
 constexpr int mfmaColBlocksPerWave(int C) { return C >= 128 ? 2 : 1; }
-constexpr int mfmaBlocksInFlight(int Q, int C) {
-  // Register budget: each block in flight holds Q/32 A fragments and
-  // Q/32 * column-blocks B fragments (4 VGPRs each).
-  return (Q / 32) * (1 + mfmaColBlocksPerWave(C)) <= 4 ? 4 : 2;
-}
+// as many fetching waves as multiplying waves (five-wave workgroups place badly on the CU)
+constexpr int mfmaThreads(int C) { return 128 * (C / 16 / mfmaColBlocksPerWave(C)); }
+// Register budget: two eight-wave workgroups per CU need four waves per SIMD.
+constexpr int mfmaWavesPerSimd(int Q, int C) { return (Q <= 64 && C == 64) ? 4 : 2; }
+constexpr int kOffsetChunk = 28;  // offsets whose pair lists are resident in LDS at once
+constexpr int kBatchBlocks = 4;   // 16-entry blocks multiplied together
+// Gathered rows staged in LDS per round: about 25 KiB, which one wave can hold
+// in registers while they travel (at most 24 16-byte pieces per lane).
+constexpr int mfmaStageRows(int Q) { return Q <= 32 ? 256 : (Q <= 64 ? 192 : 96); }
 
-constexpr int kOffsetChunk = 9;  // offsets whose pair lists are resident in LDS at once
-
-// Workgroup = TR result rows x all C columns; wave w owns columns
-// [w*16*NB, (w+1)*16*NB) of the fp32 accumulator tile in LDS, so no two waves
-// ever touch the same accumulator element and every element sees its
-// contributions in ascending offset order.
+// Workgroup = TR result rows x all C columns, WAVES multiplying waves and one
+// fetching wave.  Multiplying wave w owns columns [w*16*NB, (w+1)*16*NB) of the
+// fp32 accumulator tile in LDS, so no two waves ever touch the same accumulator
+// element and every element sees its contributions in ascending offset order.
 //
 // Per chunk of kOffsetChunk offsets:
-//   A   lanes hold map[k][row] for all offsets of the chunk (loaded while the
-//       previous chunk was being multiplied), ballot which rows have a partner
-//       and compact the (row, partner) entries of every offset into LDS lists;
-//       one wave turns the list lengths into a flat list of 16-entry blocks;
-//   B   every wave walks the block list, several blocks in flight: gather 16
-//       partner rows as the MFMA A operand (zero rows pad a short block),
-//       multiply by its B fragments of W[k], add the 16 x 16*NB result into
-//       the accumulator rows of the entries.
-// The accumulator tile is stored with its 16-column groups XOR-swizzled by the
-// row index so that the four rows a wave updates at once fall into different
-// LDS banks more often than not.
+//   A   multiplying wave w loads map[k][row] for the offsets k = w (mod WAVES)
+//       of the chunk and all rows of the tile, ballots which rows have a
+//       partner and, after the per-offset counts have been exchanged, compacts
+//       one entry per pair (partner row << 8 | result row) into a flat list
+//       ordered by offset.  The list is cut into blocks of up to 16 entries of
+//       one offset, and the block list is padded to a whole batch.
+//   B   the flat list is walked in rounds of STEP entries.  The partner rows of
+//       a round are fetched by the fetching wave alone, with row-contiguous
+//       16-byte loads (fetching them in the MFMA operand's own lane order
+//       touches 16 rows per load and runs at a third of the L1 rate, once per
+//       column wave), and written to the LDS stage between two barriers when
+//       the multiplying waves have finished the round before.  A wave of its
+//       own keeps these loads out of the multiplying waves' in-order load
+//       counter, where waiting for the next W fragments would also wait for
+//       them.  Every multiplying wave reads its operand fragments from the
+//       staged rows, multiplies W[k]^T (16 result columns x Q, fetched one
+//       batch ahead) by the block's rows (Q x 16 pairs), which leaves four
+//       consecutive result columns of one pair in every lane, and adds them to
+//       the accumulator row of that pair with one 16-byte read-modify-write.
+//       Lanes past the end of a short block repeat its first entry and
+//       accumulate into a spare row.
 template <typename E, int Q, int C>
-__global__ __launch_bounds__(64 * (C / 16 / mfmaColBlocksPerWave(C)))
+__global__ __launch_bounds__(mfmaThreads(C)) __attribute__((amdgpu_waves_per_eu(mfmaWavesPerSimd(Q, C), mfmaWavesPerSimd(Q, C))))
 void gatherConvMfma(const typename E::storage *A, const typename E::storage *packedW,
-                    const int32_t *map, int R, int K, OffsetCounts inl,
-                    const int32_t *dev_counts, typename E::storage *result) {
+                    const int32_t *map, int R, int K, typename E::storage *result) {
   typedef typename E::vec8 vec8;
+  typedef typename E::storage S;
   constexpr int NB = mfmaColBlocksPerWave(C);
-  constexpr int WAVES = C / 16 / NB;
-  constexpr int NT = 64 * WAVES;
+  constexpr int WAVES = C / 16 / NB;            // multiplying waves
+  constexpr int NT = mfmaThreads(C);
   constexpr int TR = mfmaTileRows(C);
   constexpr int NSEG = TR / 64;
-  constexpr int SEG_ITERS = (NSEG + WAVES - 1) / WAVES;  // segments a wave scans
   constexpr int KB = Q / 32;
   constexpr int KC = kOffsetChunk;
-  constexpr int D = mfmaBlocksInFlight(Q, C);
-  constexpr int GROUPS = C / 16;  // 16-column groups per accumulator row (power of two)
-  constexpr int MAX_BLOCKS = KC * (TR / 16);
+  constexpr int ALLW = NT / 64;                 // multiplying + fetching waves
+  constexpr int FW = ALLW - WAVES;              // fetching waves
+  constexpr int KPW = (KC + ALLW - 1) / ALLW;   // offsets a wave scans per chunk
+  constexpr int G = kBatchBlocks;
+  constexpr int GROUPS = C / 16;
+  constexpr int MAX_ENT = KC * TR;
+  constexpr int MAX_BLK = KC * (TR / 16) + G;
+  constexpr int ACC_STRIDE = C + 4;             // floats; rows 16 apart fall into distinct banks
+  constexpr int ROW_BYTES = Q * 2;              // one gathered row (2-byte elements)
+  constexpr int STAGE_STRIDE = ROW_BYTES + 16;  // padded: 16 rows x 16 bytes hit 64 distinct banks
+  constexpr int PPR = ROW_BYTES / 16;           // 16-byte pieces per row
+  constexpr int SROWS = mfmaStageRows(Q);
+  constexpr int STEP = SROWS - G * 16;          // a batch starting inside a round ends inside its stage
+  constexpr int PT = SROWS * PPR / (64 * FW);   // pieces per lane of a fetching wave
+  static_assert(SROWS * PPR % (64 * FW) == 0 && PT <= 24, "stage must split evenly over the fetching waves");
+  static_assert(KC <= 64 && MAX_ENT <= 65536 && TR <= 256, "descriptor packing");
 
-  __shared__ float s_acc[TR * C];
-  __shared__ int32_t s_src[KC][TR];
-  __shared__ __attribute__((aligned(4))) uint8_t s_row[KC][TR];
-  __shared__ int s_cnt[KC][NSEG];
-  __shared__ int s_tot[KC];
-  __shared__ uint16_t s_blk[MAX_BLOCKS];
-  __shared__ int s_nblk;
+  __shared__ __attribute__((aligned(16))) float s_acc[(TR + 1) * ACC_STRIDE];
+  __shared__ __attribute__((aligned(16))) char s_stage[SROWS * STAGE_STRIDE];
+  __shared__ uint32_t s_ent[MAX_ENT];   // partner row << 8 | result row in the tile
+  __shared__ uint32_t s_blk[MAX_BLK];   // offset in chunk << 24 | first entry << 8 | entries
+  __shared__ int s_cnt[KC];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool fetcher = wave >= WAVES;
+  const int ftid = tid - 64 * WAVES;            // thread index among the fetching waves
   const int r0 = blockIdx.x * TR;
-  const int grp0 = wave * NB;  // first 16-column group of this wave
   const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
-  for (int i = tid; i < TR * C; i += NT) s_acc[i] = 0.f;
+  for (int i = tid; i < (TR + 1) * ACC_STRIDE; i += NT) s_acc[i] = 0.f;
 
-  // map entries of the chunk being prepared, per segment this wave scans
-  int idx[SEG_ITERS][KC];
-  auto load_chunk = [&](int kc) {
-#pragma unroll
-    for (int it = 0; it < SEG_ITERS; ++it) {
-      const int seg = wave + it * WAVES;
-      const int r = r0 + seg * 64 + lane;
-#pragma unroll
-      for (int kk = 0; kk < KC; ++kk) {
-        // Unconditional loads from clamped addresses keep all of them in flight;
-        // offsets without pairs hold -1 everywhere in the map.
-        const bool ok = seg < NSEG && kc + kk < K && r < R;
-        const int k_safe = kc + kk < K ? kc + kk : K - 1;
-        const int r_safe = (seg < NSEG && r < R) ? r : R - 1;
-        const int v = map[(size_t)k_safe * R + r_safe];
-        idx[it][kk] = ok ? v : -1;
-      }
-    }
-  };
-  load_chunk(0);
+  // per-lane constants of the multiply phase
+  const char *a_bytes = reinterpret_cast<const char *>(A);
+  const char *b_base = reinterpret_cast<const char *>(packedW) +
+                       ((size_t)wave * NB * KB * 64 + lane) * 16;
+  constexpr uint32_t kBytesPerOffset = (uint32_t)GROUPS * KB * 64 * 16;  // packed W[k]
+  const int pair = lane & 15;
+  const int quad = lane >> 4;
+  char *acc_lane = reinterpret_cast<char *>(s_acc) + (wave * 16 * NB + 4 * quad) * 4;
+  const char *stage_lane = s_stage + quad * 16;
 
   for (int kc = 0; kc < K; kc += KC) {
     const int kn = (K - kc) < KC ? (K - kc) : KC;
-    // A: per-segment hit counts, then compaction into the per-offset lists.
+    // A: map entries of this wave's offsets; unconditional loads from clamped
+    // addresses keep all of them in flight (offsets without pairs hold -1).
+    int idx[KPW][NSEG];
 #pragma unroll
-    for (int it = 0; it < SEG_ITERS; ++it) {
-      const int seg = wave + it * WAVES;
-      if (seg < NSEG) {
+    for (int j = 0; j < KPW; ++j) {
+      const int kk = wave + j * ALLW;
+      const int k_safe = kk < kn ? kc + kk : kc;
 #pragma unroll
-        for (int kk = 0; kk < KC; ++kk) {
-          const unsigned long long b = __ballot(idx[it][kk] >= 0);
-          if (lane == 0) s_cnt[kk][seg] = __popcll(b);
-        }
+      for (int seg = 0; seg < NSEG; ++seg) {
+        const int r = r0 + seg * 64 + lane;
+        idx[j][seg] = map[(size_t)k_safe * R + (r < R ? r : R - 1)];
       }
+    }
+    // Pinning the loaded values here keeps the loads above unconditional and all
+    // in flight; selecting on them directly lets the compiler branch around
+    // every single load and wait for it.
+#pragma unroll
+    for (int j = 0; j < KPW; ++j)
+#pragma unroll
+      for (int seg = 0; seg < NSEG; ++seg) asm volatile("" : "+v"(idx[j][seg]));
+#pragma unroll
+    for (int j = 0; j < KPW; ++j) {
+      const int kk = wave + j * ALLW;
+      int c = 0;
+#pragma unroll
+      for (int seg = 0; seg < NSEG; ++seg) {
+        const int r = r0 + seg * 64 + lane;
+        if (!(kk < kn && r < R)) idx[j][seg] = -1;
+        c += __popcll(__ballot(idx[j][seg] >= 0));
+      }
+      if (lane == 0 && kk < KC) s_cnt[kk] = c;
     }
     __syncthreads();
+    // every wave scans the counts: entries and blocks in front of each offset
+    const int cnt = lane < KC ? s_cnt[lane < KC ? lane : 0] : 0;
+    const int nb_mine = (cnt + 15) >> 4;
+    int ent_incl = cnt, blk_incl = nb_mine;
 #pragma unroll
-    for (int it = 0; it < SEG_ITERS; ++it) {
-      const int seg = wave + it * WAVES;
-      if (seg < NSEG) {
-#pragma unroll
-        for (int kk = 0; kk < KC; ++kk) {
-          const unsigned long long b = __ballot(idx[it][kk] >= 0);
-          if (idx[it][kk] >= 0) {
-            int slot = __popcll(b & lt_mask);
-#pragma unroll
-            for (int s = 0; s < NSEG; ++s)
-              if (s < seg) slot += s_cnt[kk][s];
-            s_row[kk][slot] = (uint8_t)(seg * 64 + lane);
-            s_src[kk][slot] = idx[it][kk];
-          }
-        }
+    for (int off = 1; off < 64; off <<= 1) {
+      const int t0 = __shfl_up(ent_incl, off, kWave);
+      const int t1 = __shfl_up(blk_incl, off, kWave);
+      if (lane >= off) {
+        ent_incl += t0;
+        blk_incl += t1;
       }
     }
-    if (wave == 0) {
-      // list lengths -> flat list of blocks (offset-in-chunk << 8 | block number)
-      int tot = 0;
-      if (lane < kn) {
+    const int total = __builtin_amdgcn_readlane(ent_incl, 63);
+    const int nblk = __builtin_amdgcn_readlane(blk_incl, 63);
+    const int nbatch = (nblk + G - 1) / G;
+    const int ent_first = ent_incl - cnt;
 #pragma unroll
-        for (int s = 0; s < NSEG; ++s) tot += s_cnt[lane][s];
-      }
-      if (lane < KC) s_tot[lane] = tot;
-      const int nb = (tot + 15) >> 4;
-      int incl = nb;
+    for (int j = 0; j < KPW; ++j) {
+      const int kk = wave + j * ALLW;
+      int base = __shfl(ent_first, kk & 63, kWave);
 #pragma unroll
-      for (int off = 1; off < 32; off <<= 1) {
-        const int t = __shfl_up(incl, off, kWave);
-        if (lane >= off) incl += t;
+      for (int seg = 0; seg < NSEG; ++seg) {
+        const unsigned long long b = __ballot(idx[j][seg] >= 0);
+        if (idx[j][seg] >= 0)
+          s_ent[base + __popcll(b & lt_mask)] =
+              ((uint32_t)idx[j][seg] << 8) | (uint32_t)(seg * 64 + lane);
+        base += __popcll(b);
       }
-      const int first = incl - nb;
-      for (int b = 0; b < nb; ++b) s_blk[first + b] = (uint16_t)((lane << 8) | b);
-      if (lane == KC - 1) s_nblk = incl;
+    }
+    // lane kk of the wave that scanned offset kk cuts its list into blocks
+    if (lane < KC && (lane % ALLW) == wave) {
+      const int first_blk = blk_incl - nb_mine;
+      for (int b = 0; b < nb_mine; ++b) {
+        const int left = cnt - 16 * b;
+        s_blk[first_blk + b] = ((uint32_t)lane << 24) | ((uint32_t)(ent_first + 16 * b) << 8) |
+                               (uint32_t)(left < 16 ? left : 16);
+      }
+    }
+    if (wave == WAVES && nblk > 0) {
+      // empty blocks that fill the last batch: offset and position of the last entry
+      const int last_k = 63 - __builtin_clzll(__ballot(cnt > 0));
+      if (lane < nbatch * G - nblk)
+        s_blk[nblk + lane] = ((uint32_t)last_k << 24) | ((uint32_t)(total - 1) << 8);
     }
     __syncthreads();
-    // next chunk's map entries travel while this chunk is multiplied
-    if (kc + KC < K) load_chunk(kc + KC);
 
-    // B: blocks of 16 entries, D blocks in flight per wave.
-    const int nblk = s_nblk;
-    for (int i0 = 0; i0 < nblk; i0 += D) {
-      int blk_kk[D], blk_left[D];
-      uint32_t blk_rows[D];
-      vec8 afr[D][KB];
-      vec8 bfr[D][KB][NB];
+    // B: the round a batch belongs to follows from the first entry of its first block
+    const int last_round =
+        nblk > 0 ? (int)((s_blk[(nbatch - 1) * G] >> 8) & 0xffffu) / STEP : 0;
+    if (fetcher) {
+      if (nblk > 0) {
+        for (int round = 0; round <= last_round; ++round) {
+          u32x4 piece[PT];
 #pragma unroll
-      for (int d = 0; d < D; ++d) {
-        blk_kk[d] = -1;
-        if (i0 + d < nblk) {
-          const int e = s_blk[i0 + d];
-          blk_kk[d] = e >> 8;
-          const int b0 = (e & 0xff) << 4;
-          blk_left[d] = s_tot[blk_kk[d]] - b0;  // entries from b0 on (>= 1)
-          const int slot = b0 + (lane & 15);
-          int src = -1;
-          if ((lane & 15) < blk_left[d]) src = s_src[blk_kk[d]][slot];
-          blk_rows[d] = *reinterpret_cast<const uint32_t *>(&s_row[blk_kk[d]][b0 + 4 * (lane >> 4)]);
-          const vec8 zero = {};
-#pragma unroll
-          for (int kb = 0; kb < KB; ++kb) {
-            afr[d][kb] = zero;
-            if (src >= 0)
-              afr[d][kb] = *reinterpret_cast<const vec8 *>(A + (size_t)src * Q + kb * 32 +
-                                                           (lane >> 4) * 8);
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-              const size_t frag =
-                  ((size_t)(kc + blk_kk[d]) * GROUPS + (grp0 + nb)) * KB + kb;
-              bfr[d][kb][nb] = *reinterpret_cast<const vec8 *>(packedW + (frag * 64 + lane) * 8);
-            }
+          for (int i = 0; i < PT; ++i) {
+            const int p = ftid + i * 64 * FW;
+            int ci = round * STEP + p / PPR;
+            ci = ci < total ? ci : total - 1;
+            const uint32_t src = s_ent[ci] >> 8;
+            piece[i] = *reinterpret_cast<const u32x4 *>(a_bytes + (size_t)src * ROW_BYTES +
+                                                        (p % PPR) * 16);
           }
+          if (round > 0) __syncthreads();  // the multiplying waves have left the stage
+#pragma unroll
+          for (int i = 0; i < PT; ++i) {
+            const int p = ftid + i * 64 * FW;
+            *reinterpret_cast<u32x4 *>(&s_stage[(p / PPR) * STAGE_STRIDE + (p % PPR) * 16]) = piece[i];
+          }
+          __syncthreads();
         }
       }
+    } else if (nblk > 0) {
+      vec8 wnext[G][KB][NB];
+      uint32_t dnext[G];
+      auto fetch_batch = [&](int b0) {
+        const uint32_t dv = s_blk[b0 + (lane & (G - 1))];
 #pragma unroll
-      for (int d = 0; d < D; ++d) {
-        if (blk_kk[d] < 0) continue;
-        float4v acc[NB];
+        for (int g = 0; g < G; ++g) {
+          dnext[g] = (uint32_t)__builtin_amdgcn_readlane((int)dv, g);
+          const char *bk = b_base + (size_t)(kc + (int)(dnext[g] >> 24)) * kBytesPerOffset;
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          acc[nb] = float4v{0.f, 0.f, 0.f, 0.f};
+          for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-          for (int kb = 0; kb < KB; ++kb) acc[nb] = E::mfma(afr[d][kb], bfr[d][kb][nb], acc[nb]);
+            for (int nb = 0; nb < NB; ++nb)
+              wnext[g][kb][nb] = *reinterpret_cast<const vec8 *>(bk + (nb * KB + kb) * 1024);
         }
-        // lane holds result rows 4*(lane/16)+v (v = 0..3) of the block, column lane%16
-        float *cell[NB][4];
-        float old[NB][4];
+      };
+      fetch_batch(0);
+      __syncthreads();  // round 0 is staged
+      int round = 0;
+      for (int bt = 0; bt < nbatch; ++bt) {
+        vec8 wcur[G][KB][NB];
+        uint32_t dcur[G];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const int row = (blk_rows[d] >> (8 * v)) & 0xff;
+        for (int g = 0; g < G; ++g) {
+          dcur[g] = dnext[g];
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) wcur[g][kb][nb] = wnext[g][kb][nb];
+        }
+        if (bt + 1 < nbatch) fetch_batch((bt + 1) * G);
+        // the stage moves on when the batch starts past the current round
+        while ((int)((dcur[0] >> 8) & 0xffffu) >= (round + 1) * STEP) {
+          __syncthreads();
+          __syncthreads();
+          ++round;
+        }
+        const int stage_first = round * STEP;
+        vec8 afr[G][KB];
+        int acc_row[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const int first = (int)((dcur[g] >> 8) & 0xffffu);
+          const int n = (int)(dcur[g] & 0xffu);
+          const int e = first + (pair < n ? pair : 0);
+          const uint32_t ent = s_ent[e];
+          acc_row[g] = pair < n ? (int)(ent & 0xffu) : TR;
+          const char *arow = stage_lane + (e - stage_first) * STAGE_STRIDE;
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb)
+            afr[g][kb] = *reinterpret_cast<const vec8 *>(arow + kb * 64);
+        }
+        float4v prod[G][NB];
+#pragma unroll
+        for (int g = 0; g < G; ++g)
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) {
-            const int grp = (grp0 + nb) ^ (row & (GROUPS - 1));
-            cell[nb][v] = &s_acc[row * C + grp * 16 + (lane & 15)];
+            prod[g][nb] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+              prod[g][nb] = E::mfma(wcur[g][kb][nb], afr[g][kb], prod[g][nb]);
+          }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          char *dst = acc_lane + acc_row[g] * (ACC_STRIDE * 4);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            // lane holds result columns 16*nb + 4*quad + (0..3) of its pair
+            float4v old = *reinterpret_cast<float4v *>(dst + nb * 64);
+            old += prod[g][nb];
+            *reinterpret_cast<float4v *>(dst + nb * 64) = old;
           }
         }
-        const int live = blk_left[d] - 4 * (lane >> 4);  // rows v < live exist
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) old[nb][v] = v < live ? *cell[nb][v] : 0.f;
-        }
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb)
-            if (v < live) *cell[nb][v] = old[nb][v] + acc[nb][v];
-        }
       }
+      // rounds the fetching wave staged beyond the last batch cannot exist:
+      // last_round is the round of the last batch
     }
-    __syncthreads();  // lists are rewritten by the next chunk
+    __syncthreads();
   }
   for (int i = tid; i < TR * C / 8; i += NT) {
-    const int r = i / (C / 8);
+    const int rr = i / (C / 8);
     const int c8 = (i % (C / 8)) * 8;
-    if (r0 + r >= R) break;
-    const int grp = (c8 >> 4) ^ (r & (GROUPS - 1));
-    const float *src_row = &s_acc[r * C + grp * 16 + (c8 & 15)];
-    typename E::storage tmp[8];
+    if (r0 + rr >= R) break;
+    S tmp[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) E::store(&tmp[e], src_row[e]);
-    *reinterpret_cast<uint4 *>(result + (size_t)(r0 + r) * C + c8) =
+    for (int e = 0; e < 8; ++e) E::store(&tmp[e], s_acc[rr * ACC_STRIDE + c8 + e]);
+    *reinterpret_cast<uint4 *>(result + (size_t)(r0 + rr) * C + c8) =
         *reinterpret_cast<const uint4 *>(tmp);
   }
 }
@@ -645,40 +713,37 @@ hipError_t prepareCounts(const LaunchCtx &lc, const ConvProblem &p, OffsetCounts
 
 template <typename E, int Q, int C>
 void launchMfmaInstance(const LaunchCtx &lc, const void *A, const void *packed,
-                        const int32_t *map, int R, int K, const OffsetCounts &inl,
-                        const int32_t *dev_counts, void *result) {
-  constexpr int NT = 64 * (C / 16 / mfmaColBlocksPerWave(C));
+                        const int32_t *map, int R, int K, void *result) {
+  constexpr int NT = mfmaThreads(C);
   constexpr int TR = mfmaTileRows(C);
   const int blocks = (R + TR - 1) / TR;
   lc.begin("gatherConvMfma");
   gatherConvMfma<E, Q, C><<<blocks, NT, 0, lc.stream>>>(
       static_cast<const typename E::storage *>(A),
-      static_cast<const typename E::storage *>(packed), map, R, K, inl, dev_counts,
+      static_cast<const typename E::storage *>(packed), map, R, K,
       static_cast<typename E::storage *>(result));
   lc.end();
 }
 
 template <typename E, int Q>
 void launchMfmaByC(const LaunchCtx &lc, int C, const void *A, const void *packed,
-                   const int32_t *map, int R, int K, const OffsetCounts &inl,
-                   const int32_t *dev_counts, void *result) {
+                   const int32_t *map, int R, int K, void *result) {
   switch (C) {
-    case 16: launchMfmaInstance<E, Q, 16>(lc, A, packed, map, R, K, inl, dev_counts, result); break;
-    case 32: launchMfmaInstance<E, Q, 32>(lc, A, packed, map, R, K, inl, dev_counts, result); break;
-    case 64: launchMfmaInstance<E, Q, 64>(lc, A, packed, map, R, K, inl, dev_counts, result); break;
-    case 128: launchMfmaInstance<E, Q, 128>(lc, A, packed, map, R, K, inl, dev_counts, result); break;
+    case 16: launchMfmaInstance<E, Q, 16>(lc, A, packed, map, R, K, result); break;
+    case 32: launchMfmaInstance<E, Q, 32>(lc, A, packed, map, R, K, result); break;
+    case 64: launchMfmaInstance<E, Q, 64>(lc, A, packed, map, R, K, result); break;
+    case 128: launchMfmaInstance<E, Q, 128>(lc, A, packed, map, R, K, result); break;
     default: break;
   }
 }
 
 template <typename E>
 void launchMfma(const LaunchCtx &lc, int Q, int C, const void *A, const void *packed,
-                const int32_t *map, int R, int K, const OffsetCounts &inl,
-                const int32_t *dev_counts, void *result) {
+                const int32_t *map, int R, int K, void *result) {
   switch (Q) {
-    case 32: launchMfmaByC<E, 32>(lc, C, A, packed, map, R, K, inl, dev_counts, result); break;
-    case 64: launchMfmaByC<E, 64>(lc, C, A, packed, map, R, K, inl, dev_counts, result); break;
-    case 128: launchMfmaByC<E, 128>(lc, C, A, packed, map, R, K, inl, dev_counts, result); break;
+    case 32: launchMfmaByC<E, 32>(lc, C, A, packed, map, R, K, result); break;
+    case 64: launchMfmaByC<E, 64>(lc, C, A, packed, map, R, K, result); break;
+    case 128: launchMfmaByC<E, 128>(lc, C, A, packed, map, R, K, result); break;
     default: break;
   }
 }
@@ -699,8 +764,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
           static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K, d.Q, d.C,
           static_cast<S *>(ws.packed));
       lc.end();
-      launchMfma<E>(lc, d.Q, d.C, gathered, ws.packed, ws.map, d.R, p.K, inl, ws.dev_counts,
-                    result);
+      launchMfma<E>(lc, d.Q, d.C, gathered, ws.packed, ws.map, d.R, p.K, result);
     }
     return;
   }
@@ -795,10 +859,12 @@ hipError_t launchGatherConv(const LaunchCtx &lc, const ConvProblem &p, GatherDir
                                             d.src_col, d.R, d.n_src, ws.map);
     lc.end();
   }
-  // The MFMA kernel moves rows with 16-byte accesses.
+  // The MFMA kernel moves rows with 16-byte accesses and packs a partner row
+  // into 24 bits of a list entry.
   const bool ptr_ok =
       ((reinterpret_cast<uintptr_t>(gathered) | reinterpret_cast<uintptr_t>(result)) & 15u) == 0;
-  const bool use_mfma = mfmaShapeOk(p.dtype, d.Q, d.C) && ptr_ok && !forceSimt();
+  const bool use_mfma = mfmaShapeOk(p.dtype, d.Q, d.C) && ptr_ok && d.n_src <= (1 << 24) &&
+                        !forceSimt();
   switch (p.dtype) {
     case ElemType::kHalf:
       launchGatherTyped<HalfElem>(lc, p, d, ws, inl, gathered, filters, use_mfma, result);
