@@ -188,14 +188,28 @@ __global__ __launch_bounds__(256) void gatherConvSimt(const typename E::storage 
 // Filter repacked into 16x16x32 B-operand fragments:
 // packed[(((k*(C/16) + nb)*(Q/32) + kb)*64 + lane)*8 + e]
 //   = B(k, q = kb*32 + 8*(lane/16) + e, c = nb*16 + lane%16).
+// One launch for the two independent preparations of the MFMA path: blocks
+// below fill_blocks set the row map to -1 (16-byte stores), the others repack
+// the filter.
 template <typename E>
-__global__ __launch_bounds__(256) void packFilterFragments(const typename E::storage *W,
-                                                           int64_t sK, int64_t sQ, int64_t sC,
-                                                           int K, int Q, int C,
-                                                           typename E::storage *packed) {
+__global__ __launch_bounds__(256) void fillMapPackFilter(int32_t *map, size_t map_elems,
+                                                         int fill_blocks,
+                                                         const typename E::storage *W, int64_t sK,
+                                                         int64_t sQ, int64_t sC, int K, int Q,
+                                                         int C, typename E::storage *packed) {
+  if ((int)blockIdx.x < fill_blocks) {
+    const size_t quads = map_elems / 4;
+    int4 *dst = reinterpret_cast<int4 *>(map);
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < quads;
+         i += (size_t)fill_blocks * 256)
+      dst[i] = make_int4(-1, -1, -1, -1);
+    if (blockIdx.x == 0 && threadIdx.x < (map_elems & 3)) map[quads * 4 + threadIdx.x] = -1;
+    return;
+  }
+  const int pack_blocks = gridDim.x - fill_blocks;
   const size_t total = (size_t)K * (C / 16) * (Q / 32) * 64;
-  for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < total;
-       t += (size_t)gridDim.x * 256) {
+  for (size_t t = (size_t)(blockIdx.x - fill_blocks) * 256 + threadIdx.x; t < total;
+       t += (size_t)pack_blocks * 256) {
     const int lane = (int)(t & 63);
     size_t rest = t >> 6;
     const int kb = (int)(rest % (Q / 32));
@@ -748,26 +762,44 @@ void launchMfma(const LaunchCtx &lc, int Q, int C, const void *A, const void *pa
   }
 }
 
+void launchScatterRowMap(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d,
+                         const GatherWorkspace &ws, const OffsetCounts &inl, int max_count) {
+  if (max_count <= 0) return;
+  dim3 grid((max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256, p.K);
+  lc.begin("scatterRowMap");
+  scatterRowMap<<<grid, 256, 0, lc.stream>>>(p.indice_pairs, p.L, inl, ws.dev_counts, d.row_col,
+                                          d.src_col, d.R, d.n_src, ws.map);
+  lc.end();
+}
+
 template <typename E>
 void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d,
-                       const GatherWorkspace &ws, const OffsetCounts &inl, const void *gathered,
-                       const FilterView &f, bool use_mfma, void *result) {
+                       const GatherWorkspace &ws, const OffsetCounts &inl, int max_count,
+                       const void *gathered, const FilterView &f, bool use_mfma, void *result) {
   typedef typename E::storage S;
   // B(k, q, c): forward q = ci, c = co; backward data q = co, c = ci.
   const int64_t sQ = d.row_col == 1 ? f.stride_ci : f.stride_co;
   const int64_t sC = d.row_col == 1 ? f.stride_co : f.stride_ci;
+  const size_t map_elems = (size_t)p.K * d.R;
   if (use_mfma) {
     if constexpr (!std::is_same<E, FloatElem>::value) {
       const size_t frags = (size_t)p.K * (d.C / 16) * (d.Q / 32) * 64;
-      lc.begin("packFilterFragments");
-      packFilterFragments<E><<<gridFor(frags), 256, 0, lc.stream>>>(
-          static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K, d.Q, d.C,
-          static_cast<S *>(ws.packed));
+      const int fill_blocks = gridFor(map_elems / 4 + 1, 2048);
+      const int pack_blocks = gridFor(frags, 512);
+      lc.begin("fillMapPackFilter");
+      fillMapPackFilter<E><<<fill_blocks + pack_blocks, 256, 0, lc.stream>>>(
+          ws.map, map_elems, fill_blocks, static_cast<const S *>(f.base), f.stride_k, sQ, sC,
+          p.K, d.Q, d.C, static_cast<S *>(ws.packed));
       lc.end();
+      launchScatterRowMap(lc, p, d, ws, inl, max_count);
       launchMfma<E>(lc, d.Q, d.C, gathered, ws.packed, ws.map, d.R, p.K, result);
     }
     return;
   }
+  lc.begin("fillInt32");
+  fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems, -1);
+  lc.end();
+  launchScatterRowMap(lc, p, d, ws, inl, max_count);
   dim3 grid((d.R + 31) / 32, (d.C + 63) / 64);
   lc.begin("gatherConvSimt");
   gatherConvSimt<E><<<grid, 256, 0, lc.stream>>>(static_cast<const S *>(gathered), d.Q,
@@ -848,17 +880,6 @@ hipError_t launchGatherConv(const LaunchCtx &lc, const ConvProblem &p, GatherDir
   hipError_t err = prepareCounts(lc, p, &inl, ws.dev_counts, &max_count);
   if (err != hipSuccess) return err;
 
-  const size_t map_elems = (size_t)p.K * d.R;
-  lc.begin("fillInt32");
-  fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems, -1);
-  lc.end();
-  if (max_count > 0) {
-    dim3 grid((max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256, p.K);
-    lc.begin("scatterRowMap");
-    scatterRowMap<<<grid, 256, 0, lc.stream>>>(p.indice_pairs, p.L, inl, ws.dev_counts, d.row_col,
-                                            d.src_col, d.R, d.n_src, ws.map);
-    lc.end();
-  }
   // The MFMA kernel moves rows with 16-byte accesses and packs a partner row
   // into 24 bits of a list entry.
   const bool ptr_ok =
@@ -867,13 +888,13 @@ hipError_t launchGatherConv(const LaunchCtx &lc, const ConvProblem &p, GatherDir
                         !forceSimt();
   switch (p.dtype) {
     case ElemType::kHalf:
-      launchGatherTyped<HalfElem>(lc, p, d, ws, inl, gathered, filters, use_mfma, result);
+      launchGatherTyped<HalfElem>(lc, p, d, ws, inl, max_count, gathered, filters, use_mfma, result);
       break;
     case ElemType::kBFloat16:
-      launchGatherTyped<BFloat16Elem>(lc, p, d, ws, inl, gathered, filters, use_mfma, result);
+      launchGatherTyped<BFloat16Elem>(lc, p, d, ws, inl, max_count, gathered, filters, use_mfma, result);
       break;
     case ElemType::kFloat:
-      launchGatherTyped<FloatElem>(lc, p, d, ws, inl, gathered, filters, false, result);
+      launchGatherTyped<FloatElem>(lc, p, d, ws, inl, max_count, gathered, filters, false, result);
       break;
   }
   return hipGetLastError();

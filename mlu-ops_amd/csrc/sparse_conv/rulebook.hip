@@ -32,7 +32,7 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kWave = 64;
 constexpr uint32_t kEmptyKey = 0xffffffffu;  // no cell index reaches 2^31
-constexpr int kGroup = 16;                   // offsets resolved together per lane
+constexpr int kGroup = 8;                    // offsets resolved together per lane
 constexpr int kMaxInlineOffsets = 128;       // kernel volumes with an in-argument offset table
 constexpr int kWordsPerBlock = 1024;  // bitmap words (64 cells each) per block
 
@@ -153,8 +153,11 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
                                                        const uint32_t *keys, const int32_t *vals,
                                                        uint32_t mask, unsigned long long *bitmap,
                                                        int32_t *cand, int32_t *counts,
-                                                       int n_wave) {
+                                                       int n_wave, int k_per_slice) {
   const int j = blockIdx.x * kBlock + threadIdx.x;
+  // blockIdx.y selects a slice of the offsets: more waves in flight than rows alone give
+  const int k_lo = blockIdx.y * k_per_slice;
+  const int k_hi = k_lo + k_per_slice < g.K ? k_lo + k_per_slice : g.K;
   const int lane = threadIdx.x & (kWave - 1);
   const int wt = j >> 6;
   if (wt >= n_wave) return;  // whole wave beyond the last row
@@ -162,7 +165,7 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
   int4 c = make_int4(-1, 0, 0, 0);
   if (active) c = loadCoord(indices, j, aligned);
   const bool n_ok = active && (unsigned)c.x < (unsigned)g.batch;
-  for (int k0 = 0; k0 < g.K; k0 += kGroup) {
+  for (int k0 = k_lo; k0 < k_hi; k0 += kGroup) {
     uint32_t cell[kGroup];
     int res[kGroup];
 #pragma unroll
@@ -170,7 +173,7 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
       cell[u] = kEmptyKey;
       res[u] = -1;
       const int k = k0 + u;
-      if (k < g.K) {
+      if (k < k_hi) {
         int kd, kh, kw;
         decodeOffset(tab, g, k, &kd, &kh, &kw);
         const int od = axisOut(c.y, g.pad[0], kd, g.dil[0], g.stride[0], g.out[0]);
@@ -230,7 +233,7 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
       const int k = k0 + u;
-      if (k < g.K) {
+      if (k < k_hi) {
         if (active) cand[(size_t)k * g.L + j] = res[u];
         const unsigned long long b = __ballot(res[u] >= 0);
         if (lane == 0) counts[(size_t)k * n_wave + wt] = __popcll(b);
@@ -280,14 +283,16 @@ __global__ __launch_bounds__(kBlock) void rbEmitPairs(int L, int K, const int32_
                                                       const int32_t *indice_num,
                                                       const unsigned long long *bitmap,
                                                       const uint32_t *word_rank,
-                                                      int32_t *pairs) {
+                                                      int32_t *pairs, int k_per_slice) {
   const int j = blockIdx.x * kBlock + threadIdx.x;
+  const int k_lo = blockIdx.y * k_per_slice;
+  const int k_hi = k_lo + k_per_slice < K ? k_lo + k_per_slice : K;
   const int lane = threadIdx.x & (kWave - 1);
   const int wt = j >> 6;
   if (wt >= n_wave) return;
   const bool active = j < L;
   const unsigned long long lt_mask = (1ull << lane) - 1ull;
-  for (int k0 = 0; k0 < K; k0 += kGroup) {
+  for (int k0 = k_lo; k0 < k_hi; k0 += kGroup) {
     int r[kGroup], base[kGroup], total[kGroup];
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
@@ -295,7 +300,7 @@ __global__ __launch_bounds__(kBlock) void rbEmitPairs(int L, int K, const int32_
       r[u] = -1;
       base[u] = 0;
       total[u] = 0;
-      if (k < K) {
+      if (k < k_hi) {
         if (active) r[u] = cand[(size_t)k * L + j];
         base[u] = wave_offs[(size_t)k * n_wave + wt];
         total[u] = indice_num[k];
@@ -313,7 +318,7 @@ __global__ __launch_bounds__(kBlock) void rbEmitPairs(int L, int K, const int32_
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
       const int k = k0 + u;
-      if (k < K) {
+      if (k < k_hi) {
         const unsigned long long b = __ballot(r[u] >= 0);
         int32_t *in_col = pairs + (size_t)k * 2 * L;
         int32_t *out_col = in_col + L;
@@ -520,6 +525,15 @@ inline int fillBlocks(size_t n) {
   return (int)(b < 1 ? 1 : (b > 4096 ? 4096 : b));
 }
 
+// Offsets per blockIdx.y slice of the probe and emit kernels: one group of
+// kGroup where the kernel volume allows, at most 16 slices.
+int offsetsPerSlice(int K) {
+  int slices = (K + kGroup - 1) / kGroup;
+  if (slices > 16) slices = 16;
+  if (slices < 1) slices = 1;
+  return (K + slices - 1) / slices;
+}
+
 }  // namespace
 
 size_t rulebookWorkspaceBytes(const RulebookGeom &g) { return carve(g, nullptr).bytes; }
@@ -546,16 +560,19 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
                                                      out_indices, g.out_rows);
   lc.end();
   lc.begin("rbProbeCount");
-  rbProbeCount<true><<<l_blocks, kBlock, 0, lc.stream>>>(d, tab, indices, al, ws.keys, ws.vals,
-                                                         mask, nullptr, ws.cand, ws.counts,
-                                                         ws.n_wave);
+  const int k_per = offsetsPerSlice(g.K);
+  const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
+  rbProbeCount<true><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al, ws.keys, ws.vals,
+                                                           mask, nullptr, ws.cand, ws.counts,
+                                                           ws.n_wave, k_per);
   lc.end();
   lc.begin("rbScanRows");
   rbScanRows<<<g.K, kBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
   lc.end();
   lc.begin("rbEmitPairs");
-  rbEmitPairs<true><<<l_blocks, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
-                                                     indice_num, nullptr, nullptr, indice_pairs);
+  rbEmitPairs<true><<<slice_grid, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
+                                                       indice_num, nullptr, nullptr, indice_pairs,
+                                                       k_per);
   lc.end();
   return hipGetLastError();
 }
@@ -576,9 +593,11 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
       reinterpret_cast<uint32_t *>(ws.bitmap), ws.bitmap_fill_words, 0u);
   lc.end();
   lc.begin("rbProbeCount");
-  rbProbeCount<false><<<l_blocks, kBlock, 0, lc.stream>>>(d, tab, indices, al_in, nullptr,
-                                                          nullptr, 0, ws.bitmap, ws.cand,
-                                                          ws.counts, ws.n_wave);
+  const int k_per = offsetsPerSlice(g.K);
+  const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
+  rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al_in, nullptr,
+                                                            nullptr, 0, ws.bitmap, ws.cand,
+                                                            ws.counts, ws.n_wave, k_per);
   lc.end();
   lc.begin("rbScanRows");
   rbScanRows<<<g.K, kBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
@@ -600,9 +619,9 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                                              g.out_rows);
   lc.end();
   lc.begin("rbEmitPairs");
-  rbEmitPairs<false><<<l_blocks, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
-                                                      indice_num, ws.bitmap, ws.word_rank,
-                                                      indice_pairs);
+  rbEmitPairs<false><<<slice_grid, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
+                                                        indice_num, ws.bitmap, ws.word_rank,
+                                                        indice_pairs, k_per);
   lc.end();
   return hipGetLastError();
 }
