@@ -214,6 +214,17 @@ def cpu_baseline(step, reps=3):
             "rulebook_mvoxels_per_s": step.L / rb / 1e6}
 
 
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary
+    of this workload (counters cannot be read from inside the process), or None."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "pmc_traffic_%s.json" % workload)
+    try:
+        with open(path) as f:
+            return json.load(f)["kernels"][kernel]["total_bytes"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -223,6 +234,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only-step", action="store_true",
                     help="run just warmup + timed steps (for profiler runs)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="with --only-step: also run one 64 MiB device-to-device copy, the known-size "
+                         "kernel that scales the profiler's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the rulebook and the "
@@ -262,6 +276,12 @@ def main():
         "rulebook_ms": rb_ms, "rulebook_ms_min": min(per["get_indice_pairs"]),
     }
     if args.only_step:
+        if args.calibration_copy:
+            src = torch.ones(16 * 1024 * 1024, dtype=torch.float32, device="cuda")
+            dst = torch.empty_like(src)
+            torch.cuda.synchronize()
+            dst.copy_(src)
+            torch.cuda.synchronize()
         print(json.dumps(result))
         return
 
@@ -286,7 +306,8 @@ def main():
         alg_bytes, what = step.forward_bytes(), "forward bytes L*Ci*s + N*Co*s + K*Ci*Co*s + 8P"
     achieved = alg_bytes / (dom_ms * 1e-3) / 1e9
     result["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": dominant,
+                          "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(args.workload, dominant),
+                          "kernel": dominant,
                           "kernel_avg_us": dom_ms * 1e3, "algorithmic_bytes": alg_bytes, "bytes_model": what}
     if "gatherConvMfma" in agg:
         g_ms = agg["gatherConvMfma"][0] / agg["gatherConvMfma"][1]
