@@ -319,6 +319,16 @@ def main():
     # the two backward operators of the same layer, reported beside the metric
     _, per_b = time_ops(torch, [("backward_data", step.backward_data), ("backward_filter", step.backward_filter)],
                         max(args.steps // 4, 5))
+    handle.set_kernel_timing(True)
+    for _ in range(5):
+        step.backward_data()
+        step.backward_filter()
+    agg_b = {}
+    for name, ms in handle.kernel_timings():
+        tot, cnt = agg_b.get(name, (0.0, 0))
+        agg_b[name] = (tot + ms, cnt + 1)
+    handle.set_kernel_timing(False)
+    result["backward_kernels"] = {n: {"avg_us": t / c * 1e3, "launches": c / 5} for n, (t, c) in agg_b.items()}
     result["backward_data_ms"] = median(per_b["backward_data"])
     result["backward_filter_ms"] = median(per_b["backward_filter"])
     result["backward_data_tflops"] = step.conv_flops() / (result["backward_data_ms"] * 1e-3) / 1e12

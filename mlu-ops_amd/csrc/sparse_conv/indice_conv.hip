@@ -622,6 +622,213 @@ __global__ __launch_bounds__(256) void reduceFilterPartials(const float *partial
   }
 }
 
+// ---- MFMA backward filter ----------------------------------------------------------
+// dW[k] = X_k^T . dY_k over the pairs of offset k.  The pairs of every offset
+// are cut into slices of slice_len pairs; one workgroup multiplies one slice of
+// one offset and writes a fp32 Ci x Co partial tile, sliceSum adds the tiles of an
+// offset in slice order (no float atomics, the same bits on every run).
+struct SliceTable {
+  int n[kMaxInlineK];      // pairs of the offset
+  int first[kMaxInlineK];  // partial tiles in front of the offset's first slice
+};
+
+constexpr int kFilterStepPairs = 64;     // pairs multiplied per barrier
+constexpr int kFilterIndexChunk = 1024;  // pair indices resident in LDS at once
+constexpr int kFilterMaxSlices = 768;    // about three workgroups per CU
+
+// Both operands are needed with the pair index running along the MFMA's K
+// dimension, i.e. transposed relative to the row-major tensors: rows are
+// gathered with row-contiguous 16-byte loads and written to LDS transposed
+// ([channel][pair], 2-byte stores), from where an operand fragment (8
+// consecutive pairs of one channel) is one 16-byte read.  Wave w multiplies the
+// 16-row blocks w, w+4, ... of dW[k] against all column blocks.
+template <typename E, int CI, int CO>
+__global__ __launch_bounds__(256) void backwardFilterMfma(
+    const typename E::storage *X, const typename E::storage *dY, const int32_t *pairs, int L,
+    int n_in, int n_out, int K, SliceTable tab, int slice_len, float *partial) {
+  typedef typename E::vec8 vec8;
+  typedef typename E::storage S;
+  constexpr int SP = kFilterStepPairs;
+  constexpr int STRIDE = SP * 2 + 16;     // bytes per channel row: 16 rows hit 64 distinct banks
+  constexpr int XP = SP * CI / 8;         // 16-byte pieces of X per step
+  constexpr int YP = SP * CO / 8;
+  constexpr int XT = XP / 256 > 0 ? XP / 256 : 1;
+  constexpr int YT = YP / 256 > 0 ? YP / 256 : 1;
+  constexpr int CBW = (CI / 16 + 3) / 4;  // row blocks per wave
+  constexpr int COB = CO / 16;
+  static_assert(XP % 256 == 0 || XP < 256, "piece split");
+  static_assert(YP % 256 == 0 || YP < 256, "piece split");
+
+  __shared__ __attribute__((aligned(16))) char s_x[CI * STRIDE];
+  __shared__ __attribute__((aligned(16))) char s_y[CO * STRIDE];
+  __shared__ int s_in[kFilterIndexChunk];
+  __shared__ int s_out[kFilterIndexChunk];
+
+  // blockIdx.x numbers the slices of all offsets; offset = last one starting at or before it
+  int k = K - 1;
+  while (k > 0 && tab.first[k] > (int)blockIdx.x) --k;
+  const int n = tab.n[k];
+  const int p_begin = ((int)blockIdx.x - tab.first[k]) * slice_len;
+  if (p_begin >= n) return;
+  const int p_end = p_begin + slice_len < n ? p_begin + slice_len : n;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int32_t *in_col = pairs + (size_t)k * 2 * L;
+  const int32_t *out_col = in_col + L;
+
+  float4v acc[CBW][COB];
+#pragma unroll
+  for (int a = 0; a < CBW; ++a)
+#pragma unroll
+    for (int b = 0; b < COB; ++b) acc[a][b] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 xr[XT], yr[YT];
+  auto fetch_step = [&](int local) {  // local = first pair of the step within the index chunk
+#pragma unroll
+    for (int i = 0; i < XT; ++i) {
+      const int q = tid + i * 256;
+      xr[i] = u32x4{0u, 0u, 0u, 0u};
+      if (XP >= 256 || q < XP) {
+        const int row = s_in[local + q / (CI / 8)];
+        if (row >= 0)
+          xr[i] = *reinterpret_cast<const u32x4 *>(X + (size_t)row * CI + (q % (CI / 8)) * 8);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < YT; ++i) {
+      const int q = tid + i * 256;
+      yr[i] = u32x4{0u, 0u, 0u, 0u};
+      if (YP >= 256 || q < YP) {
+        const int row = s_out[local + q / (CO / 8)];
+        if (row >= 0)
+          yr[i] = *reinterpret_cast<const u32x4 *>(dY + (size_t)row * CO + (q % (CO / 8)) * 8);
+      }
+    }
+  };
+  auto store_step = [&]() {
+#pragma unroll
+    for (int i = 0; i < XT; ++i) {
+      const int q = tid + i * 256;
+      if (XP >= 256 || q < XP) {
+        const int pr = q / (CI / 8), c0 = (q % (CI / 8)) * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          *reinterpret_cast<u16 *>(&s_x[(c0 + e) * STRIDE + pr * 2]) =
+              (u16)(xr[i][e >> 1] >> ((e & 1) * 16));
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < YT; ++i) {
+      const int q = tid + i * 256;
+      if (YP >= 256 || q < YP) {
+        const int pr = q / (CO / 8), c0 = (q % (CO / 8)) * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          *reinterpret_cast<u16 *>(&s_y[(c0 + e) * STRIDE + pr * 2]) =
+              (u16)(yr[i][e >> 1] >> ((e & 1) * 16));
+      }
+    }
+  };
+
+  for (int c_begin = p_begin; c_begin < p_end; c_begin += kFilterIndexChunk) {
+    const int c_len = p_end - c_begin < kFilterIndexChunk ? p_end - c_begin : kFilterIndexChunk;
+    const int c_pad = (c_len + SP - 1) / SP * SP;
+    __syncthreads();  // the previous chunk's indices are no longer read
+    for (int t = tid; t < c_pad; t += 256) {
+      int i = -1, o = -1;
+      if (t < c_len) {
+        i = in_col[c_begin + t];
+        o = out_col[c_begin + t];
+        if ((unsigned)i >= (unsigned)n_in || (unsigned)o >= (unsigned)n_out) i = o = -1;
+      }
+      s_in[t] = i;
+      s_out[t] = o;
+    }
+    __syncthreads();
+    fetch_step(0);
+    for (int local = 0; local < c_pad; local += SP) {
+      __syncthreads();  // every wave has read the previous step's operands
+      store_step();
+      __syncthreads();
+      if (local + SP < c_pad) fetch_step(local + SP);
+#pragma unroll
+      for (int kb = 0; kb < SP / 32; ++kb) {
+        vec8 bfr[COB];
+#pragma unroll
+        for (int b = 0; b < COB; ++b)
+          bfr[b] = *reinterpret_cast<const vec8 *>(
+              &s_y[(b * 16 + (lane & 15)) * STRIDE + kb * 64 + (lane >> 4) * 16]);
+#pragma unroll
+        for (int a = 0; a < CBW; ++a) {
+          const int cb = wave + a * 4;
+          if (cb < CI / 16) {
+            const vec8 afr = *reinterpret_cast<const vec8 *>(
+                &s_x[(cb * 16 + (lane & 15)) * STRIDE + kb * 64 + (lane >> 4) * 16]);
+#pragma unroll
+            for (int b = 0; b < COB; ++b) acc[a][b] = E::mfma(afr, bfr[b], acc[a][b]);
+          }
+        }
+      }
+    }
+  }
+  // lane holds rows 4*(lane/16)+v, column lane%16 of every 16 x 16 block
+  float *tile = partial + (size_t)blockIdx.x * CI * CO;
+#pragma unroll
+  for (int a = 0; a < CBW; ++a) {
+    const int cb = wave + a * 4;
+    if (cb < CI / 16) {
+#pragma unroll
+      for (int b = 0; b < COB; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          tile[(size_t)(cb * 16 + 4 * (lane >> 4) + v) * CO + b * 16 + (lane & 15)] = acc[a][b][v];
+    }
+  }
+}
+
+// dW[k] = sum of the offset's partial tiles, rounded once.  A block adds 64
+// consecutive elements: wave g of 16 takes the slices g, g+16, ... in eight
+// independent running sums, the sums are combined pairwise in a fixed order,
+// so the result depends on the slice count only, never on timing.
+constexpr int kSliceSumWaves = 16;
+template <typename E>
+__global__ __launch_bounds__(64 * kSliceSumWaves) void sliceSum(const float *partial,
+                                                                SliceTable tab, int slice_len,
+                                                                int tile_elems,
+                                                                typename E::storage *dW) {
+  constexpr int W = kSliceSumWaves;
+  __shared__ float s_part[W][64];
+  const int k = blockIdx.y;
+  const int lane = threadIdx.x & 63;
+  const int g = threadIdx.x >> 6;
+  const int e = blockIdx.x * 64 + lane;
+  const int slices = (tab.n[k] + slice_len - 1) / slice_len;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (e < tile_elems) {
+    const float *src = partial + (size_t)tab.first[k] * tile_elems + e;
+    for (int i0 = g; i0 < slices; i0 += 8 * W) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + W * u;
+        if (i < slices) acc[u] += src[(size_t)i * tile_elems];
+      }
+    }
+  }
+  s_part[g][lane] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+  __syncthreads();
+  if (g == 0 && e < tile_elems) {
+    float t[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) t[i] = s_part[i][lane];
+#pragma unroll
+    for (int span = 1; span < W; span *= 2)
+#pragma unroll
+      for (int i = 0; i < W; i += 2 * span) t[i] += t[i + span];
+    E::store(dW + (size_t)k * tile_elems + e, t[0]);
+  }
+}
+
 // ---- host side -----------------------------------------------------------------------
 
 inline size_t alignUp(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
@@ -816,6 +1023,11 @@ struct FilterGradWorkspace {
   size_t bytes = 0;
 };
 
+bool filterMfmaShapeOk(const ConvProblem &p) {
+  auto ok = [](int c) { return c == 16 || c == 32 || c == 64 || c == 128; };
+  return p.dtype != ElemType::kFloat && ok(p.Ci) && ok(p.Co) && p.K <= kMaxInlineK;
+}
+
 int filterGradSplits(const ConvProblem &p) {
   // Bounded by the tensor shape only, so the workspace query and the launch
   // agree whatever indice_num holds.
@@ -836,10 +1048,74 @@ FilterGradWorkspace carveFilterGrad(const ConvProblem &p, void *base) {
   };
   if (p.K > kMaxInlineK) ws.dev_counts = reinterpret_cast<int32_t *>(take((size_t)p.K * 4));
   ws.splits = filterGradSplits(p);
-  if (ws.splits > 1)
-    ws.partial = reinterpret_cast<float *>(take((size_t)ws.splits * p.K * p.Ci * p.Co * 4));
+  size_t tiles = ws.splits > 1 ? (size_t)ws.splits * p.K : 0;
+  // the MFMA path writes at most kFilterMaxSlices + K partial tiles
+  if (filterMfmaShapeOk(p) && (size_t)kFilterMaxSlices + p.K > tiles)
+    tiles = (size_t)kFilterMaxSlices + p.K;
+  if (tiles > 0) ws.partial = reinterpret_cast<float *>(take(tiles * p.Ci * p.Co * 4));
   ws.bytes = off + kBaseAlign;
   return ws;
+}
+
+template <typename E, int CI, int CO>
+void launchFilterMfmaInstance(const LaunchCtx &lc, const ConvProblem &p, const SliceTable &tab,
+                              int slice_len, int total_slices, float *partial, const void *features,
+                              const void *output_grad, void *filters_grad) {
+  typedef typename E::storage S;
+  lc.begin("backwardFilterMfma");
+  if (total_slices > 0)
+    backwardFilterMfma<E, CI, CO><<<total_slices, 256, 0, lc.stream>>>(
+        static_cast<const S *>(features), static_cast<const S *>(output_grad), p.indice_pairs,
+        p.L, p.L, p.num_out, p.K, tab, slice_len, partial);
+  lc.end();
+  lc.begin("sliceSum");
+  sliceSum<E><<<dim3((CI * CO + 63) / 64, p.K), 64 * kSliceSumWaves, 0, lc.stream>>>(
+      partial, tab, slice_len, CI * CO, static_cast<S *>(filters_grad));
+  lc.end();
+}
+
+template <typename E, int CI>
+void launchFilterMfmaByCo(const LaunchCtx &lc, const ConvProblem &p, const SliceTable &tab,
+                          int slice_len, int total_slices, float *partial, const void *features,
+                          const void *output_grad, void *filters_grad) {
+  switch (p.Co) {
+    case 16: launchFilterMfmaInstance<E, CI, 16>(lc, p, tab, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
+    case 32: launchFilterMfmaInstance<E, CI, 32>(lc, p, tab, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
+    case 64: launchFilterMfmaInstance<E, CI, 64>(lc, p, tab, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
+    case 128: launchFilterMfmaInstance<E, CI, 128>(lc, p, tab, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
+    default: break;
+  }
+}
+
+// Slice length from the real pair count: about kFilterMaxSlices workgroups
+// whatever the density, and never more than kFilterMaxSlices + K partial tiles.
+template <typename E>
+void launchFilterMfma(const LaunchCtx &lc, const ConvProblem &p, const FilterGradWorkspace &ws,
+                      const OffsetCounts &inl, const void *features, const void *output_grad,
+                      void *filters_grad) {
+  if constexpr (!std::is_same<E, FloatElem>::value) {
+    SliceTable tab;
+    long long total = 0;
+    for (int k = 0; k < p.K; ++k) total += inl.n[k];
+    int slice_len = (int)((total + kFilterMaxSlices - 1) / kFilterMaxSlices);
+    slice_len = (slice_len + kFilterStepPairs - 1) / kFilterStepPairs * kFilterStepPairs;
+    if (slice_len < kFilterStepPairs) slice_len = kFilterStepPairs;
+    int first = 0;
+    for (int k = 0; k < kMaxInlineK; ++k) {
+      const int n = k < p.K ? inl.n[k] : 0;
+      const int slices = (n + slice_len - 1) / slice_len;
+      tab.n[k] = n;
+      tab.first[k] = first;
+      first += slices;
+    }
+    switch (p.Ci) {
+      case 16: launchFilterMfmaByCo<E, 16>(lc, p, tab, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
+      case 32: launchFilterMfmaByCo<E, 32>(lc, p, tab, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
+      case 64: launchFilterMfmaByCo<E, 64>(lc, p, tab, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
+      case 128: launchFilterMfmaByCo<E, 128>(lc, p, tab, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
+      default: break;
+    }
+  }
 }
 
 template <typename E>
@@ -847,6 +1123,13 @@ void launchFilterGradTyped(const LaunchCtx &lc, const ConvProblem &p,
                            const FilterGradWorkspace &ws, const OffsetCounts &inl,
                            const void *features, const void *output_grad, void *filters_grad) {
   typedef typename E::storage S;
+  // The MFMA path moves rows with 16-byte loads.
+  const bool ptr_ok = ((reinterpret_cast<uintptr_t>(features) |
+                        reinterpret_cast<uintptr_t>(output_grad)) & 15u) == 0;
+  if (filterMfmaShapeOk(p) && ptr_ok && !forceSimt()) {
+    launchFilterMfma<E>(lc, p, ws, inl, features, output_grad, filters_grad);
+    return;
+  }
   const int tiles = ((p.Ci + 31) / 32) * ((p.Co + 63) / 64);
   dim3 grid(tiles, p.K, ws.splits);
   lc.begin("backwardFilterSimt");
