@@ -111,13 +111,14 @@ __device__ __forceinline__ void decodeOffset(const OffsetTable &tab, const GeomD
   }
 }
 
-// Open-addressing table over linear cell indices: keys[] holds the cell (or
-// kEmptyKey), vals[] the highest row index stored for that cell.  32-bit
-// atomics only: a 64-bit compare-and-swap costs several times more here.
+// Open-addressing table over linear cell indices: slot s holds the cell (or
+// kEmptyKey) in table[2s] and the highest row index stored for that cell in
+// table[2s+1], so a probe is one 8-byte load and an insert touches one line.
+// 32-bit atomics only: a 64-bit compare-and-swap costs several times more here.
 __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t *indices,
-                                                       bool aligned, uint32_t *keys,
-                                                       int32_t *vals, uint32_t mask,
-                                                       int32_t *out_indices, int out_rows) {
+                                                       bool aligned, uint32_t *table,
+                                                       uint32_t mask, int32_t *out_indices,
+                                                       int out_rows) {
   int j = blockIdx.x * kBlock + threadIdx.x;
   if (j < g.L) {
     int4 c = loadCoord(indices, j, aligned);
@@ -129,9 +130,9 @@ __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t 
           (uint32_t)(((c.x * g.out[0] + c.y) * g.out[1] + c.z) * g.out[2] + c.w);
       uint32_t slot = hashCell(cell) & mask;
       while (true) {
-        const uint32_t old = atomicCAS(&keys[slot], kEmptyKey, cell);
+        const uint32_t old = atomicCAS(&table[2 * slot], kEmptyKey, cell);
         if (old == kEmptyKey || old == cell) {
-          atomicMax(&vals[slot], j);
+          atomicMax(reinterpret_cast<int32_t *>(&table[2 * slot + 1]), j);
           break;
         }
         slot = (slot + 1) & mask;
@@ -150,7 +151,7 @@ __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t 
 template <bool SUBM>
 __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable tab,
                                                        const int32_t *indices, bool aligned,
-                                                       const uint32_t *keys, const int32_t *vals,
+                                                       const uint32_t *table,
                                                        uint32_t mask, unsigned long long *bitmap,
                                                        int32_t *cand, int32_t *counts,
                                                        int n_wave, int k_per_slice) {
@@ -198,7 +199,7 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
 #pragma unroll
         for (int u = 0; u < kGroup; ++u) {
           key[u] = kEmptyKey;
-          if (pending & (1u << u)) key[u] = keys[slot[u]];
+          if (pending & (1u << u)) key[u] = table[2 * slot[u]];
         }
 #pragma unroll
         for (int u = 0; u < kGroup; ++u) {
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
       }
 #pragma unroll
       for (int u = 0; u < kGroup; ++u) {
-        if (hit & (1u << u)) res[u] = vals[slot[u]];
+        if (hit & (1u << u)) res[u] = (int)table[2 * slot[u] + 1];
       }
     } else {
 #pragma unroll
@@ -227,6 +228,92 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
           unsigned long long *word = bitmap + (cell[u] >> 6);
           if ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & bit) == 0)
             atomicOr(word, bit);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      const int k = k0 + u;
+      if (k < k_hi) {
+        if (active) cand[(size_t)k * g.L + j] = res[u];
+        const unsigned long long b = __ballot(res[u] >= 0);
+        if (lane == 0) counts[(size_t)k * n_wave + wt] = __popcll(b);
+      }
+    }
+  }
+}
+
+// Submanifold probe for unit strides (the usual case), kernel edges <= 32 and
+// K <= kMaxInlineOffsets.  With stride 1 the output cell of (row, offset) is the
+// row's own padded cell minus a per-offset constant, and whether it lies inside
+// the output space is one bit per axis and kernel position, computed once per
+// row: the per-offset work shrinks to a few integer instructions around the
+// probe itself.
+struct UnitStrideOffsets {
+  uint32_t packed[kMaxInlineOffsets];  // kd | kh << 8 | kw << 16
+  uint32_t delta[kMaxInlineOffsets];   // linear distance from the padded cell
+};
+
+__global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
+    GeomDev g, UnitStrideOffsets tab, const int32_t *indices, bool aligned, const uint2 *table,
+    uint32_t mask, int32_t *cand, int32_t *counts, int n_wave, int k_per_slice) {
+  const int j = blockIdx.x * kBlock + threadIdx.x;
+  const int k_lo = blockIdx.y * k_per_slice;
+  const int k_hi = k_lo + k_per_slice < g.K ? k_lo + k_per_slice : g.K;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wt = j >> 6;
+  if (wt >= n_wave) return;  // whole wave beyond the last row
+  const bool active = j < g.L;
+  int4 c = make_int4(-1, 0, 0, 0);
+  if (active) c = loadCoord(indices, j, aligned);
+  const bool n_ok = active && (unsigned)c.x < (unsigned)g.batch;
+  // bit t of an axis mask: kernel position t lands inside the output space
+  uint32_t ok_d = 0, ok_h = 0, ok_w = 0;
+  for (int t = 0; t < g.ks[0]; ++t)
+    ok_d |= (uint32_t)((unsigned)(c.y + g.pad[0] - t * g.dil[0]) < (unsigned)g.out[0]) << t;
+  for (int t = 0; t < g.ks[1]; ++t)
+    ok_h |= (uint32_t)((unsigned)(c.z + g.pad[1] - t * g.dil[1]) < (unsigned)g.out[1]) << t;
+  for (int t = 0; t < g.ks[2]; ++t)
+    ok_w |= (uint32_t)((unsigned)(c.w + g.pad[2] - t * g.dil[2]) < (unsigned)g.out[2]) << t;
+  if (!n_ok) ok_d = 0;
+  // modulo 2^32; exact for every cell inside the output space
+  const uint32_t padded = (((uint32_t)c.x * g.out[0] + (uint32_t)(c.y + g.pad[0])) * g.out[1] +
+                           (uint32_t)(c.z + g.pad[1])) * g.out[2] + (uint32_t)(c.w + g.pad[2]);
+  for (int k0 = k_lo; k0 < k_hi; k0 += kGroup) {
+    uint32_t cell[kGroup], slot[kGroup];
+    int res[kGroup];
+    uint32_t pending = 0;
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
+      const int k = k0 + u < k_hi ? k0 + u : k_hi - 1;  // clamped: a valid table entry
+      const uint32_t pk = tab.packed[k];
+      const bool ok = k0 + u < k_hi &&
+                      ((ok_d >> (pk & 0xff)) & (ok_h >> ((pk >> 8) & 0xff)) & (ok_w >> (pk >> 16)) & 1u);
+      cell[u] = padded - tab.delta[k];
+      slot[u] = hashCell(cell[u]) & mask;
+      res[u] = -1;
+      if (ok) pending |= 1u << u;
+    }
+    // Every round issues one 8-byte load per unresolved probe of the lane, all
+    // independent; the wave leaves when its longest probe sequence ends.
+    while (__any(pending != 0)) {
+      uint2 kv[kGroup];
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        kv[u] = make_uint2(kEmptyKey, 0u);
+        if (pending & (1u << u)) kv[u] = table[slot[u]];
+      }
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        if (pending & (1u << u)) {
+          if (kv[u].x == cell[u]) {
+            res[u] = (int)kv[u].y;
+            pending &= ~(1u << u);
+          } else if (kv[u].x == kEmptyKey) {
+            pending &= ~(1u << u);
+          } else {
+            slot[u] = (slot[u] + 1) & mask;
+          }
         }
       }
     }
@@ -451,8 +538,7 @@ OffsetTable makeOffsetTable(const RulebookGeom &g) {
 
 struct Workspace {
   // submanifold
-  uint32_t *keys = nullptr;  // keys[table_cap] immediately followed by vals[table_cap]
-  int32_t *vals = nullptr;
+  uint32_t *table = nullptr;  // table_cap slots of (cell, row)
   uint32_t table_cap = 0;
   // regular
   unsigned long long *bitmap = nullptr;
@@ -483,8 +569,7 @@ Workspace carve(const RulebookGeom &g, void *base) {
   ws.n_wave = (g.L + kWave - 1) / kWave;
   if (g.sub_m) {
     ws.table_cap = tableCapacity(g.L);
-    ws.keys = reinterpret_cast<uint32_t *>(take((size_t)ws.table_cap * 8));
-    ws.vals = ws.keys ? reinterpret_cast<int32_t *>(ws.keys + ws.table_cap) : nullptr;
+    ws.table = reinterpret_cast<uint32_t *>(take((size_t)ws.table_cap * 8));
   } else {
     const size_t cells = (size_t)g.batch * g.out_space[0] * g.out_space[1] * g.out_space[2];
     ws.n_words = (cells + 63) / 64;
@@ -549,23 +634,45 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
   const int row_blocks = (rows + kBlock - 1) / kBlock;
   const int l_blocks = (g.L + kBlock - 1) / kBlock;
 
-  const OffsetTable tab = makeOffsetTable(g);
-  // keys become kEmptyKey and vals -1 with the same all-ones pattern
+  // cells become kEmptyKey and rows -1 with the same all-ones pattern
   lc.begin("rbFill32");
   rbFill32<<<fillBlocks((size_t)ws.table_cap / 2), kBlock, 0, lc.stream>>>(
-      ws.keys, (size_t)ws.table_cap * 2, kEmptyKey);
+      ws.table, (size_t)ws.table_cap * 2, kEmptyKey);
   lc.end();
   lc.begin("rbSubmInsert");
-  rbSubmInsert<<<row_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.keys, ws.vals, mask,
-                                                     out_indices, g.out_rows);
+  rbSubmInsert<<<row_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.table, mask, out_indices,
+                                                     g.out_rows);
   lc.end();
-  lc.begin("rbProbeCount");
   const int k_per = offsetsPerSlice(g.K);
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
-  rbProbeCount<true><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al, ws.keys, ws.vals,
-                                                           mask, nullptr, ws.cand, ws.counts,
-                                                           ws.n_wave, k_per);
-  lc.end();
+  const bool unit_stride = g.stride[0] == 1 && g.stride[1] == 1 && g.stride[2] == 1 &&
+                           g.ksize[0] <= 32 && g.ksize[1] <= 32 && g.ksize[2] <= 32 &&
+                           g.K <= kMaxInlineOffsets;
+  if (unit_stride) {
+    UnitStrideOffsets ut;
+    int k = 0;
+    for (int kd = 0; kd < g.ksize[0]; ++kd)
+      for (int kh = 0; kh < g.ksize[1]; ++kh)
+        for (int kw = 0; kw < g.ksize[2]; ++kw, ++k) {
+          ut.packed[k] = (uint32_t)kd | ((uint32_t)kh << 8) | ((uint32_t)kw << 16);
+          ut.delta[k] = ((uint32_t)(kd * g.dilation[0]) * (uint32_t)g.out_space[1] +
+                         (uint32_t)(kh * g.dilation[1])) * (uint32_t)g.out_space[2] +
+                        (uint32_t)(kw * g.dilation[2]);
+        }
+    for (; k < kMaxInlineOffsets; ++k) ut.packed[k] = ut.delta[k] = 0;
+    lc.begin("rbSubmProbeUnitStride");
+    rbSubmProbeUnitStride<<<slice_grid, kBlock, 0, lc.stream>>>(
+        d, ut, indices, al, reinterpret_cast<const uint2 *>(ws.table), mask, ws.cand, ws.counts,
+        ws.n_wave, k_per);
+    lc.end();
+  } else {
+    const OffsetTable tab = makeOffsetTable(g);
+    lc.begin("rbProbeCount");
+    rbProbeCount<true><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al, ws.table, mask,
+                                                             nullptr, ws.cand, ws.counts,
+                                                             ws.n_wave, k_per);
+    lc.end();
+  }
   lc.begin("rbScanRows");
   rbScanRows<<<g.K, kBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
   lc.end();
@@ -595,9 +702,9 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
   lc.begin("rbProbeCount");
   const int k_per = offsetsPerSlice(g.K);
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
-  rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al_in, nullptr,
-                                                            nullptr, 0, ws.bitmap, ws.cand,
-                                                            ws.counts, ws.n_wave, k_per);
+  rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al_in, nullptr, 0,
+                                                            ws.bitmap, ws.cand, ws.counts,
+                                                            ws.n_wave, k_per);
   lc.end();
   lc.begin("rbScanRows");
   rbScanRows<<<g.K, kBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
