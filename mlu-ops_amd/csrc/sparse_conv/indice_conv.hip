@@ -29,6 +29,7 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include "core/wave_scan.h"
 #include "sparse_conv/indice_conv.h"
 
 namespace mluop {
@@ -360,16 +361,8 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
     // every wave scans the counts: entries and blocks in front of each offset
     const int cnt = lane < KC ? s_cnt[lane < KC ? lane : 0] : 0;
     const int nb_mine = (cnt + 15) >> 4;
-    int ent_incl = cnt, blk_incl = nb_mine;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const int t0 = __shfl_up(ent_incl, off, kWave);
-      const int t1 = __shfl_up(blk_incl, off, kWave);
-      if (lane >= off) {
-        ent_incl += t0;
-        blk_incl += t1;
-      }
-    }
+    const int ent_incl = waveInclusiveScan(cnt);
+    const int blk_incl = waveInclusiveScan(nb_mine);
     const int total = __builtin_amdgcn_readlane(ent_incl, 63);
     const int nblk = __builtin_amdgcn_readlane(blk_incl, 63);
     const int nbatch = (nblk + G - 1) / G;

@@ -23,6 +23,7 @@
 
 #include <cstdint>
 
+#include "core/wave_scan.h"
 #include "sparse_conv/rulebook.h"
 
 namespace mluop {
@@ -329,33 +330,45 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
   }
 }
 
-// Exclusive prefix sum over `n` ints per row of `data` (one block per row), the
-// row total goes to totals[row].
-__global__ __launch_bounds__(kBlock) void rbScanRows(int32_t *data, int n, int32_t *totals) {
-  __shared__ int s_wsum[kBlock / kWave];
+// Exclusive prefix sum over `n` ints per row of `data` (one block of 1024
+// threads per row, four consecutive elements per thread and pass), the row
+// total goes to totals[row].
+constexpr int kScanBlock = 1024;
+constexpr int kScanItems = 4;
+__global__ __launch_bounds__(kScanBlock) void rbScanRows(int32_t *data, int n, int32_t *totals) {
+  constexpr int WAVES = kScanBlock / kWave;
+  __shared__ int s_wsum[WAVES];
+  __shared__ int s_total;
   int32_t *row = data + (size_t)blockIdx.x * n;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   int carry = 0;
-  for (int base = 0; base < n; base += kBlock) {
-    const int i = base + threadIdx.x;
-    const int v = i < n ? row[i] : 0;
-    int incl = v;
+  for (int base = 0; base < n; base += kScanBlock * kScanItems) {
+    const int i0 = base + threadIdx.x * kScanItems;
+    int v[kScanItems];
+    int mine = 0;
 #pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      int t = __shfl_up(incl, off, kWave);
-      if (lane >= off) incl += t;
+    for (int e = 0; e < kScanItems; ++e) {
+      v[e] = i0 + e < n ? row[i0 + e] : 0;
+      mine += v[e];
     }
+    const int incl = waveInclusiveScan(mine);
     if (lane == kWave - 1) s_wsum[wave] = incl;
     __syncthreads();
-    int woff = 0, total = 0;
-#pragma unroll
-    for (int w = 0; w < kBlock / kWave; ++w) {
-      if (w < wave) woff += s_wsum[w];
-      total += s_wsum[w];
+    if (wave == 0) {
+      const int w = lane < WAVES ? s_wsum[lane] : 0;
+      const int wi = waveInclusiveScan(w);
+      if (lane < WAVES) s_wsum[lane] = wi - w;
+      if (lane == kWave - 1) s_total = wi;
     }
-    if (i < n) row[i] = carry + woff + incl - v;
-    carry += total;
+    __syncthreads();
+    int run = carry + s_wsum[wave] + incl - mine;
+#pragma unroll
+    for (int e = 0; e < kScanItems; ++e) {
+      if (i0 + e < n) row[i0 + e] = run;
+      run += v[e];
+    }
+    carry += s_total;
     __syncthreads();
   }
   if (threadIdx.x == 0) totals[blockIdx.x] = carry;
@@ -674,7 +687,7 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
     lc.end();
   }
   lc.begin("rbScanRows");
-  rbScanRows<<<g.K, kBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
+  rbScanRows<<<g.K, kScanBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
   lc.end();
   lc.begin("rbEmitPairs");
   rbEmitPairs<true><<<slice_grid, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
@@ -707,14 +720,14 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                                             ws.n_wave, k_per);
   lc.end();
   lc.begin("rbScanRows");
-  rbScanRows<<<g.K, kBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
+  rbScanRows<<<g.K, kScanBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
   lc.end();
   lc.begin("rbBitmapBlockSum");
   rbBitmapBlockSum<<<ws.n_bitmap_blocks, kBlock, 0, lc.stream>>>(ws.bitmap, ws.n_words,
                                                               ws.block_sum);
   lc.end();
   lc.begin("rbScanRows");
-  rbScanRows<<<1, kBlock, 0, lc.stream>>>(ws.block_sum, ws.n_bitmap_blocks, ws.num_act_out);
+  rbScanRows<<<1, kScanBlock, 0, lc.stream>>>(ws.block_sum, ws.n_bitmap_blocks, ws.num_act_out);
   lc.end();
   hipError_t err = hipMemcpyAsync(host_num_act_out, ws.num_act_out, sizeof(int32_t),
                                   hipMemcpyDeviceToHost, lc.stream);
