@@ -1,0 +1,161 @@
+"""PyTorch caller layer over the C API: the call sequence mmcv's sparse-conv ops run against
+mlu-ops (descriptor -> workspace size -> mluOpGetIndicePairs -> num_act_out -> device-to-host
+copy of indice_num -> the three indice-convolution operators), wrapped in an autograd function and
+two modules, `SubMConv3d` and `SparseConv3d`.
+
+A `SparseTensor` carries features [L, C], int32 indices [L, 4] = (n, d, h, w), the spatial shape
+and the batch size, plus a cache of rulebooks keyed by `indice_key`, so that stacked submanifold
+layers with the same key build the rulebook once (the reference design's layer chain,
+docs/design_docs/indice_convolution_forward/indice_convolution_forward.md:229-234).
+
+torch is used for device memory, the stream and the autograd graph only; every number is computed
+by libmluops.so.  Weights are stored [kd, kh, kw, Ci, Co] (LAYOUT_ARRAY), the one layout all three
+operators accept (indice_convolution_backward_filter.cpp:227-242 in the reference)."""
+import math
+
+import torch
+
+from . import (LAYOUT_ARRAY, get_indice_pairs, indice_conv_backward_data, indice_conv_backward_filter,
+               indice_conv_forward, make_handle_on_current_stream, regular_output_space)
+
+_handles = {}
+
+
+def _handle():
+    """One library handle per (device, stream): a handle is used from one stream at a time."""
+    key = (torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream)
+    if key not in _handles:
+        _handles[key] = make_handle_on_current_stream()
+    return _handles[key]
+
+
+class Rulebook:
+    """indice_pairs [K,2,L] (device), indice_num as host ints, out_indices, num_act_out."""
+
+    def __init__(self, pairs, out_indices, indice_num_host, num_act_out, filter_space, sub_m, out_space):
+        self.pairs = pairs
+        self.out_indices = out_indices
+        self.indice_num = indice_num_host
+        self.num_act_out = num_act_out
+        self.filter_space = tuple(filter_space)
+        self.sub_m = sub_m
+        self.out_space = tuple(out_space)
+
+
+class SparseTensor:
+    def __init__(self, features, indices, spatial_shape, batch_size, rulebooks=None):
+        assert indices.dtype == torch.int32 and indices.dim() == 2 and indices.shape[1] == 4
+        assert features.shape[0] == indices.shape[0]
+        self.features = features
+        self.indices = indices.contiguous()
+        self.spatial_shape = tuple(int(s) for s in spatial_shape)
+        self.batch_size = int(batch_size)
+        self.rulebooks = {} if rulebooks is None else rulebooks
+
+    def replace_features(self, features):
+        return SparseTensor(features, self.indices, self.spatial_shape, self.batch_size, self.rulebooks)
+
+    def dense(self):
+        """[N, C, D, H, W] dense tensor (for inspection and tests)."""
+        d, h, w = self.spatial_shape
+        out = torch.zeros((self.batch_size, d, h, w, self.features.shape[1]), dtype=self.features.dtype,
+                          device=self.features.device)
+        i = self.indices.long()
+        out[i[:, 0], i[:, 1], i[:, 2], i[:, 3]] = self.features
+        return out.permute(0, 4, 1, 2, 3).contiguous()
+
+
+class _IndiceConv(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, features, weight, rulebook):
+        handle = _handle()
+        features = features.contiguous()
+        weight = weight.contiguous()
+        out = indice_conv_forward(handle, features, weight, LAYOUT_ARRAY, rulebook.pairs, rulebook.indice_num,
+                                  rulebook.num_act_out, rulebook.sub_m)
+        ctx.save_for_backward(features, weight)
+        ctx.rulebook = rulebook
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        features, weight = ctx.saved_tensors
+        rb = ctx.rulebook
+        handle = _handle()
+        grad_out = grad_out.contiguous()
+        grad_features = grad_weight = None
+        if ctx.needs_input_grad[0]:
+            grad_features = indice_conv_backward_data(handle, grad_out, weight, LAYOUT_ARRAY, rb.pairs,
+                                                      rb.indice_num, rb.sub_m, features.shape[1])
+        if ctx.needs_input_grad[1]:
+            grad_weight = indice_conv_backward_filter(handle, features, grad_out, rb.pairs, rb.indice_num,
+                                                      rb.filter_space, rb.sub_m)
+        return grad_features, grad_weight, None
+
+
+def _triple(v):
+    return [int(v)] * 3 if isinstance(v, int) else [int(x) for x in v]
+
+
+class _ConvBase(torch.nn.Module):
+    def __init__(self, in_channels, out_channels, kernel_size, stride, padding, dilation, sub_m, bias,
+                 indice_key):
+        super().__init__()
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size = _triple(kernel_size)
+        self.stride, self.padding, self.dilation = _triple(stride), _triple(padding), _triple(dilation)
+        self.sub_m = sub_m
+        self.indice_key = indice_key
+        k = self.kernel_size[0] * self.kernel_size[1] * self.kernel_size[2]
+        bound = 1.0 / math.sqrt(k * in_channels)
+        self.weight = torch.nn.Parameter(
+            torch.empty(*self.kernel_size, in_channels, out_channels).uniform_(-bound, bound))
+        self.bias = torch.nn.Parameter(torch.zeros(out_channels)) if bias else None
+
+    def _rulebook(self, x):
+        if self.indice_key is not None and self.indice_key in x.rulebooks:
+            rb = x.rulebooks[self.indice_key]
+            assert rb.filter_space == tuple(self.kernel_size) and rb.sub_m == self.sub_m
+            return rb
+        if self.sub_m:
+            out_space = list(x.spatial_shape)
+        else:
+            out_space = regular_output_space(x.spatial_shape, self.kernel_size, self.padding, self.stride,
+                                             self.dilation)
+        pairs, out_indices, num, n_out = get_indice_pairs(
+            _handle(), x.indices, x.batch_size, x.spatial_shape, self.kernel_size, out_space, self.padding,
+            self.stride, self.dilation, self.sub_m)
+        # the operators take indice_num as host int64: one device-to-host copy per rulebook
+        rb = Rulebook(pairs, out_indices[:n_out], num.cpu().tolist(), n_out, self.kernel_size, self.sub_m,
+                      out_space)
+        if self.indice_key is not None:
+            x.rulebooks[self.indice_key] = rb
+        return rb
+
+    def forward(self, x):
+        rb = self._rulebook(x)
+        feats = _IndiceConv.apply(x.features, self.weight.to(x.features.dtype), rb)
+        if self.bias is not None:
+            feats = feats + self.bias.to(feats.dtype)
+        if self.sub_m:
+            return x.replace_features(feats)
+        return SparseTensor(feats, rb.out_indices.contiguous(), rb.out_space, x.batch_size)
+
+
+class SubMConv3d(_ConvBase):
+    """Submanifold 3-D sparse convolution: outputs live on the input's active cells."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, dilation=1, bias=False, indice_key=None):
+        ks = _triple(kernel_size)
+        dil = _triple(dilation)
+        pad = [d * (k // 2) for k, d in zip(ks, dil)]
+        super().__init__(in_channels, out_channels, ks, 1, pad, dil, True, bias, indice_key)
+
+
+class SparseConv3d(_ConvBase):
+    """Regular (strided / dilated) 3-D sparse convolution: every cell an active input reaches is active."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1, bias=False,
+                 indice_key=None):
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, False, bias,
+                         indice_key)

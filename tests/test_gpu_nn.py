@@ -1,0 +1,102 @@
+"""The PyTorch caller layer (mluop_hip.nn) against dense torch.conv3d + autograd in float64 on the
+CPU: a submanifold layer, a second one sharing its rulebook through `indice_key`, and a strided
+regular layer, forward values and the gradients of features and weights."""
+import numpy as np
+import pytest
+
+from spconv_cases import random_voxels
+
+pytestmark = pytest.mark.gpu
+
+
+def dense_reference(idx, feats, weights, space, batch):
+    """Runs the same three layers densely in float64; returns (out rows at out cells, grads)."""
+    import torch
+    import torch.nn.functional as F
+    D, H, W = space
+    x = torch.tensor(feats, dtype=torch.float64, requires_grad=True)
+    ws = [torch.tensor(w, dtype=torch.float64, requires_grad=True) for w in weights]
+    ii = torch.from_numpy(idx.astype(np.int64))
+    dense = torch.zeros((batch, D, H, W, feats.shape[1]), dtype=torch.float64)
+    dense = dense.index_put((ii[:, 0], ii[:, 1], ii[:, 2], ii[:, 3]), x)
+    mask = torch.zeros((batch, 1, D, H, W), dtype=torch.float64)
+    mask[ii[:, 0], 0, ii[:, 1], ii[:, 2], ii[:, 3]] = 1.0
+    t = dense.permute(0, 4, 1, 2, 3)
+
+    def conv(t, w, stride, pad):
+        return F.conv3d(t, w.permute(4, 3, 0, 1, 2), stride=stride, padding=pad)
+
+    t = conv(t, ws[0], 1, 1) * mask          # submanifold: outputs only on active inputs
+    t = conv(t, ws[1], 1, 1) * mask
+    t = conv(t, ws[2], 2, 1)                 # regular: every reached cell is active
+    reach = conv(mask, torch.ones((3, 3, 3, 1, 1), dtype=torch.float64), 2, 1) > 0
+    return x, ws, t, reach[:, 0]
+
+
+def test_layers_match_dense_autograd(gpu_handle):
+    import torch
+    from mluop_hip import nn as spnn
+    rng = np.random.default_rng(21)
+    batch, space, L, ci, cm, co = 2, (8, 10, 12), 300, 16, 32, 16
+    idx = random_voxels(rng, batch, space, L)
+    feats = rng.standard_normal((L, ci)).astype(np.float32)
+    torch.manual_seed(3)
+    l1 = spnn.SubMConv3d(ci, cm, 3, indice_key="subm1").cuda()
+    l2 = spnn.SubMConv3d(cm, cm, 3, indice_key="subm1").cuda()
+    l3 = spnn.SparseConv3d(cm, co, 3, stride=2, padding=1).cuda()
+    x = torch.from_numpy(feats).cuda().requires_grad_(True)
+    st = spnn.SparseTensor(x, torch.from_numpy(idx).cuda(), space, batch)
+    y1 = l1(st)
+    assert len(st.rulebooks) == 1
+    y2 = l2(y1)
+    assert len(st.rulebooks) == 1 and y2.rulebooks is st.rulebooks   # second layer reused the rulebook
+    y3 = l3(y2)
+    out_idx = y3.indices.cpu().numpy().astype(np.int64)
+    g = rng.standard_normal(tuple(y3.features.shape)).astype(np.float32)
+    (y3.features * torch.from_numpy(g).cuda()).sum().backward()
+    torch.cuda.synchronize()
+
+    weights = [l.weight.detach().cpu().numpy() for l in (l1, l2, l3)]
+    rx, rws, rt, reach = dense_reference(idx, feats, weights, space, batch)
+    # same active output cells, in ascending linear order
+    ref_cells = np.argwhere(reach.numpy())
+    assert np.array_equal(out_idx, ref_cells)
+    oi = torch.from_numpy(out_idx)
+    ref_rows = rt.permute(0, 2, 3, 4, 1)[oi[:, 0], oi[:, 1], oi[:, 2], oi[:, 3]]
+    (ref_rows * torch.from_numpy(g).double()).sum().backward()
+
+    def close(a, b, what):
+        a, b = np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)
+        d1 = np.abs(a - b).sum() / (np.abs(b).sum() + 1e-9)
+        d2 = np.sqrt(((a - b) ** 2).sum() / ((b ** 2).sum() + 1e-9))
+        assert d1 <= 1e-5 and d2 <= 1e-5, "%s diff1=%.3e diff2=%.3e" % (what, d1, d2)
+
+    close(y3.features.detach().cpu().numpy(), ref_rows.detach().numpy(), "forward")
+    close(x.grad.cpu().numpy(), rx.grad.numpy(), "grad features")
+    for layer, rw, name in zip((l1, l2, l3), rws, ("w1", "w2", "w3")):
+        close(layer.weight.grad.cpu().numpy(), rw.grad.numpy(), "grad " + name)
+
+
+def test_half_precision_layer_runs_mfma_path(gpu_handle):
+    """fp16 features through SubMConv3d(64, 64): graded at the fp16 threshold against float64."""
+    import torch
+    from mluop_hip import nn as spnn
+    rng = np.random.default_rng(22)
+    batch, space, L = 1, (10, 12, 12), 700
+    idx = random_voxels(rng, batch, space, L)
+    feats = torch.from_numpy(rng.standard_normal((L, 64)).astype(np.float32)).half()
+    layer = spnn.SubMConv3d(64, 64, 3).cuda()
+    with torch.no_grad():
+        layer.weight.copy_(layer.weight.half().float())
+    st = spnn.SparseTensor(feats.cuda(), torch.from_numpy(idx).cuda(), space, batch)
+    y = layer(st).features.detach().float().cpu().numpy()
+    rb = next(iter([layer._rulebook(st)]))
+    pairs = rb.pairs.cpu().numpy()
+    w = layer.weight.detach().cpu().double().numpy().reshape(27, 64, 64)
+    ref = np.zeros((L, 64))
+    f64 = feats.double().numpy()
+    for k in range(27):
+        n = rb.indice_num[k]
+        np.add.at(ref, pairs[k, 1, :n], f64[pairs[k, 0, :n]] @ w[k])
+    d1 = np.abs(y - ref).sum() / (np.abs(ref).sum() + 1e-9)
+    assert d1 <= 3e-3, d1
