@@ -48,9 +48,13 @@ struct GeomDev {
   int L;
 };
 
+// Home slot of a cell (before masking): the run of 16 cells along W it belongs
+// to is hashed, the position inside the run is kept.  Neighbours along W have
+// neighbouring home slots, so one 12-byte load answers three probes.
 __device__ __forceinline__ uint32_t hashCell(uint32_t key) {
-  uint32_t h = key * 0x9E3779B1u;
-  return h ^ (h >> 15);
+  uint32_t h = (key >> 4) * 0x9E3779B1u;
+  h ^= h >> 15;
+  return (h << 4) | (key & 15u);
 }
 
 __device__ __forceinline__ int4 loadCoord(const int32_t *indices, int j, bool aligned) {
@@ -112,14 +116,13 @@ __device__ __forceinline__ void decodeOffset(const OffsetTable &tab, const GeomD
   }
 }
 
-// Open-addressing table over linear cell indices: slot s holds the cell (or
-// kEmptyKey) in table[2s] and the highest row index stored for that cell in
-// table[2s+1], so a probe is one 8-byte load and an insert touches one line.
-// 32-bit atomics only: a 64-bit compare-and-swap costs several times more here.
+// Open-addressing table over linear cell indices: keys[] holds the cell (or
+// kEmptyKey), vals[] the highest row index stored for that cell.  32-bit
+// atomics only: a 64-bit compare-and-swap costs several times more here.
 __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t *indices,
-                                                       bool aligned, uint32_t *table,
-                                                       uint32_t mask, int32_t *out_indices,
-                                                       int out_rows) {
+                                                       bool aligned, uint32_t *keys,
+                                                       int32_t *vals, uint32_t mask,
+                                                       int32_t *out_indices, int out_rows) {
   int j = blockIdx.x * kBlock + threadIdx.x;
   if (j < g.L) {
     int4 c = loadCoord(indices, j, aligned);
@@ -131,9 +134,9 @@ __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t 
           (uint32_t)(((c.x * g.out[0] + c.y) * g.out[1] + c.z) * g.out[2] + c.w);
       uint32_t slot = hashCell(cell) & mask;
       while (true) {
-        const uint32_t old = atomicCAS(&table[2 * slot], kEmptyKey, cell);
+        const uint32_t old = atomicCAS(&keys[slot], kEmptyKey, cell);
         if (old == kEmptyKey || old == cell) {
-          atomicMax(reinterpret_cast<int32_t *>(&table[2 * slot + 1]), j);
+          atomicMax(&vals[slot], j);
           break;
         }
         slot = (slot + 1) & mask;
@@ -152,7 +155,7 @@ __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t 
 template <bool SUBM>
 __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable tab,
                                                        const int32_t *indices, bool aligned,
-                                                       const uint32_t *table,
+                                                       const uint32_t *keys, const int32_t *vals,
                                                        uint32_t mask, unsigned long long *bitmap,
                                                        int32_t *cand, int32_t *counts,
                                                        int n_wave, int k_per_slice) {
@@ -200,7 +203,7 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
 #pragma unroll
         for (int u = 0; u < kGroup; ++u) {
           key[u] = kEmptyKey;
-          if (pending & (1u << u)) key[u] = table[2 * slot[u]];
+          if (pending & (1u << u)) key[u] = keys[slot[u]];
         }
 #pragma unroll
         for (int u = 0; u < kGroup; ++u) {
@@ -218,7 +221,7 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
       }
 #pragma unroll
       for (int u = 0; u < kGroup; ++u) {
-        if (hit & (1u << u)) res[u] = (int)table[2 * slot[u] + 1];
+        if (hit & (1u << u)) res[u] = vals[slot[u]];
       }
     } else {
 #pragma unroll
@@ -256,8 +259,9 @@ struct UnitStrideOffsets {
 };
 
 __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
-    GeomDev g, UnitStrideOffsets tab, const int32_t *indices, bool aligned, const uint2 *table,
-    uint32_t mask, int32_t *cand, int32_t *counts, int n_wave, int k_per_slice) {
+    GeomDev g, UnitStrideOffsets tab, const int32_t *indices, bool aligned, const uint32_t *keys,
+    const int32_t *vals, uint32_t mask, int32_t *cand, int32_t *counts, int n_wave,
+    int k_per_slice) {
   const int j = blockIdx.x * kBlock + threadIdx.x;
   const int k_lo = blockIdx.y * k_per_slice;
   const int k_hi = k_lo + k_per_slice < g.K ? k_lo + k_per_slice : g.K;
@@ -283,7 +287,7 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
   for (int k0 = k_lo; k0 < k_hi; k0 += kGroup) {
     uint32_t cell[kGroup], slot[kGroup];
     int res[kGroup];
-    uint32_t pending = 0;
+    uint32_t pending = 0, hit = 0;
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
       const int k = k0 + u < k_hi ? k0 + u : k_hi - 1;  // clamped: a valid table entry
@@ -295,22 +299,22 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
       res[u] = -1;
       if (ok) pending |= 1u << u;
     }
-    // Every round issues one 8-byte load per unresolved probe of the lane, all
+    // Every round issues one load per unresolved probe of the lane, all
     // independent; the wave leaves when its longest probe sequence ends.
     while (__any(pending != 0)) {
-      uint2 kv[kGroup];
+      uint32_t key[kGroup];
 #pragma unroll
       for (int u = 0; u < kGroup; ++u) {
-        kv[u] = make_uint2(kEmptyKey, 0u);
-        if (pending & (1u << u)) kv[u] = table[slot[u]];
+        key[u] = kEmptyKey;
+        if (pending & (1u << u)) key[u] = keys[slot[u]];
       }
 #pragma unroll
       for (int u = 0; u < kGroup; ++u) {
         if (pending & (1u << u)) {
-          if (kv[u].x == cell[u]) {
-            res[u] = (int)kv[u].y;
+          if (key[u] == cell[u]) {
+            hit |= 1u << u;
             pending &= ~(1u << u);
-          } else if (kv[u].x == kEmptyKey) {
+          } else if (key[u] == kEmptyKey) {
             pending &= ~(1u << u);
           } else {
             slot[u] = (slot[u] + 1) & mask;
@@ -320,8 +324,179 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
     }
 #pragma unroll
     for (int u = 0; u < kGroup; ++u) {
+      if (hit & (1u << u)) res[u] = vals[slot[u]];
+    }
+#pragma unroll
+    for (int u = 0; u < kGroup; ++u) {
       const int k = k0 + u;
       if (k < k_hi) {
+        if (active) cand[(size_t)k * g.L + j] = res[u];
+        const unsigned long long b = __ballot(res[u] >= 0);
+        if (lane == 0) counts[(size_t)k * n_wave + wt] = __popcll(b);
+      }
+    }
+  }
+}
+
+// Unit strides with a kernel 3 wide along W at dilation 1 (3x3x3 and its
+// relatives).  The three offsets that differ only in kw look at three
+// consecutive cells; when those lie in one run of 16 their home slots are
+// consecutive, and one load of the eight keys from the first home slot on
+// holds the three home slots plus five more of every probe sequence: walking
+// it (a key equal to the cell is a hit, an empty slot a definite miss) settles
+// nearly every probe of the wave in one memory round trip, where probing slot
+// by slot costs one dependent round trip per step of the longest sequence
+// among the wave's 576 probes.  Sequences that leave the window continue slot
+// by slot.
+constexpr int kWindow = 8;
+constexpr int kWindowB = 4;
+struct KeyWindow {
+  uint32_t k[kWindow];
+};
+struct KeyWindowB {
+  uint32_t k[kWindowB];
+};
+constexpr int kTriples = 3;  // (kd, kh) pairs resolved together per lane
+
+__global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
+    GeomDev g, UnitStrideOffsets tab, const int32_t *indices, bool aligned, const uint32_t *keys,
+    const int32_t *vals, uint32_t mask, int32_t *cand, int32_t *counts, int n_wave,
+    int triples_per_slice) {
+  constexpr int N = kTriples * 3;
+  const int j = blockIdx.x * kBlock + threadIdx.x;
+  const int n_triples = g.K / 3;
+  const int t_lo = blockIdx.y * triples_per_slice;
+  const int t_hi = t_lo + triples_per_slice < n_triples ? t_lo + triples_per_slice : n_triples;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wt = j >> 6;
+  if (wt >= n_wave) return;  // whole wave beyond the last row
+  const bool active = j < g.L;
+  int4 c = make_int4(-1, 0, 0, 0);
+  if (active) c = loadCoord(indices, j, aligned);
+  const bool n_ok = active && (unsigned)c.x < (unsigned)g.batch;
+  uint32_t ok_d = 0, ok_h = 0, ok_w = 0;
+  for (int t = 0; t < g.ks[0]; ++t)
+    ok_d |= (uint32_t)((unsigned)(c.y + g.pad[0] - t * g.dil[0]) < (unsigned)g.out[0]) << t;
+  for (int t = 0; t < g.ks[1]; ++t)
+    ok_h |= (uint32_t)((unsigned)(c.z + g.pad[1] - t * g.dil[1]) < (unsigned)g.out[1]) << t;
+  for (int t = 0; t < 3; ++t)
+    ok_w |= (uint32_t)((unsigned)(c.w + g.pad[2] - t) < (unsigned)g.out[2]) << t;
+  if (!n_ok) ok_d = 0;
+  const uint32_t padded = (((uint32_t)c.x * g.out[0] + (uint32_t)(c.y + g.pad[0])) * g.out[1] +
+                           (uint32_t)(c.z + g.pad[1])) * g.out[2] + (uint32_t)(c.w + g.pad[2]);
+  for (int t0 = t_lo; t0 < t_hi; t0 += kTriples) {
+    uint32_t cell[N], slot[N];
+    int res[N];
+    uint32_t want = 0;
+    uint32_t pending = 0, hit = 0;
+#pragma unroll
+    for (int a = 0; a < kTriples; ++a) {
+      const int t = t0 + a < t_hi ? t0 + a : t_hi - 1;  // clamped: a valid table entry
+      const uint32_t pk = tab.packed[3 * t];
+      const bool ok_t = t0 + a < t_hi && ((ok_d >> (pk & 0xff)) & (ok_h >> ((pk >> 8) & 0xff)) & 1u);
+      const uint32_t c0 = padded - tab.delta[3 * t + 2];  // kw = 2 is the lowest cell
+      const uint32_t r = c0 & 15u;                         // position of c0 in its run
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw) {
+        const int u = 3 * a + kw;
+        cell[u] = c0 + (uint32_t)(2 - kw);
+        res[u] = -1;
+        if (ok_t && ((ok_w >> kw) & 1u)) want |= 1u << u;
+      }
+      // Window A starts at c0's home slot and serves the cells of c0's run;
+      // window B starts at the home slot of the next run's first cell and
+      // serves the one or two cells beyond a run boundary (r = 14, 15).
+      const uint32_t sa = hashCell(c0) & mask;
+      const uint32_t cb = c0 + (16u - r);
+      const uint32_t sb = hashCell(cb) & mask;
+      const uint32_t wa = (want >> (3 * a)) & 7u;  // bit kw; cell c0 + (2 - kw)
+      const uint32_t in_b = r == 15u ? 3u : (r == 14u ? 1u : 0u);  // kw = 0 (and 1) beyond the run
+      const bool load_a = (wa & ~in_b) != 0 && sa + kWindow <= mask + 1u;
+      const bool load_b = (wa & in_b) != 0 && sb + kWindowB <= mask + 1u;
+      KeyWindow win_a;
+      KeyWindowB win_b;
+#pragma unroll
+      for (int i = 0; i < kWindow; ++i) win_a.k[i] = kEmptyKey;
+#pragma unroll
+      for (int i = 0; i < kWindowB; ++i) win_b.k[i] = kEmptyKey;
+      if (load_a) win_a = *reinterpret_cast<const KeyWindow *>(keys + sa);
+      if (load_b) win_b = *reinterpret_cast<const KeyWindowB *>(keys + sb);
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw) {
+        const int u = 3 * a + kw;
+        if (!(want & (1u << u))) continue;
+        const bool beyond = (in_b >> kw) & 1u;
+        const bool loaded = beyond ? load_b : load_a;
+        if (!loaded) {  // window would leave the table: slot by slot from the home slot
+          slot[u] = hashCell(cell[u]) & mask;
+          pending |= 1u << u;
+          continue;
+        }
+        // walk the window from the cell's home slot
+        const uint32_t base = beyond ? sb : sa;
+        const int first = beyond ? (int)(r + 2u - (uint32_t)kw) - 16 : 2 - kw;
+        bool open = true;
+        if (beyond) {
+#pragma unroll
+          for (int i = 0; i < kWindowB; ++i) {
+            const uint32_t key = win_b.k[i];
+            if (open && i >= first && key == cell[u]) {
+              hit |= 1u << u;
+              slot[u] = base + (uint32_t)i;
+              open = false;
+            } else if (open && i >= first && key == kEmptyKey) {
+              open = false;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < kWindow; ++i) {
+            const uint32_t key = win_a.k[i];
+            if (open && i >= first && key == cell[u]) {
+              hit |= 1u << u;
+              slot[u] = base + (uint32_t)i;
+              open = false;
+            } else if (open && i >= first && key == kEmptyKey) {
+              open = false;
+            }
+          }
+        }
+        if (open) {
+          slot[u] = (base + (uint32_t)(beyond ? kWindowB : kWindow)) & mask;
+          pending |= 1u << u;
+        }
+      }
+    }
+    while (__any(pending != 0)) {
+      uint32_t key[N];
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+        key[u] = kEmptyKey;
+        if (pending & (1u << u)) key[u] = keys[slot[u]];
+      }
+#pragma unroll
+      for (int u = 0; u < N; ++u) {
+        if (pending & (1u << u)) {
+          if (key[u] == cell[u]) {
+            hit |= 1u << u;
+            pending &= ~(1u << u);
+          } else if (key[u] == kEmptyKey) {
+            pending &= ~(1u << u);
+          } else {
+            slot[u] = (slot[u] + 1) & mask;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+      if (hit & (1u << u)) res[u] = vals[slot[u]];
+    }
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+      const int t = t0 + u / 3;
+      if (t < t_hi) {
+        const int k = 3 * t + u % 3;
         if (active) cand[(size_t)k * g.L + j] = res[u];
         const unsigned long long b = __ballot(res[u] >= 0);
         if (lane == 0) counts[(size_t)k * n_wave + wt] = __popcll(b);
@@ -528,11 +703,13 @@ __global__ __launch_bounds__(kBlock) void rbRankAndDecode(GeomDev g,
 
 inline size_t alignUp(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
-// Load factor of at most 1/4: an unsuccessful lookup (most of them are) then
-// ends after about 1.4 probes on average.
+// Load factor between 1/16 and 1/8.  Home slots keep runs of cells together, so
+// occupied stretches grow with the load and a probe sequence that leaves the
+// first window costs the whole wave another memory round trip; 8 L measured
+// best against 4 L (longer sequences) and 16 L (more lines to clear and fetch).
 inline uint32_t tableCapacity(int L) {
   uint32_t cap = 64;
-  while (cap < 4u * (uint32_t)L) cap <<= 1;
+  while (cap < 8u * (uint32_t)L) cap <<= 1;
   return cap;
 }
 
@@ -551,7 +728,8 @@ OffsetTable makeOffsetTable(const RulebookGeom &g) {
 
 struct Workspace {
   // submanifold
-  uint32_t *table = nullptr;  // table_cap slots of (cell, row)
+  uint32_t *keys = nullptr;  // keys[table_cap] immediately followed by vals[table_cap]
+  int32_t *vals = nullptr;
   uint32_t table_cap = 0;
   // regular
   unsigned long long *bitmap = nullptr;
@@ -582,7 +760,8 @@ Workspace carve(const RulebookGeom &g, void *base) {
   ws.n_wave = (g.L + kWave - 1) / kWave;
   if (g.sub_m) {
     ws.table_cap = tableCapacity(g.L);
-    ws.table = reinterpret_cast<uint32_t *>(take((size_t)ws.table_cap * 8));
+    ws.keys = reinterpret_cast<uint32_t *>(take((size_t)ws.table_cap * 8));
+    ws.vals = ws.keys ? reinterpret_cast<int32_t *>(ws.keys + ws.table_cap) : nullptr;
   } else {
     const size_t cells = (size_t)g.batch * g.out_space[0] * g.out_space[1] * g.out_space[2];
     ws.n_words = (cells + 63) / 64;
@@ -650,11 +829,11 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
   // cells become kEmptyKey and rows -1 with the same all-ones pattern
   lc.begin("rbFill32");
   rbFill32<<<fillBlocks((size_t)ws.table_cap / 2), kBlock, 0, lc.stream>>>(
-      ws.table, (size_t)ws.table_cap * 2, kEmptyKey);
+      ws.keys, (size_t)ws.table_cap * 2, kEmptyKey);
   lc.end();
   lc.begin("rbSubmInsert");
-  rbSubmInsert<<<row_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.table, mask, out_indices,
-                                                     g.out_rows);
+  rbSubmInsert<<<row_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.keys, ws.vals, mask,
+                                                     out_indices, g.out_rows);
   lc.end();
   const int k_per = offsetsPerSlice(g.K);
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
@@ -673,16 +852,24 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
                         (uint32_t)(kw * g.dilation[2]);
         }
     for (; k < kMaxInlineOffsets; ++k) ut.packed[k] = ut.delta[k] = 0;
-    lc.begin("rbSubmProbeUnitStride");
-    rbSubmProbeUnitStride<<<slice_grid, kBlock, 0, lc.stream>>>(
-        d, ut, indices, al, reinterpret_cast<const uint2 *>(ws.table), mask, ws.cand, ws.counts,
-        ws.n_wave, k_per);
-    lc.end();
+    if (g.ksize[2] == 3 && g.dilation[2] == 1) {
+      const int n_triples = g.K / 3;
+      const int t_per = kTriples;
+      lc.begin("rbSubmProbeRuns");
+      rbSubmProbeRuns<<<dim3(l_blocks, (n_triples + t_per - 1) / t_per), kBlock, 0, lc.stream>>>(
+          d, ut, indices, al, ws.keys, ws.vals, mask, ws.cand, ws.counts, ws.n_wave, t_per);
+      lc.end();
+    } else {
+      lc.begin("rbSubmProbeUnitStride");
+      rbSubmProbeUnitStride<<<slice_grid, kBlock, 0, lc.stream>>>(
+          d, ut, indices, al, ws.keys, ws.vals, mask, ws.cand, ws.counts, ws.n_wave, k_per);
+      lc.end();
+    }
   } else {
     const OffsetTable tab = makeOffsetTable(g);
     lc.begin("rbProbeCount");
-    rbProbeCount<true><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al, ws.table, mask,
-                                                             nullptr, ws.cand, ws.counts,
+    rbProbeCount<true><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al, ws.keys, ws.vals,
+                                                             mask, nullptr, ws.cand, ws.counts,
                                                              ws.n_wave, k_per);
     lc.end();
   }
@@ -715,9 +902,9 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
   lc.begin("rbProbeCount");
   const int k_per = offsetsPerSlice(g.K);
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
-  rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al_in, nullptr, 0,
-                                                            ws.bitmap, ws.cand, ws.counts,
-                                                            ws.n_wave, k_per);
+  rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al_in, nullptr,
+                                                            nullptr, 0, ws.bitmap, ws.cand,
+                                                            ws.counts, ws.n_wave, k_per);
   lc.end();
   lc.begin("rbScanRows");
   rbScanRows<<<g.K, kScanBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
