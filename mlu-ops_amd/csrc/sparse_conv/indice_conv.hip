@@ -56,9 +56,13 @@ __device__ __forceinline__ int offsetCount(const OffsetCounts &inl, const int32_
 
 // ---- element types ---------------------------------------------------------
 
+// MFMA traits: an operand fragment is 16 bytes per lane (vec8: kVec elements),
+// kChunk reduction channels per fragment; kBatch 16-pair blocks are multiplied
+// together (bounded by the registers the W fragments of a batch take).
 struct HalfElem {
   typedef _Float16 storage;
   typedef half8 vec8;
+  static constexpr int kVec = 8, kChunk = 32, kBatch = 4;
   static __device__ __forceinline__ float load(const storage *p) { return (float)*p; }
   static __device__ __forceinline__ void store(storage *p, float v) { *p = (_Float16)v; }
   static __device__ __forceinline__ float4v mfma(vec8 a, vec8 b, float4v c) {
@@ -69,6 +73,7 @@ struct HalfElem {
 struct BFloat16Elem {
   typedef u16 storage;
   typedef bf16x8 vec8;
+  static constexpr int kVec = 8, kChunk = 32, kBatch = 4;
   static __device__ __forceinline__ float load(const storage *p) {
     return __uint_as_float((uint32_t)*p << 16);
   }
@@ -88,8 +93,19 @@ struct BFloat16Elem {
 
 struct FloatElem {
   typedef float storage;
+  typedef float4v vec8;  // four floats: lane (m, kq) holds reduction channels 4*kq + (0..3) of a 16-chunk
+  static constexpr int kVec = 4, kChunk = 16, kBatch = 2;
   static __device__ __forceinline__ float load(const storage *p) { return *p; }
   static __device__ __forceinline__ void store(storage *p, float v) { *p = v; }
+  // Four 16x16x4 steps; step s pairs element s of both fragments, i.e. channel
+  // 4*kq + s in MFMA reduction slot kq: a permutation of the chunk's 16 channels.
+  static __device__ __forceinline__ float4v mfma(vec8 a, vec8 b, float4v c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[0], b[0], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[1], b[1], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[2], b[2], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[3], b[3], c, 0, 0, 0);
+    return c;
+  }
 };
 
 // ---- row map ---------------------------------------------------------------
@@ -186,9 +202,11 @@ __global__ __launch_bounds__(256) void gatherConvSimt(const typename E::storage 
 
 // ---- MFMA gather convolution ---------------------------------------------------
 
-// Filter repacked into 16x16x32 B-operand fragments:
-// packed[(((k*(C/16) + nb)*(Q/32) + kb)*64 + lane)*8 + e]
-//   = B(k, q = kb*32 + 8*(lane/16) + e, c = nb*16 + lane%16).
+// Filter repacked into MFMA operand fragments of 16 bytes per lane (VEC elements,
+// CHUNK reduction channels per fragment; 8 and 32 for the 2-byte types, 4 and 16
+// for float):
+// packed[(((k*(C/16) + nb)*(Q/CHUNK) + kb)*64 + lane)*VEC + e]
+//   = B(k, q = kb*CHUNK + VEC*(lane/16) + e, c = nb*16 + lane%16).
 // One launch for the two independent preparations of the MFMA path: blocks
 // below fill_blocks set the row map to -1 (16-byte stores), the others repack
 // the filter.
@@ -208,20 +226,21 @@ __global__ __launch_bounds__(256) void fillMapPackFilter(int32_t *map, size_t ma
     return;
   }
   const int pack_blocks = gridDim.x - fill_blocks;
-  const size_t total = (size_t)K * (C / 16) * (Q / 32) * 64;
+  constexpr int VEC = E::kVec, CHUNK = E::kChunk;
+  const size_t total = (size_t)K * (C / 16) * (Q / CHUNK) * 64;
   for (size_t t = (size_t)(blockIdx.x - fill_blocks) * 256 + threadIdx.x; t < total;
        t += (size_t)pack_blocks * 256) {
     const int lane = (int)(t & 63);
     size_t rest = t >> 6;
-    const int kb = (int)(rest % (Q / 32));
-    rest /= (Q / 32);
+    const int kb = (int)(rest % (Q / CHUNK));
+    rest /= (Q / CHUNK);
     const int nb = (int)(rest % (C / 16));
     const int k = (int)(rest / (C / 16));
     const int c = nb * 16 + (lane & 15);
-    const int qb = kb * 32 + 8 * (lane >> 4);
+    const int qb = kb * CHUNK + VEC * (lane >> 4);
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
-      packed[t * 8 + e] = W[(size_t)k * sK + (size_t)(qb + e) * sQ + (size_t)c * sC];
+    for (int e = 0; e < VEC; ++e)
+      packed[t * VEC + e] = W[(size_t)k * sK + (size_t)(qb + e) * sQ + (size_t)c * sC];
   }
 }
 
@@ -235,10 +254,11 @@ constexpr int mfmaThreads(int C) { return 128 * (C / 16 / mfmaColBlocksPerWave(C
 // Register budget: two eight-wave workgroups per CU need four waves per SIMD.
 constexpr int mfmaWavesPerSimd(int Q, int C) { return (Q <= 64 && C == 64) ? 4 : 2; }
 constexpr int kOffsetChunk = 28;  // offsets whose pair lists are resident in LDS at once
-constexpr int kBatchBlocks = 4;   // 16-entry blocks multiplied together
 // Gathered rows staged in LDS per round: about 25 KiB, which one wave can hold
 // in registers while they travel (at most 24 16-byte pieces per lane).
-constexpr int mfmaStageRows(int Q) { return Q <= 32 ? 256 : (Q <= 64 ? 192 : 96); }
+constexpr int mfmaStageRows(int row_bytes) {
+  return row_bytes <= 64 ? 256 : (row_bytes <= 128 ? 192 : 96);
+}
 
 // Workgroup = TR result rows x all C columns, WAVES multiplying waves and one
 // fetching wave.  Multiplying wave w owns columns [w*16*NB, (w+1)*16*NB) of the
@@ -278,20 +298,20 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   constexpr int NT = mfmaThreads(C);
   constexpr int TR = mfmaTileRows(C);
   constexpr int NSEG = TR / 64;
-  constexpr int KB = Q / 32;
+  constexpr int KB = Q / E::kChunk;           // operand fragments per row
   constexpr int KC = kOffsetChunk;
   constexpr int ALLW = NT / 64;                 // multiplying + fetching waves
   constexpr int FW = ALLW - WAVES;              // fetching waves
   constexpr int KPW = (KC + ALLW - 1) / ALLW;   // offsets a wave scans per chunk
-  constexpr int G = kBatchBlocks;
+  constexpr int G = E::kBatch;
   constexpr int GROUPS = C / 16;
   constexpr int MAX_ENT = KC * TR;
   constexpr int MAX_BLK = KC * (TR / 16) + G;
   constexpr int ACC_STRIDE = C + 4;             // floats; rows 16 apart fall into distinct banks
-  constexpr int ROW_BYTES = Q * 2;              // one gathered row (2-byte elements)
+  constexpr int ROW_BYTES = Q * (int)sizeof(S);  // one gathered row
   constexpr int STAGE_STRIDE = ROW_BYTES + 16;  // padded: 16 rows x 16 bytes hit 64 distinct banks
   constexpr int PPR = ROW_BYTES / 16;           // 16-byte pieces per row
-  constexpr int SROWS = mfmaStageRows(Q);
+  constexpr int SROWS = mfmaStageRows(ROW_BYTES);
   constexpr int STEP = SROWS - G * 16;          // a batch starting inside a round ends inside its stage
   constexpr int PT = SROWS * PPR / (64 * FW);   // pieces per lane of a fetching wave
   static_assert(SROWS * PPR % (64 * FW) == 0 && PT <= 24, "stage must split evenly over the fetching waves");
@@ -501,14 +521,15 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
     }
     __syncthreads();
   }
-  for (int i = tid; i < TR * C / 8; i += NT) {
-    const int rr = i / (C / 8);
-    const int c8 = (i % (C / 8)) * 8;
+  constexpr int VALS = 16 / (int)sizeof(S);  // result values per 16-byte store
+  for (int i = tid; i < TR * C / VALS; i += NT) {
+    const int rr = i / (C / VALS);
+    const int c0 = (i % (C / VALS)) * VALS;
     if (r0 + rr >= R) break;
-    S tmp[8];
+    S tmp[VALS];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) E::store(&tmp[e], s_acc[rr * ACC_STRIDE + c8 + e]);
-    *reinterpret_cast<uint4 *>(result + (size_t)(r0 + rr) * C + c8) =
+    for (int e = 0; e < VALS; ++e) E::store(&tmp[e], s_acc[rr * ACC_STRIDE + c0 + e]);
+    *reinterpret_cast<uint4 *>(result + (size_t)(r0 + rr) * C + c0) =
         *reinterpret_cast<const uint4 *>(tmp);
   }
 }
@@ -632,8 +653,8 @@ constexpr int kFilterMaxSlices = 768;    // about three workgroups per CU
 // Both operands are needed with the pair index running along the MFMA's K
 // dimension, i.e. transposed relative to the row-major tensors: rows are
 // gathered with row-contiguous 16-byte loads and written to LDS transposed
-// ([channel][pair], 2-byte stores), from where an operand fragment (8
-// consecutive pairs of one channel) is one 16-byte read.  Wave w multiplies the
+// ([channel][pair], element-sized stores), from where an operand fragment (8
+// consecutive pairs of one channel, 4 for float) is one 16-byte read.  Wave w multiplies the
 // 16-row blocks w, w+4, ... of dW[k] against all column blocks.
 template <typename E, int CI, int CO>
 __global__ __launch_bounds__(256) void backwardFilterMfma(
@@ -642,9 +663,10 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
   typedef typename E::vec8 vec8;
   typedef typename E::storage S;
   constexpr int SP = kFilterStepPairs;
-  constexpr int STRIDE = SP * 2 + 16;     // bytes per channel row: 16 rows hit 64 distinct banks
-  constexpr int XP = SP * CI / 8;         // 16-byte pieces of X per step
-  constexpr int YP = SP * CO / 8;
+  constexpr int EPP = 16 / (int)sizeof(S);          // elements per 16-byte piece
+  constexpr int STRIDE = SP * (int)sizeof(S) + 16;  // bytes per channel row: 16 rows hit 64 distinct banks
+  constexpr int XP = SP * CI / EPP;                 // 16-byte pieces of X per step
+  constexpr int YP = SP * CO / EPP;
   constexpr int XT = XP / 256 > 0 ? XP / 256 : 1;
   constexpr int YT = YP / 256 > 0 ? YP / 256 : 1;
   constexpr int CBW = (CI / 16 + 3) / 4;  // row blocks per wave
@@ -683,9 +705,9 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
       const int q = tid + i * 256;
       xr[i] = u32x4{0u, 0u, 0u, 0u};
       if (XP >= 256 || q < XP) {
-        const int row = s_in[local + q / (CI / 8)];
+        const int row = s_in[local + q / (CI / EPP)];
         if (row >= 0)
-          xr[i] = *reinterpret_cast<const u32x4 *>(X + (size_t)row * CI + (q % (CI / 8)) * 8);
+          xr[i] = *reinterpret_cast<const u32x4 *>(X + (size_t)row * CI + (q % (CI / EPP)) * EPP);
       }
     }
 #pragma unroll
@@ -693,9 +715,9 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
       const int q = tid + i * 256;
       yr[i] = u32x4{0u, 0u, 0u, 0u};
       if (YP >= 256 || q < YP) {
-        const int row = s_out[local + q / (CO / 8)];
+        const int row = s_out[local + q / (CO / EPP)];
         if (row >= 0)
-          yr[i] = *reinterpret_cast<const u32x4 *>(dY + (size_t)row * CO + (q % (CO / 8)) * 8);
+          yr[i] = *reinterpret_cast<const u32x4 *>(dY + (size_t)row * CO + (q % (CO / EPP)) * EPP);
       }
     }
   };
@@ -704,22 +726,30 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
     for (int i = 0; i < XT; ++i) {
       const int q = tid + i * 256;
       if (XP >= 256 || q < XP) {
-        const int pr = q / (CI / 8), c0 = (q % (CI / 8)) * 8;
+        const int pr = q / (CI / EPP), c0 = (q % (CI / EPP)) * EPP;
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          *reinterpret_cast<u16 *>(&s_x[(c0 + e) * STRIDE + pr * 2]) =
-              (u16)(xr[i][e >> 1] >> ((e & 1) * 16));
+        for (int e = 0; e < EPP; ++e) {
+          if constexpr (sizeof(S) == 2)
+            *reinterpret_cast<u16 *>(&s_x[(c0 + e) * STRIDE + pr * 2]) =
+                (u16)(xr[i][e >> 1] >> ((e & 1) * 16));
+          else
+            *reinterpret_cast<uint32_t *>(&s_x[(c0 + e) * STRIDE + pr * 4]) = xr[i][e];
+        }
       }
     }
 #pragma unroll
     for (int i = 0; i < YT; ++i) {
       const int q = tid + i * 256;
       if (YP >= 256 || q < YP) {
-        const int pr = q / (CO / 8), c0 = (q % (CO / 8)) * 8;
+        const int pr = q / (CO / EPP), c0 = (q % (CO / EPP)) * EPP;
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          *reinterpret_cast<u16 *>(&s_y[(c0 + e) * STRIDE + pr * 2]) =
-              (u16)(yr[i][e >> 1] >> ((e & 1) * 16));
+        for (int e = 0; e < EPP; ++e) {
+          if constexpr (sizeof(S) == 2)
+            *reinterpret_cast<u16 *>(&s_y[(c0 + e) * STRIDE + pr * 2]) =
+                (u16)(yr[i][e >> 1] >> ((e & 1) * 16));
+          else
+            *reinterpret_cast<uint32_t *>(&s_y[(c0 + e) * STRIDE + pr * 4]) = yr[i][e];
+        }
       }
     }
   };
@@ -746,7 +776,7 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
       __syncthreads();
       if (local + SP < c_pad) fetch_step(local + SP);
 #pragma unroll
-      for (int kb = 0; kb < SP / 32; ++kb) {
+      for (int kb = 0; kb < SP / E::kChunk; ++kb) {
         vec8 bfr[COB];
 #pragma unroll
         for (int b = 0; b < COB; ++b)
@@ -844,9 +874,11 @@ bool forceSimt() {
   return v != nullptr && v[0] == '1';
 }
 
+// fp16/bf16: 16x16x32 MFMA, reduction channels in {32, 64, 128}; float: 16x16x4 MFMA,
+// reduction channels in {16, 32, 64} (a 512-byte row would leave too little LDS for the stage).
 bool mfmaShapeOk(ElemType t, int Q, int C) {
-  if (t == ElemType::kFloat) return false;
-  const bool q_ok = (Q == 32 || Q == 64 || Q == 128);
+  const bool q_ok = t == ElemType::kFloat ? (Q == 16 || Q == 32 || Q == 64)
+                                          : (Q == 32 || Q == 64 || Q == 128);
   const bool c_ok = (C == 16 || C == 32 || C == 64 || C == 128);
   return q_ok && c_ok;
 }
@@ -954,10 +986,16 @@ void launchMfmaByC(const LaunchCtx &lc, int C, const void *A, const void *packed
 template <typename E>
 void launchMfma(const LaunchCtx &lc, int Q, int C, const void *A, const void *packed,
                 const int32_t *map, int R, int K, void *result) {
+  constexpr bool is_float = std::is_same<E, FloatElem>::value;
   switch (Q) {
+    case 16:
+      if constexpr (is_float) launchMfmaByC<E, 16>(lc, C, A, packed, map, R, K, result);
+      break;
     case 32: launchMfmaByC<E, 32>(lc, C, A, packed, map, R, K, result); break;
     case 64: launchMfmaByC<E, 64>(lc, C, A, packed, map, R, K, result); break;
-    case 128: launchMfmaByC<E, 128>(lc, C, A, packed, map, R, K, result); break;
+    case 128:
+      if constexpr (!is_float) launchMfmaByC<E, 128>(lc, C, A, packed, map, R, K, result);
+      break;
     default: break;
   }
 }
@@ -982,18 +1020,16 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
   const int64_t sC = d.row_col == 1 ? f.stride_co : f.stride_ci;
   const size_t map_elems = (size_t)p.K * d.R;
   if (use_mfma) {
-    if constexpr (!std::is_same<E, FloatElem>::value) {
-      const size_t frags = (size_t)p.K * (d.C / 16) * (d.Q / 32) * 64;
-      const int fill_blocks = gridFor(map_elems / 4 + 1, 2048);
-      const int pack_blocks = gridFor(frags, 512);
-      lc.begin("fillMapPackFilter");
-      fillMapPackFilter<E><<<fill_blocks + pack_blocks, 256, 0, lc.stream>>>(
-          ws.map, map_elems, fill_blocks, static_cast<const S *>(f.base), f.stride_k, sQ, sC,
-          p.K, d.Q, d.C, static_cast<S *>(ws.packed));
-      lc.end();
-      launchScatterRowMap(lc, p, d, ws, inl, max_count);
-      launchMfma<E>(lc, d.Q, d.C, gathered, ws.packed, ws.map, d.R, p.K, result);
-    }
+    const size_t frags = (size_t)p.K * (d.C / 16) * (d.Q / E::kChunk) * 64;
+    const int fill_blocks = gridFor(map_elems / 4 + 1, 2048);
+    const int pack_blocks = gridFor(frags, 512);
+    lc.begin("fillMapPackFilter");
+    fillMapPackFilter<E><<<fill_blocks + pack_blocks, 256, 0, lc.stream>>>(
+        ws.map, map_elems, fill_blocks, static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K,
+        d.Q, d.C, static_cast<S *>(ws.packed));
+    lc.end();
+    launchScatterRowMap(lc, p, d, ws, inl, max_count);
+    launchMfma<E>(lc, d.Q, d.C, gathered, ws.packed, ws.map, d.R, p.K, result);
     return;
   }
   lc.begin("fillInt32");
@@ -1018,7 +1054,7 @@ struct FilterGradWorkspace {
 
 bool filterMfmaShapeOk(const ConvProblem &p) {
   auto ok = [](int c) { return c == 16 || c == 32 || c == 64 || c == 128; };
-  return p.dtype != ElemType::kFloat && ok(p.Ci) && ok(p.Co) && p.K <= kMaxInlineK;
+  return ok(p.Ci) && ok(p.Co) && p.K <= kMaxInlineK;
 }
 
 int filterGradSplits(const ConvProblem &p) {
@@ -1086,7 +1122,7 @@ template <typename E>
 void launchFilterMfma(const LaunchCtx &lc, const ConvProblem &p, const FilterGradWorkspace &ws,
                       const OffsetCounts &inl, const void *features, const void *output_grad,
                       void *filters_grad) {
-  if constexpr (!std::is_same<E, FloatElem>::value) {
+  {
     SliceTable tab;
     long long total = 0;
     for (int k = 0; k < p.K; ++k) total += inl.n[k];
@@ -1170,7 +1206,7 @@ hipError_t launchGatherConv(const LaunchCtx &lc, const ConvProblem &p, GatherDir
       launchGatherTyped<BFloat16Elem>(lc, p, d, ws, inl, max_count, gathered, filters, use_mfma, result);
       break;
     case ElemType::kFloat:
-      launchGatherTyped<FloatElem>(lc, p, d, ws, inl, max_count, gathered, filters, false, result);
+      launchGatherTyped<FloatElem>(lc, p, d, ws, inl, max_count, gathered, filters, use_mfma, result);
       break;
   }
   return hipGetLastError();
