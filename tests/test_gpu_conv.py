@@ -88,6 +88,7 @@ SHAPES = [
     (1, (8, 8, 8), 300, (3, 3, 3), 128, 64, False, (1, 1, 1)),
     (1, (6, 6, 6), 100, (3, 3, 3), 21, 10, True, (1, 1, 1)),   # odd channel counts -> SIMT
     (1, (6, 6, 6), 100, (1, 3, 3), 13, 70, False, (1, 2, 1)),
+    (1, (10, 10, 10), 400, (5, 5, 7), 32, 32, True, (1, 1, 1)),   # K = 175: counts in device memory, seven chunks of offsets
 ]
 
 

@@ -61,6 +61,34 @@ def test_subm_rulebook_matches_oracle(gpu_handle, case):
         assert np.array_equal(n, n[::-1])
 
 
+SUBM_GEOMETRY_CASES = [
+    # (batch, space, L, ks, pad, dil, duplicates, seed): submanifold layers off the 3x3x3 / dilation 1 path
+    (2, (9, 9, 40), 900, (3, 3, 3), (1, 1, 1), (1, 1, 1), 60, 22),    # long W rows: runs of 16 cells, duplicates
+    (1, (4, 4, 100), 1200, (3, 3, 3), (1, 1, 1), (1, 1, 1), 0, 23),   # 75 % dense: long probe sequences
+    (1, (10, 10, 10), 400, (6, 5, 5), (3, 2, 2), (1, 1, 1), 0, 24),   # K = 150 > 128: offsets decoded by division
+    (1, (10, 10, 10), 400, (3, 3, 3), (0, 1, 1), (1, 1, 1), 0, 25),   # pad 0 on one axis: asymmetric window
+]
+
+
+@pytest.mark.parametrize("case", SUBM_GEOMETRY_CASES)
+def test_subm_rulebook_other_geometries(gpu_handle, case):
+    batch, space, L, ks, pad, dil, dup, seed = case
+    rng = np.random.default_rng(seed)
+    idx = random_voxels(rng, batch, space, L, shuffle=True, duplicates=dup)
+    print("subm geometry case", case, flush=True)
+    compare(gpu_handle, idx, batch, space, ks, list(pad), [1, 1, 1], list(dil), True)
+
+
+def test_subm_with_dilation_is_rejected_like_the_reference(gpu_handle):
+    """Submanifold mode requires stride 1 and dilation 1 (the reference's parameter check)."""
+    import mluop_hip
+    rng = np.random.default_rng(26)
+    idx = random_voxels(rng, 1, (8, 8, 8), 100)
+    with pytest.raises(mluop_hip.MluOpError) as e:
+        run_gpu(gpu_handle, idx, 1, (8, 8, 8), (3, 3, 3), [8, 8, 8], [2, 2, 2], [1, 1, 1], [2, 2, 2], True)
+    assert e.value.status == mluop_hip.STATUS_BAD_PARAM
+
+
 REGULAR_CASES = [
     # (batch, space, L, ks, pad, stride, dil, seed)
     (1, (6, 6, 6), 40, (3, 3, 3), (1, 1, 1), (2, 2, 2), (1, 1, 1), 0),
