@@ -57,12 +57,11 @@ __device__ __forceinline__ int offsetCount(const OffsetCounts &inl, const int32_
 // ---- element types ---------------------------------------------------------
 
 // MFMA traits: an operand fragment is 16 bytes per lane (vec8: kVec elements),
-// kChunk reduction channels per fragment; kBatch 16-pair blocks are multiplied
-// together (bounded by the registers the W fragments of a batch take).
+// kChunk reduction channels per fragment.
 struct HalfElem {
   typedef _Float16 storage;
   typedef half8 vec8;
-  static constexpr int kVec = 8, kChunk = 32, kBatch = 4;
+  static constexpr int kVec = 8, kChunk = 32;
   static __device__ __forceinline__ float load(const storage *p) { return (float)*p; }
   static __device__ __forceinline__ void store(storage *p, float v) { *p = (_Float16)v; }
   static __device__ __forceinline__ float4v mfma(vec8 a, vec8 b, float4v c) {
@@ -73,7 +72,7 @@ struct HalfElem {
 struct BFloat16Elem {
   typedef u16 storage;
   typedef bf16x8 vec8;
-  static constexpr int kVec = 8, kChunk = 32, kBatch = 4;
+  static constexpr int kVec = 8, kChunk = 32;
   static __device__ __forceinline__ float load(const storage *p) {
     return __uint_as_float((uint32_t)*p << 16);
   }
@@ -94,7 +93,7 @@ struct BFloat16Elem {
 struct FloatElem {
   typedef float storage;
   typedef float4v vec8;  // four floats: lane (m, kq) holds reduction channels 4*kq + (0..3) of a 16-chunk
-  static constexpr int kVec = 4, kChunk = 16, kBatch = 2;
+  static constexpr int kVec = 4, kChunk = 16;
   static __device__ __forceinline__ float load(const storage *p) { return *p; }
   static __device__ __forceinline__ void store(storage *p, float v) { *p = v; }
   // Four 16x16x4 steps; step s pairs element s of both fragments, i.e. channel
@@ -257,7 +256,12 @@ constexpr int kOffsetChunk = 28;  // offsets whose pair lists are resident in LD
 // Gathered rows staged in LDS per round: about 25 KiB, which one wave can hold
 // in registers while they travel (at most 24 16-byte pieces per lane).
 constexpr int mfmaStageRows(int row_bytes) {
-  return row_bytes <= 64 ? 256 : (row_bytes <= 128 ? 192 : 96);
+  return row_bytes <= 64 ? 256 : (row_bytes <= 128 ? 192 : (row_bytes <= 256 ? 96 : 48));
+}
+// 16-pair blocks multiplied together; bounded by the registers the W fragments of two batches
+// take (16 bytes per lane for every 16-byte piece of a row and every 16 result columns).
+constexpr int mfmaBatchBlocks(int elem_bytes, int Q) {
+  return elem_bytes == 2 ? 4 : (Q <= 64 ? 2 : 1);
 }
 
 // Workgroup = TR result rows x all C columns, WAVES multiplying waves and one
@@ -303,7 +307,7 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   constexpr int ALLW = NT / 64;                 // multiplying + fetching waves
   constexpr int FW = ALLW - WAVES;              // fetching waves
   constexpr int KPW = (KC + ALLW - 1) / ALLW;   // offsets a wave scans per chunk
-  constexpr int G = E::kBatch;
+  constexpr int G = mfmaBatchBlocks((int)sizeof(S), Q);
   constexpr int GROUPS = C / 16;
   constexpr int MAX_ENT = KC * TR;
   constexpr int MAX_BLK = KC * (TR / 16) + G;
@@ -875,9 +879,9 @@ bool forceSimt() {
 }
 
 // fp16/bf16: 16x16x32 MFMA, reduction channels in {32, 64, 128}; float: 16x16x4 MFMA,
-// reduction channels in {16, 32, 64} (a 512-byte row would leave too little LDS for the stage).
+// reduction channels in {16, 32, 64, 128}.
 bool mfmaShapeOk(ElemType t, int Q, int C) {
-  const bool q_ok = t == ElemType::kFloat ? (Q == 16 || Q == 32 || Q == 64)
+  const bool q_ok = t == ElemType::kFloat ? (Q == 16 || Q == 32 || Q == 64 || Q == 128)
                                           : (Q == 32 || Q == 64 || Q == 128);
   const bool c_ok = (C == 16 || C == 32 || C == 64 || C == 128);
   return q_ok && c_ok;
@@ -993,9 +997,7 @@ void launchMfma(const LaunchCtx &lc, int Q, int C, const void *A, const void *pa
       break;
     case 32: launchMfmaByC<E, 32>(lc, C, A, packed, map, R, K, result); break;
     case 64: launchMfmaByC<E, 64>(lc, C, A, packed, map, R, K, result); break;
-    case 128:
-      if constexpr (!is_float) launchMfmaByC<E, 128>(lc, C, A, packed, map, R, K, result);
-      break;
+    case 128: launchMfmaByC<E, 128>(lc, C, A, packed, map, R, K, result); break;
     default: break;
   }
 }
