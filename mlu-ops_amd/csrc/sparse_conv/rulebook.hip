@@ -338,35 +338,33 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
   }
 }
 
-// Unit strides with a kernel 3 wide along W at dilation 1 (3x3x3 and its
-// relatives).  The three offsets that differ only in kw look at three
-// consecutive cells; when those lie in one run of 16 their home slots are
-// consecutive, and one load of the eight keys from the first home slot on
-// holds the three home slots plus five more of every probe sequence: walking
-// it (a key equal to the cell is a hit, an empty slot a definite miss) settles
-// nearly every probe of the wave in one memory round trip, where probing slot
-// by slot costs one dependent round trip per step of the longest sequence
-// among the wave's 576 probes.  Sequences that leave the window continue slot
-// by slot.
+// Unit strides with a kernel KW (3 or 5) wide along W at dilation 1.  The KW
+// offsets that differ only in kw look at KW consecutive cells; when those lie
+// in one run of 16 their home slots are consecutive, and one load of the eight
+// keys from the first home slot on holds the home slots plus the next steps of
+// every probe sequence: walking it (a key equal to the cell is a hit, an empty
+// slot a definite miss) settles nearly every probe of the wave in one memory
+// round trip, where probing slot by slot costs one dependent round trip per
+// step of the longest sequence among the wave's hundreds of probes.  Cells
+// beyond a run boundary are served by a second window from the next run's
+// first home slot.  Sequences that leave their window continue slot by slot.
 constexpr int kWindow = 8;
-constexpr int kWindowB = 4;
 struct KeyWindow {
   uint32_t k[kWindow];
 };
-struct KeyWindowB {
-  uint32_t k[kWindowB];
-};
-constexpr int kTriples = 3;  // (kd, kh) pairs resolved together per lane
+constexpr int kGroupsPerPass = 3;  // (kd, kh) pairs resolved together per lane
 
+template <int KW>
 __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
     GeomDev g, UnitStrideOffsets tab, const int32_t *indices, bool aligned, const uint32_t *keys,
     const int32_t *vals, uint32_t mask, int32_t *cand, int32_t *counts, int n_wave,
-    int triples_per_slice) {
-  constexpr int N = kTriples * 3;
+    int groups_per_slice) {
+  constexpr int N = kGroupsPerPass * KW;
+  static_assert(KW <= kWindow && N <= 32, "window and bit masks");
   const int j = blockIdx.x * kBlock + threadIdx.x;
-  const int n_triples = g.K / 3;
-  const int t_lo = blockIdx.y * triples_per_slice;
-  const int t_hi = t_lo + triples_per_slice < n_triples ? t_lo + triples_per_slice : n_triples;
+  const int n_groups = g.K / KW;
+  const int t_lo = blockIdx.y * groups_per_slice;
+  const int t_hi = t_lo + groups_per_slice < n_groups ? t_lo + groups_per_slice : n_groups;
   const int lane = threadIdx.x & (kWave - 1);
   const int wt = j >> 6;
   if (wt >= n_wave) return;  // whole wave beyond the last row
@@ -379,53 +377,51 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
     ok_d |= (uint32_t)((unsigned)(c.y + g.pad[0] - t * g.dil[0]) < (unsigned)g.out[0]) << t;
   for (int t = 0; t < g.ks[1]; ++t)
     ok_h |= (uint32_t)((unsigned)(c.z + g.pad[1] - t * g.dil[1]) < (unsigned)g.out[1]) << t;
-  for (int t = 0; t < 3; ++t)
+#pragma unroll
+  for (int t = 0; t < KW; ++t)
     ok_w |= (uint32_t)((unsigned)(c.w + g.pad[2] - t) < (unsigned)g.out[2]) << t;
   if (!n_ok) ok_d = 0;
   const uint32_t padded = (((uint32_t)c.x * g.out[0] + (uint32_t)(c.y + g.pad[0])) * g.out[1] +
                            (uint32_t)(c.z + g.pad[1])) * g.out[2] + (uint32_t)(c.w + g.pad[2]);
-  for (int t0 = t_lo; t0 < t_hi; t0 += kTriples) {
+  for (int t0 = t_lo; t0 < t_hi; t0 += kGroupsPerPass) {
     uint32_t cell[N], slot[N];
     int res[N];
-    uint32_t want = 0;
-    uint32_t pending = 0, hit = 0;
+    uint32_t want = 0, pending = 0, hit = 0;
 #pragma unroll
-    for (int a = 0; a < kTriples; ++a) {
+    for (int a = 0; a < kGroupsPerPass; ++a) {
       const int t = t0 + a < t_hi ? t0 + a : t_hi - 1;  // clamped: a valid table entry
-      const uint32_t pk = tab.packed[3 * t];
+      const uint32_t pk = tab.packed[KW * t];
       const bool ok_t = t0 + a < t_hi && ((ok_d >> (pk & 0xff)) & (ok_h >> ((pk >> 8) & 0xff)) & 1u);
-      const uint32_t c0 = padded - tab.delta[3 * t + 2];  // kw = 2 is the lowest cell
-      const uint32_t r = c0 & 15u;                         // position of c0 in its run
+      const uint32_t c0 = padded - tab.delta[KW * t + KW - 1];  // kw = KW-1 is the lowest cell
+      const int r = (int)(c0 & 15u);                            // position of c0 in its run
+      // cell c0 + d belongs to kw = KW-1-d; it lies beyond c0's run when r + d > 15
+      uint32_t want_a = 0, want_b = 0;
 #pragma unroll
-      for (int kw = 0; kw < 3; ++kw) {
-        const int u = 3 * a + kw;
-        cell[u] = c0 + (uint32_t)(2 - kw);
+      for (int d = 0; d < KW; ++d) {
+        const int u = KW * a + (KW - 1 - d);
+        cell[u] = c0 + (uint32_t)d;
         res[u] = -1;
-        if (ok_t && ((ok_w >> kw) & 1u)) want |= 1u << u;
+        if (ok_t && ((ok_w >> (KW - 1 - d)) & 1u)) {
+          want |= 1u << u;
+          if (r + d > 15) want_b |= 1u << d; else want_a |= 1u << d;
+        }
       }
-      // Window A starts at c0's home slot and serves the cells of c0's run;
-      // window B starts at the home slot of the next run's first cell and
-      // serves the one or two cells beyond a run boundary (r = 14, 15).
+      // Window A starts at c0's home slot, window B at the home slot of the
+      // next run's first cell; a window must end inside the table.
       const uint32_t sa = hashCell(c0) & mask;
-      const uint32_t cb = c0 + (16u - r);
-      const uint32_t sb = hashCell(cb) & mask;
-      const uint32_t wa = (want >> (3 * a)) & 7u;  // bit kw; cell c0 + (2 - kw)
-      const uint32_t in_b = r == 15u ? 3u : (r == 14u ? 1u : 0u);  // kw = 0 (and 1) beyond the run
-      const bool load_a = (wa & ~in_b) != 0 && sa + kWindow <= mask + 1u;
-      const bool load_b = (wa & in_b) != 0 && sb + kWindowB <= mask + 1u;
-      KeyWindow win_a;
-      KeyWindowB win_b;
+      const uint32_t sb = hashCell(c0 + (uint32_t)(16 - r)) & mask;
+      const bool load_a = want_a != 0 && sa + kWindow <= mask + 1u;
+      const bool load_b = want_b != 0 && sb + kWindow <= mask + 1u;
+      KeyWindow win_a, win_b;
 #pragma unroll
-      for (int i = 0; i < kWindow; ++i) win_a.k[i] = kEmptyKey;
-#pragma unroll
-      for (int i = 0; i < kWindowB; ++i) win_b.k[i] = kEmptyKey;
+      for (int i = 0; i < kWindow; ++i) win_a.k[i] = win_b.k[i] = kEmptyKey;
       if (load_a) win_a = *reinterpret_cast<const KeyWindow *>(keys + sa);
-      if (load_b) win_b = *reinterpret_cast<const KeyWindowB *>(keys + sb);
+      if (load_b) win_b = *reinterpret_cast<const KeyWindow *>(keys + sb);
 #pragma unroll
-      for (int kw = 0; kw < 3; ++kw) {
-        const int u = 3 * a + kw;
+      for (int d = 0; d < KW; ++d) {
+        const int u = KW * a + (KW - 1 - d);
         if (!(want & (1u << u))) continue;
-        const bool beyond = (in_b >> kw) & 1u;
+        const bool beyond = r + d > 15;
         const bool loaded = beyond ? load_b : load_a;
         if (!loaded) {  // window would leave the table: slot by slot from the home slot
           slot[u] = hashCell(cell[u]) & mask;
@@ -434,35 +430,21 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
         }
         // walk the window from the cell's home slot
         const uint32_t base = beyond ? sb : sa;
-        const int first = beyond ? (int)(r + 2u - (uint32_t)kw) - 16 : 2 - kw;
+        const int first = beyond ? r + d - 16 : d;
         bool open = true;
-        if (beyond) {
 #pragma unroll
-          for (int i = 0; i < kWindowB; ++i) {
-            const uint32_t key = win_b.k[i];
-            if (open && i >= first && key == cell[u]) {
-              hit |= 1u << u;
-              slot[u] = base + (uint32_t)i;
-              open = false;
-            } else if (open && i >= first && key == kEmptyKey) {
-              open = false;
-            }
-          }
-        } else {
-#pragma unroll
-          for (int i = 0; i < kWindow; ++i) {
-            const uint32_t key = win_a.k[i];
-            if (open && i >= first && key == cell[u]) {
-              hit |= 1u << u;
-              slot[u] = base + (uint32_t)i;
-              open = false;
-            } else if (open && i >= first && key == kEmptyKey) {
-              open = false;
-            }
+        for (int i = 0; i < kWindow; ++i) {
+          const uint32_t key = beyond ? win_b.k[i] : win_a.k[i];
+          if (open && i >= first && key == cell[u]) {
+            hit |= 1u << u;
+            slot[u] = base + (uint32_t)i;
+            open = false;
+          } else if (open && i >= first && key == kEmptyKey) {
+            open = false;
           }
         }
         if (open) {
-          slot[u] = (base + (uint32_t)(beyond ? kWindowB : kWindow)) & mask;
+          slot[u] = (base + (uint32_t)kWindow) & mask;
           pending |= 1u << u;
         }
       }
@@ -494,9 +476,9 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
     }
 #pragma unroll
     for (int u = 0; u < N; ++u) {
-      const int t = t0 + u / 3;
+      const int t = t0 + u / KW;
       if (t < t_hi) {
-        const int k = 3 * t + u % 3;
+        const int k = KW * t + u % KW;
         if (active) cand[(size_t)k * g.L + j] = res[u];
         const unsigned long long b = __ballot(res[u] >= 0);
         if (lane == 0) counts[(size_t)k * n_wave + wt] = __popcll(b);
@@ -852,12 +834,18 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
                         (uint32_t)(kw * g.dilation[2]);
         }
     for (; k < kMaxInlineOffsets; ++k) ut.packed[k] = ut.delta[k] = 0;
-    if (g.ksize[2] == 3 && g.dilation[2] == 1) {
-      const int n_triples = g.K / 3;
-      const int t_per = kTriples;
+    if ((g.ksize[2] == 3 || g.ksize[2] == 5) && g.dilation[2] == 1) {
+      // one pass of kGroupsPerPass (kd, kh) pairs per wave while that leaves enough waves
+      const int n_groups = g.K / g.ksize[2];
+      const int t_per = n_groups > 4 * kGroupsPerPass ? 2 * kGroupsPerPass : kGroupsPerPass;
+      const dim3 grid(l_blocks, (n_groups + t_per - 1) / t_per);
       lc.begin("rbSubmProbeRuns");
-      rbSubmProbeRuns<<<dim3(l_blocks, (n_triples + t_per - 1) / t_per), kBlock, 0, lc.stream>>>(
-          d, ut, indices, al, ws.keys, ws.vals, mask, ws.cand, ws.counts, ws.n_wave, t_per);
+      if (g.ksize[2] == 3)
+        rbSubmProbeRuns<3><<<grid, kBlock, 0, lc.stream>>>(d, ut, indices, al, ws.keys, ws.vals, mask,
+                                                           ws.cand, ws.counts, ws.n_wave, t_per);
+      else
+        rbSubmProbeRuns<5><<<grid, kBlock, 0, lc.stream>>>(d, ut, indices, al, ws.keys, ws.vals, mask,
+                                                           ws.cand, ws.counts, ws.n_wave, t_per);
       lc.end();
     } else {
       lc.begin("rbSubmProbeUnitStride");
