@@ -250,8 +250,12 @@ constexpr int mfmaTileRows(int C) {
 constexpr int mfmaColBlocksPerWave(int C) { return C >= 128 ? 2 : 1; }
 // as many fetching waves as multiplying waves (five-wave workgroups place badly on the CU)
 constexpr int mfmaThreads(int C) { return 128 * (C / 16 / mfmaColBlocksPerWave(C)); }
-// Register budget: two eight-wave workgroups per CU need four waves per SIMD.
-constexpr int mfmaWavesPerSimd(int Q, int C) { return (Q <= 64 && C == 64) ? 4 : 2; }
+// Register budget: two eight-wave workgroups per CU need four waves per SIMD
+// (128 registers a lane); the fp32 128x128 instance holds 128 registers of
+// filter fragments alone and stays at one workgroup per CU.
+constexpr int mfmaWavesPerSimd(int elem_bytes, int Q, int C) {
+  return (elem_bytes == 4 && Q == 128 && C == 128) ? 2 : (C >= 64 ? 4 : (C == 32 ? 3 : 2));
+}
 constexpr int kOffsetChunk = 28;  // offsets whose pair lists are resident in LDS at once
 // Gathered rows staged in LDS per round: about 25 KiB, which one wave can hold
 // in registers while they travel (at most 24 16-byte pieces per lane).
@@ -260,29 +264,32 @@ constexpr int mfmaStageRows(int row_bytes) {
 }
 // 16-pair blocks multiplied together; bounded by the registers the W fragments of two batches
 // take (16 bytes per lane for every 16-byte piece of a row and every 16 result columns).
-constexpr int mfmaBatchBlocks(int elem_bytes, int Q) {
-  return elem_bytes == 2 ? 4 : (Q <= 64 ? 2 : 1);
+constexpr int mfmaBatchBlocks(int elem_bytes, int Q, int C) {
+  const int regs_per_block = (Q * elem_bytes / 64) * (C >= 128 ? 2 : 1) * 4;
+  const int g = 32 / regs_per_block;
+  return g < 1 ? 1 : (g > 4 ? 4 : g);
 }
 
-// Workgroup = TR result rows x all C columns, WAVES multiplying waves and one
-// fetching wave.  Multiplying wave w owns columns [w*16*NB, (w+1)*16*NB) of the
+// Workgroup = TR result rows x C columns (column group blockIdx.y of the ldc
+// result columns), WAVES multiplying waves and as many fetching waves.
+// Multiplying wave w owns columns [w*16*NB, (w+1)*16*NB) of the
 // fp32 accumulator tile in LDS, so no two waves ever touch the same accumulator
 // element and every element sees its contributions in ascending offset order.
 //
 // Per chunk of kOffsetChunk offsets:
-//   A   multiplying wave w loads map[k][row] for the offsets k = w (mod WAVES)
-//       of the chunk and all rows of the tile, ballots which rows have a
+//   A   wave w (of all waves) loads map[k][row] for the offsets k = w (mod all
+//       waves) of the chunk and all rows of the tile, ballots which rows have a
 //       partner and, after the per-offset counts have been exchanged, compacts
 //       one entry per pair (partner row << 8 | result row) into a flat list
 //       ordered by offset.  The list is cut into blocks of up to 16 entries of
 //       one offset, and the block list is padded to a whole batch.
 //   B   the flat list is walked in rounds of STEP entries.  The partner rows of
-//       a round are fetched by the fetching wave alone, with row-contiguous
+//       a round are fetched by the fetching waves alone, with row-contiguous
 //       16-byte loads (fetching them in the MFMA operand's own lane order
 //       touches 16 rows per load and runs at a third of the L1 rate, once per
 //       column wave), and written to the LDS stage between two barriers when
-//       the multiplying waves have finished the round before.  A wave of its
-//       own keeps these loads out of the multiplying waves' in-order load
+//       the multiplying waves have finished the round before.  Waves of their
+//       own keep these loads out of the multiplying waves' in-order load
 //       counter, where waiting for the next W fragments would also wait for
 //       them.  Every multiplying wave reads its operand fragments from the
 //       staged rows, multiplies W[k]^T (16 result columns x Q, fetched one
@@ -292,9 +299,10 @@ constexpr int mfmaBatchBlocks(int elem_bytes, int Q) {
 //       Lanes past the end of a short block repeat its first entry and
 //       accumulate into a spare row.
 template <typename E, int Q, int C>
-__global__ __launch_bounds__(mfmaThreads(C)) __attribute__((amdgpu_waves_per_eu(mfmaWavesPerSimd(Q, C), mfmaWavesPerSimd(Q, C))))
+__global__ __launch_bounds__(mfmaThreads(C)) __attribute__((amdgpu_waves_per_eu(mfmaWavesPerSimd((int)sizeof(typename E::storage), Q, C),
+                                   mfmaWavesPerSimd((int)sizeof(typename E::storage), Q, C))))
 void gatherConvMfma(const typename E::storage *A, const typename E::storage *packedW,
-                    const int32_t *map, int R, int K, typename E::storage *result) {
+                    const int32_t *map, int R, int K, int ldc, typename E::storage *result) {
   typedef typename E::vec8 vec8;
   typedef typename E::storage S;
   constexpr int NB = mfmaColBlocksPerWave(C);
@@ -307,7 +315,7 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   constexpr int ALLW = NT / 64;                 // multiplying + fetching waves
   constexpr int FW = ALLW - WAVES;              // fetching waves
   constexpr int KPW = (KC + ALLW - 1) / ALLW;   // offsets a wave scans per chunk
-  constexpr int G = mfmaBatchBlocks((int)sizeof(S), Q);
+  constexpr int G = mfmaBatchBlocks((int)sizeof(S), Q, C);
   constexpr int GROUPS = C / 16;
   constexpr int MAX_ENT = KC * TR;
   constexpr int MAX_BLK = KC * (TR / 16) + G;
@@ -339,9 +347,11 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
 
   // per-lane constants of the multiply phase
   const char *a_bytes = reinterpret_cast<const char *>(A);
+  // the workgroup owns result columns [blockIdx.y*C, (blockIdx.y+1)*C) of ldc
+  const int col_group = blockIdx.y;
   const char *b_base = reinterpret_cast<const char *>(packedW) +
-                       ((size_t)wave * NB * KB * 64 + lane) * 16;
-  constexpr uint32_t kBytesPerOffset = (uint32_t)GROUPS * KB * 64 * 16;  // packed W[k]
+                       ((size_t)(col_group * GROUPS + wave * NB) * KB * 64 + lane) * 16;
+  const uint32_t kBytesPerOffset = (uint32_t)(ldc / 16) * KB * 64 * 16;  // packed W[k]
   const int pair = lane & 15;
   const int quad = lane >> 4;
   char *acc_lane = reinterpret_cast<char *>(s_acc) + (wave * 16 * NB + 4 * quad) * 4;
@@ -533,7 +543,7 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
     S tmp[VALS];
 #pragma unroll
     for (int e = 0; e < VALS; ++e) E::store(&tmp[e], s_acc[rr * ACC_STRIDE + c0 + e]);
-    *reinterpret_cast<uint4 *>(result + (size_t)(r0 + rr) * C + c0) =
+    *reinterpret_cast<uint4 *>(result + (size_t)(r0 + rr) * ldc + col_group * C + c0) =
         *reinterpret_cast<const uint4 *>(tmp);
   }
 }
@@ -961,43 +971,56 @@ hipError_t prepareCounts(const LaunchCtx &lc, const ConvProblem &p, OffsetCounts
   return err;
 }
 
+// A 128-column result with few pairs per (64-row tile, offset) runs as two
+// 64-column halves over 128-row tiles: twice the entries in every block for
+// the same accumulator size, at the price of gathering each row twice.
+int mfmaTileCols(const ConvProblem &p, const GatherDims &d) {
+  if (d.C != 128) return d.C;
+  double pairs = 0;
+  for (int k = 0; k < p.K; ++k) pairs += (double)p.indice_num[k];
+  const double per_tile_offset = pairs * mfmaTileRows(128) / ((double)d.R * p.K);
+  return per_tile_offset < 8.0 ? 64 : 128;
+}
+
 template <typename E, int Q, int C>
 void launchMfmaInstance(const LaunchCtx &lc, const void *A, const void *packed,
-                        const int32_t *map, int R, int K, void *result) {
+                        const int32_t *map, int R, int K, int ldc, void *result) {
   constexpr int NT = mfmaThreads(C);
   constexpr int TR = mfmaTileRows(C);
-  const int blocks = (R + TR - 1) / TR;
+  const dim3 grid((R + TR - 1) / TR, ldc / C);
   lc.begin("gatherConvMfma");
-  gatherConvMfma<E, Q, C><<<blocks, NT, 0, lc.stream>>>(
+  gatherConvMfma<E, Q, C><<<grid, NT, 0, lc.stream>>>(
       static_cast<const typename E::storage *>(A),
-      static_cast<const typename E::storage *>(packed), map, R, K,
+      static_cast<const typename E::storage *>(packed), map, R, K, ldc,
       static_cast<typename E::storage *>(result));
   lc.end();
 }
 
+// `tile_cols` result columns per workgroup out of C: a narrower tile has more
+// rows, so sparse rulebooks fill their 16-pair blocks better.
 template <typename E, int Q>
-void launchMfmaByC(const LaunchCtx &lc, int C, const void *A, const void *packed,
+void launchMfmaByC(const LaunchCtx &lc, int C, int tile_cols, const void *A, const void *packed,
                    const int32_t *map, int R, int K, void *result) {
-  switch (C) {
-    case 16: launchMfmaInstance<E, Q, 16>(lc, A, packed, map, R, K, result); break;
-    case 32: launchMfmaInstance<E, Q, 32>(lc, A, packed, map, R, K, result); break;
-    case 64: launchMfmaInstance<E, Q, 64>(lc, A, packed, map, R, K, result); break;
-    case 128: launchMfmaInstance<E, Q, 128>(lc, A, packed, map, R, K, result); break;
+  switch (tile_cols) {
+    case 16: launchMfmaInstance<E, Q, 16>(lc, A, packed, map, R, K, C, result); break;
+    case 32: launchMfmaInstance<E, Q, 32>(lc, A, packed, map, R, K, C, result); break;
+    case 64: launchMfmaInstance<E, Q, 64>(lc, A, packed, map, R, K, C, result); break;
+    case 128: launchMfmaInstance<E, Q, 128>(lc, A, packed, map, R, K, C, result); break;
     default: break;
   }
 }
 
 template <typename E>
-void launchMfma(const LaunchCtx &lc, int Q, int C, const void *A, const void *packed,
+void launchMfma(const LaunchCtx &lc, int Q, int C, int tile_cols, const void *A, const void *packed,
                 const int32_t *map, int R, int K, void *result) {
   constexpr bool is_float = std::is_same<E, FloatElem>::value;
   switch (Q) {
     case 16:
-      if constexpr (is_float) launchMfmaByC<E, 16>(lc, C, A, packed, map, R, K, result);
+      if constexpr (is_float) launchMfmaByC<E, 16>(lc, C, tile_cols, A, packed, map, R, K, result);
       break;
-    case 32: launchMfmaByC<E, 32>(lc, C, A, packed, map, R, K, result); break;
-    case 64: launchMfmaByC<E, 64>(lc, C, A, packed, map, R, K, result); break;
-    case 128: launchMfmaByC<E, 128>(lc, C, A, packed, map, R, K, result); break;
+    case 32: launchMfmaByC<E, 32>(lc, C, tile_cols, A, packed, map, R, K, result); break;
+    case 64: launchMfmaByC<E, 64>(lc, C, tile_cols, A, packed, map, R, K, result); break;
+    case 128: launchMfmaByC<E, 128>(lc, C, tile_cols, A, packed, map, R, K, result); break;
     default: break;
   }
 }
@@ -1031,7 +1054,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
         d.Q, d.C, static_cast<S *>(ws.packed));
     lc.end();
     launchScatterRowMap(lc, p, d, ws, inl, max_count);
-    launchMfma<E>(lc, d.Q, d.C, gathered, ws.packed, ws.map, d.R, p.K, result);
+    launchMfma<E>(lc, d.Q, d.C, mfmaTileCols(p, d), gathered, ws.packed, ws.map, d.R, p.K, result);
     return;
   }
   lc.begin("fillInt32");

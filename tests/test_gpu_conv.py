@@ -86,6 +86,8 @@ SHAPES = [
     (2, (8, 10, 10), 500, (3, 3, 3), 64, 32, False, (2, 2, 2)),
     (1, (8, 8, 8), 300, (3, 3, 3), 32, 128, True, (1, 1, 1)),
     (1, (8, 8, 8), 300, (3, 3, 3), 128, 64, False, (1, 1, 1)),
+    (1, (8, 8, 8), 300, (3, 3, 3), 128, 128, True, (1, 1, 1)),     # dense: whole 128-column tiles
+    (1, (20, 20, 20), 300, (3, 3, 3), 128, 128, True, (1, 1, 1)),  # sparse: two 64-column halves
     (1, (6, 6, 6), 100, (3, 3, 3), 21, 10, True, (1, 1, 1)),   # odd channel counts -> SIMT
     (1, (6, 6, 6), 100, (1, 3, 3), 13, 70, False, (1, 2, 1)),
     (1, (10, 10, 10), 400, (5, 5, 7), 32, 32, True, (1, 1, 1)),   # K = 175: counts in device memory, seven chunks of offsets
