@@ -1,0 +1,166 @@
+"""Case files in the reference's prototxt form: the text-format reader against the one sample the
+reference ships (tests/golden/parser_test.prototxt, a verbatim data file of its gtest), value
+decoding (value_i / value_f / value_h hex / path / random_data), and a write -> read round trip of
+a case of every operator."""
+import os
+
+import numpy as np
+import pytest
+
+import sparse_conv_oracle as oracle
+from spconv_cases import out_space, random_voxels, round_to
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def casefile():
+    from mluop_hip import casefile as cf
+    return cf
+
+
+def test_reads_the_reference_sample():
+    cf = casefile()
+    node, _ = cf.load(os.path.join(GOLDEN, "parser_test.prototxt"))
+    assert node.get("op_name") == "abs"
+    t = cf.Message(node.get("input"))
+    assert t.get("id") == "input" and t.get("shape").all("dims") == [10, 10, 10, 10]
+    assert t.get("layout") == "LAYOUT_ARRAY" and isinstance(t.get("layout"), cf.Enum)
+    r = t.get("random_data")
+    assert (r.get("seed"), r.get("upper_bound"), r.get("lower_bound"), r.get("distribution")) == \
+        (23, 100, -100, "UNIFORM")
+    tp = node.get("test_param")
+    assert tp.all("error_func") == ["DIFF1", "DIFF2"] and tp.all("error_threshold") == [0.003, 0.003]
+    assert tp.get("baseline_device") == "CPU"
+    # writing it back and reading again gives the same tree
+    assert cf.parse(cf.dump(node)) == node
+
+
+def test_text_format_details():
+    cf = casefile()
+    msg = cf.parse('a: 1 b { c: -2.5 d: "x\\"y" }  # comment\n e: [1, 2, 3] f < g: true > h: 0x10 i: 1e-3 j: 2.0f')
+    assert msg.get("a") == 1 and msg.get("b").get("c") == -2.5 and msg.get("b").get("d") == 'x"y'
+    assert msg.all("e") == [1, 2, 3] and msg.get("f").get("g") == "true"
+    assert msg.get("h") == 16 and msg.get("i") == 1e-3 and msg.get("j") == 2.0
+    with pytest.raises(ValueError):
+        cf.parse("a { b: 1")
+    with pytest.raises(ValueError):
+        cf.parse("a: 1 }")
+
+
+def test_value_kinds_decode(tmp_path):
+    cf = casefile()
+    half = cf.CaseTensor(cf.parse(
+        'id: "x" shape { dims: 3 } dtype: DTYPE_HALF value_h: "3c00" value_h: "c000" value_h: "0001"'))
+    assert np.array_equal(half.values, np.array([1.0, -2.0, 2.0 ** -24], dtype=np.float32))
+    single = cf.CaseTensor(cf.parse('shape { dims: 2 } dtype: DTYPE_FLOAT value_h: "3f800000" value_h: "c0490fdb"'))
+    assert np.array_equal(single.values, np.array([1.0, -np.float32(np.pi)], dtype=np.float32))
+    bf = cf.CaseTensor(cf.parse('shape { dims: 2 } dtype: DTYPE_BFLOAT16 value_h: "3f80" value_h: "4049"'))
+    assert np.array_equal(bf.values, np.array([1.0, 3.140625], dtype=np.float32))
+    ints = cf.CaseTensor(cf.parse("shape { dims: 2 dims: 2 } dtype: DTYPE_INT32 value_i: 1 value_i: -1 value_i: 7 value_i: 0"))
+    assert ints.values.dtype == np.int32 and ints.values.tolist() == [[1, -1], [7, 0]]
+    floats = cf.CaseTensor(cf.parse("shape { dims: 2 } dtype: DTYPE_FLOAT value_f: 0.5 value_f: -3"))
+    assert floats.values.tolist() == [0.5, -3.0]
+    np.arange(6, dtype=np.int32).tofile(tmp_path / "t.bin")
+    frm = cf.CaseTensor(cf.parse('shape { dims: 2 dims: 3 } dtype: DTYPE_INT32 path: "t.bin"'), str(tmp_path))
+    assert frm.values.tolist() == [[0, 1, 2], [3, 4, 5]]
+    rnd = cf.CaseTensor(cf.parse(
+        "shape { dims: 1000 } dtype: DTYPE_FLOAT random_data { seed: 3 upper_bound: 2 lower_bound: -1 distribution: UNIFORM }"))
+    assert rnd.values.min() >= -1 and rnd.values.max() <= 2 and abs(rnd.values.mean() - 0.5) < 0.1
+    again = cf.CaseTensor(cf.parse(
+        "shape { dims: 1000 } dtype: DTYPE_FLOAT random_data { seed: 3 upper_bound: 2 lower_bound: -1 distribution: UNIFORM }"))
+    assert np.array_equal(rnd.values, again.values)
+    with pytest.raises(AssertionError):
+        cf.CaseTensor(cf.parse("shape { dims: 3 } dtype: DTYPE_INT32 value_i: 1"))
+
+
+def test_bf16_rounding_matches_the_oracle():
+    cf = casefile()
+    x = np.random.default_rng(0).standard_normal(4096).astype(np.float32)
+    assert np.array_equal(cf.bf16_bits_to_f32(cf.f32_to_bf16_bits(x)), oracle.round_through_bf16(x))
+
+
+def small_problem(sub_m, dtype_name, seed=5):
+    rng = np.random.default_rng(seed)
+    batch, space, ks, L, ci, co = 2, (6, 7, 8), (3, 3, 3), 120, 16, 32
+    pad, dil = [1, 1, 1], [1, 1, 1]
+    stride = [1, 1, 1] if sub_m else [2, 2, 2]
+    ospace = list(space) if sub_m else out_space(space, ks, pad, stride, dil)
+    idx = random_voxels(rng, batch, space, L)
+    pairs, out_idx, num, n_out = oracle.get_indice_pairs(idx, batch, pad, stride, dil, ks, ospace, sub_m)
+    feats = round_to(rng.standard_normal((L, ci)).astype(np.float32), dtype_name)
+    w = round_to((rng.standard_normal(ks + (ci, co)) * 0.1).astype(np.float32), dtype_name)
+    dy = round_to(rng.standard_normal((n_out, co)).astype(np.float32), dtype_name)
+    return dict(batch=batch, space=space, ks=ks, pad=pad, stride=stride, dil=dil, ospace=ospace, idx=idx,
+                pairs=pairs, out_idx=out_idx, num=num, n_out=n_out, feats=feats, w=w, dy=dy, sub_m=sub_m,
+                ci=ci, co=co, L=L)
+
+
+def operator_cases(c, dtype_name):
+    """One case per operator, baselines from the CPU oracle."""
+    cf = casefile()
+    K = int(np.prod(c["ks"]))
+    num = [int(v) for v in c["num"]]
+    fwd = round_to(oracle.forward(c["feats"], c["w"].reshape(K, c["ci"], c["co"]), c["pairs"], num, c["n_out"]),
+                   dtype_name)
+    bwd = round_to(oracle.backward_data(c["dy"], c["w"].reshape(K, c["ci"], c["co"]), c["pairs"], num),
+                   dtype_name)
+    dw = round_to(oracle.backward_filter(c["feats"], c["dy"], c["pairs"], num), dtype_name).reshape(
+        c["ks"] + (c["ci"], c["co"]))
+    return [
+        cf.get_indice_pairs_case(c["idx"], c["batch"], c["pad"], c["stride"], c["dil"], c["space"], c["ks"],
+                                 c["ospace"], c["sub_m"], baseline=(c["out_idx"], c["pairs"], c["num"])),
+        cf.indice_convolution_forward_case(c["feats"], c["w"], c["pairs"], num, c["n_out"], c["sub_m"],
+                                           dtype_name, baseline=fwd),
+        cf.indice_convolution_backward_data_case(c["dy"], c["w"], c["pairs"], num, c["L"], c["sub_m"],
+                                                 dtype_name, baseline=bwd),
+        cf.indice_convolution_backward_filter_case(c["feats"], c["dy"], c["pairs"], num, c["ks"], c["sub_m"],
+                                                   dtype_name, baseline=dw),
+    ]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "float16", "bfloat16"])
+def test_written_cases_read_back_exactly(dtype_name):
+    cf = casefile()
+    c = small_problem(True, dtype_name)
+    for node in operator_cases(c, dtype_name):
+        text = cf.dump(node)
+        back = cf.parse(text)
+        assert back == node
+        for written, read in zip(node.all("input") + node.all("output"), back.all("input") + back.all("output")):
+            t = cf.CaseTensor(read)
+            assert t.values is not None and list(t.values.shape) == t.shape
+    fwd = operator_cases(c, dtype_name)[1]
+    feats = cf.CaseTensor(fwd.all("input")[0])
+    assert np.array_equal(feats.values, c["feats"])          # value_h carries the exact bits
+    p = fwd.get("indice_convolution_forward_param")
+    assert p.all("indice_num") == [int(v) for v in c["num"]] and p.get("num_active_out") == c["n_out"]
+    gp = operator_cases(c, dtype_name)[0].get("get_indice_pairs_param")
+    assert gp.all("filter_space") == [3, 3, 3] and gp.get("sub_m") == 1 and gp.get("batch") == 2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sub_m", [True, False])
+@pytest.mark.parametrize("dtype_name", ["float32", "float16", "bfloat16"])
+def test_replayed_cases_meet_their_thresholds(gpu_handle, tmp_path, sub_m, dtype_name):
+    """Cases written to disk with oracle baselines, replayed through the C API from the files."""
+    cf = casefile()
+    c = small_problem(sub_m, dtype_name, seed=6)
+    thr = 1e-5 if dtype_name == "float32" else 3e-3
+    for node in operator_cases(c, dtype_name):
+        tp = node.get("test_param")
+        if node.get("op_name") != "get_indice_pairs":
+            tp[:] = [(n, (thr if n == "error_threshold" else v)) for n, v in tp]
+        path = tmp_path / (node.get("op_name") + ".prototxt")
+        path.write_text(cf.dump(node))
+        res = cf.replay(str(path), gpu_handle)
+        assert res.errors, "no baseline compared"
+        assert res.passed, (node.get("op_name"), res.errors)
+
+
+@pytest.mark.gpu
+def test_replay_refuses_other_operators(gpu_handle):
+    cf = casefile()
+    with open(os.path.join(GOLDEN, "parser_test.prototxt")) as f:
+        text = f.read()
+    with pytest.raises(ValueError):
+        cf.replay(text, gpu_handle)
