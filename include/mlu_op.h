@@ -24,6 +24,7 @@
 #define MLUOP_VERSION (MLUOP_MAJOR * 1000 + MLUOP_MINOR * 100 + MLUOP_PATCHLEVEL)
 #define MLUOP_DIM_MAX 8
 
+#include <stdbool.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -395,6 +396,60 @@ mluOpIndiceConvolutionBackwardFilter(mluOpHandle_t handle,
                                      const size_t workspace_size,
                                      const mluOpTensorDescriptor_t filters_grad_desc,
                                      void *filters_grad);
+
+/* ---------------------------------------------------------------------------
+ * Hard voxelization: the step in front of the sparse convolutions, which turns a
+ * point cloud into the voxel coordinates and features they consume.
+ * ------------------------------------------------------------------------- */
+
+/* reference mlu_op.h:5941-5953 (kernels/voxelization/voxelization.cpp:174-222).
+ * Bytes of workspace mluOpVoxelization needs for these shapes.  Left untouched
+ * when max_points or max_voxels is 0 (nothing to do), as in the reference. */
+mluOpStatus_t MLUOP_WIN_API
+mluOpGetVoxelizationWorkspaceSize(mluOpHandle_t handle,
+                                  const mluOpTensorDescriptor_t points_desc,
+                                  const mluOpTensorDescriptor_t voxel_size_desc,
+                                  const mluOpTensorDescriptor_t coors_range_desc,
+                                  const int32_t max_points,
+                                  const int32_t max_voxels,
+                                  const int32_t NDim,
+                                  const bool deterministic,
+                                  const mluOpTensorDescriptor_t voxels_desc,
+                                  const mluOpTensorDescriptor_t coors_desc,
+                                  const mluOpTensorDescriptor_t num_points_per_voxel_desc,
+                                  const mluOpTensorDescriptor_t voxel_num_desc,
+                                  size_t *size);
+
+/* reference mlu_op.h:6050-6071 (kernels/voxelization/voxelization.cpp:224-367).
+ * points [N, F] float (x, y, z first), voxel_size [3] and coors_range [6]
+ * (x/y/z minima, then maxima) float, all in device memory.  Outputs, zero
+ * filled first: voxels [max_voxels, max_points, F] float, coors [max_voxels, 3]
+ * int32 as (z, y, x), num_points_per_voxel [max_voxels] int32, voxel_num [1]
+ * int32.  Cells are numbered in the order of their first point; a cell keeps
+ * its first max_points points, and cells past max_voxels are dropped.  Only
+ * deterministic = true and NDim = 3 are accepted (BAD_PARAM otherwise). */
+mluOpStatus_t MLUOP_WIN_API
+mluOpVoxelization(mluOpHandle_t handle,
+                  const mluOpTensorDescriptor_t points_desc,
+                  const void *points,
+                  const mluOpTensorDescriptor_t voxel_size_desc,
+                  const void *voxel_size,
+                  const mluOpTensorDescriptor_t coors_range_desc,
+                  const void *coors_range,
+                  const int32_t max_points,
+                  const int32_t max_voxels,
+                  const int32_t NDim,
+                  const bool deterministic,
+                  void *workspace,
+                  size_t workspace_size,
+                  const mluOpTensorDescriptor_t voxels_desc,
+                  void *voxels,
+                  const mluOpTensorDescriptor_t coors_desc,
+                  void *coors,
+                  const mluOpTensorDescriptor_t num_points_per_voxel_desc,
+                  void *num_points_per_voxel,
+                  const mluOpTensorDescriptor_t voxel_num_desc,
+                  void *voxel_num);
 
 #if defined(__cplusplus)
 }

@@ -1,0 +1,317 @@
+// Hard voxelization (deterministic): every point is assigned to the cell of a
+// regular grid it falls in; cells are numbered in the order of their first
+// point, keep their first max_points points in point order, and only the
+// first max_voxels cells are kept.
+//
+// The reference searches, for every point, all earlier points for the same
+// cell (kernels/voxelization/voxelization_kernel.mlu, KernelPoint2Voxel), then
+// numbers the voxels with a single core
+// (kernels/voxelization/voxelization.cpp:45-53).  Here the same result comes
+// from grouping instead of searching:
+//   1 voxCellSlots   cell of every point; the 64-bit cell id is entered into an
+//                    open-addressing table, whose slot number names the cell
+//   2 radix sort     (slot, point index) pairs by slot, least significant
+//                    digit first and therefore stable: every cell's points end
+//                    up adjacent and in point order
+//   3 voxHeads       first sorted position of every cell
+//   4 voxRanks       position of a point in its cell = sorted position - head;
+//                    the cell's first point = the point at the head
+//   5 exclusive scan over "is the first point of its cell" in point order:
+//                    the voxel number of every cell, as the sequential
+//                    numbering of the reference gives it
+//   6 voxAssign      copies points and coordinates, counts points per voxel
+// Integer atomics only (table insertion, per-voxel counts): the outputs are
+// the same bits on every run.
+#include <hip/hip_runtime.h>
+#include <cstring>
+
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
+
+#include "voxelization/voxelize.h"
+
+namespace mluop {
+namespace voxelization {
+namespace {
+
+constexpr unsigned long long kEmptyKey = ~0ull;
+constexpr int kBlock = 256;
+
+inline int gridFor(size_t n, int cap = 1 << 20) {
+  size_t b = (n + kBlock - 1) / kBlock;
+  if (b < 1) b = 1;
+  return (int)(b > (size_t)cap ? (size_t)cap : b);
+}
+
+size_t alignUp(size_t v) { return (v + 255) & ~(size_t)255; }
+
+uint32_t tableSlots(int64_t num_points) {
+  uint32_t cap = 1024;
+  while ((int64_t)cap < 2 * num_points) cap <<= 1;
+  return cap;
+}
+
+int bitsFor(uint32_t cap) {  // slot numbers 0..cap (cap itself marks "no cell")
+  int b = 1;
+  while ((1ull << b) <= cap) ++b;
+  return b;
+}
+
+__global__ __launch_bounds__(kBlock) void voxFill16(uint4 *dst, size_t quads, uint32_t *tail,
+                                                    int tail_words, uint32_t value) {
+  const uint4 v = make_uint4(value, value, value, value);
+  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < quads;
+       i += (size_t)gridDim.x * kBlock)
+    dst[i] = v;
+  if (blockIdx.x == 0 && (int)threadIdx.x < tail_words) tail[threadIdx.x] = value;
+}
+
+// Cells along one axis: the float quotient rounded half away from zero.
+__device__ inline int axisCells(float lo, float hi, float size) {
+  const float g = roundf((hi - lo) / size);
+  return (g >= 1.f && g < 2147483648.f) ? (int)g : 0;
+}
+
+// Cell index of a coordinate, or -1 outside [0, cells) (NaN included).
+__device__ inline int cellIndex(float p, float lo, float size, int cells) {
+  const float f = floorf((p - lo) / size);
+  if (!(f >= 0.f && f < 2147483648.f)) return -1;
+  const int c = (int)f;
+  return c < cells ? c : -1;
+}
+
+__device__ inline uint32_t mix64(unsigned long long k) {
+  k ^= k >> 33;
+  k *= 0xff51afd7ed558ccdull;
+  k ^= k >> 33;
+  k *= 0xc4ceb9fe1a85ec53ull;
+  k ^= k >> 33;
+  return (uint32_t)k;
+}
+
+__global__ __launch_bounds__(kBlock) void voxCellSlots(
+    const float *__restrict__ points, const float *__restrict__ voxel_size,
+    const float *__restrict__ range, int64_t n, int num_features, unsigned long long *keys,
+    uint32_t cap, int32_t *cell_zyx, uint32_t *slot_of, uint32_t *point_of) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const float sx = voxel_size[0], sy = voxel_size[1], sz = voxel_size[2];
+  const float x0 = range[0], y0 = range[1], z0 = range[2];
+  const int gx = axisCells(x0, range[3], sx);
+  const int gy = axisCells(y0, range[4], sy);
+  const int gz = axisCells(z0, range[5], sz);
+  const float *p = points + i * num_features;
+  const int cx = cellIndex(p[0], x0, sx, gx);
+  const int cy = cx < 0 ? -1 : cellIndex(p[1], y0, sy, gy);
+  const int cz = cy < 0 ? -1 : cellIndex(p[2], z0, sz, gz);
+  point_of[i] = (uint32_t)i;
+  if (cz < 0) {
+    cell_zyx[3 * i] = cell_zyx[3 * i + 1] = cell_zyx[3 * i + 2] = -1;
+    slot_of[i] = cap;
+    return;
+  }
+  cell_zyx[3 * i] = cz;
+  cell_zyx[3 * i + 1] = cy;
+  cell_zyx[3 * i + 2] = cx;
+  const unsigned long long key =
+      ((unsigned long long)cz * (unsigned long long)gy + cy) * (unsigned long long)gx + cx;
+  uint32_t slot = mix64(key) & (cap - 1);
+  // at most half of the slots are ever taken, so an empty one is always reached
+  while (true) {
+    const unsigned long long seen = atomicCAS(&keys[slot], kEmptyKey, key);
+    if (seen == kEmptyKey || seen == key) break;
+    slot = (slot + 1) & (cap - 1);
+  }
+  slot_of[i] = slot;
+}
+
+__global__ __launch_bounds__(kBlock) void voxHeads(const uint32_t *__restrict__ slot_sorted,
+                                                   int64_t n, uint32_t cap, uint32_t *head) {
+  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (p >= n) return;
+  const uint32_t s = slot_sorted[p];
+  if (s == cap) return;
+  if (p == 0 || slot_sorted[p - 1] != s) head[s] = (uint32_t)p;
+}
+
+__global__ __launch_bounds__(kBlock) void voxRanks(const uint32_t *__restrict__ slot_sorted,
+                                                   const uint32_t *__restrict__ point_sorted,
+                                                   const uint32_t *__restrict__ head, int64_t n,
+                                                   uint32_t cap, int32_t *rank, int32_t *first,
+                                                   uint32_t *is_first) {
+  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (p >= n) return;
+  const uint32_t s = slot_sorted[p];
+  const uint32_t i = point_sorted[p];
+  if (s == cap) {
+    rank[i] = -1;
+    first[i] = -1;
+    is_first[i] = 0;
+    return;
+  }
+  const uint32_t h = head[s];
+  rank[i] = (int32_t)((uint32_t)p - h);
+  first[i] = (int32_t)point_sorted[h];
+  is_first[i] = (uint32_t)p == h ? 1u : 0u;
+}
+
+__global__ __launch_bounds__(kBlock) void voxAssign(
+    const float *__restrict__ points, const int32_t *__restrict__ cell_zyx,
+    const int32_t *__restrict__ rank, const int32_t *__restrict__ first,
+    const uint32_t *__restrict__ is_first, const uint32_t *__restrict__ voxel_of_first, int64_t n,
+    int num_features, int max_points, int max_voxels, float *voxels, int32_t *coors,
+    int32_t *num_points_per_voxel, int32_t *voxel_num) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  if (i == n - 1) {
+    const uint32_t cells = voxel_of_first[i] + is_first[i];
+    *voxel_num = cells < (uint32_t)max_voxels ? (int32_t)cells : max_voxels;
+  }
+  const int32_t r = rank[i];
+  if (r < 0 || r >= max_points) return;
+  const uint32_t v = voxel_of_first[first[i]];
+  if (v >= (uint32_t)max_voxels) return;
+  const float *src = points + i * num_features;
+  float *dst = voxels + ((size_t)v * max_points + r) * num_features;
+  for (int f = 0; f < num_features; ++f) dst[f] = src[f];
+  atomicAdd(&num_points_per_voxel[v], 1);
+  if (r == 0) {
+    coors[3 * (size_t)v] = cell_zyx[3 * i];
+    coors[3 * (size_t)v + 1] = cell_zyx[3 * i + 1];
+    coors[3 * (size_t)v + 2] = cell_zyx[3 * i + 2];
+  }
+}
+
+struct Workspace {
+  int32_t *cell_zyx;
+  uint32_t *slot_of, *point_of, *slot_sorted, *point_sorted, *is_first, *voxel_of_first, *head;
+  unsigned long long *keys;
+  void *library;
+  size_t total;
+};
+
+Workspace carve(void *base, const VoxelizeShape &s, size_t library_bytes) {
+  const size_t n = (size_t)s.num_points;
+  const uint32_t cap = tableSlots(s.num_points);
+  char *p = static_cast<char *>(base);
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    char *q = p + off;
+    off += alignUp(bytes);
+    return q;
+  };
+  Workspace w;
+  w.cell_zyx = reinterpret_cast<int32_t *>(take(12 * n));
+  w.slot_of = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.point_of = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.slot_sorted = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.point_sorted = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.is_first = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.voxel_of_first = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.head = reinterpret_cast<uint32_t *>(take(4 * (size_t)cap));
+  w.keys = reinterpret_cast<unsigned long long *>(take(8 * (size_t)cap));
+  w.library = take(library_bytes);
+  w.total = off;
+  return w;
+}
+
+hipError_t fillWords(const LaunchCtx &lc, const char *name, void *dst, size_t words,
+                     uint32_t value) {
+  if (words == 0) return hipSuccess;
+  lc.begin(name);
+  voxFill16<<<gridFor(words / 4 + 1, 4096), kBlock, 0, lc.stream>>>(
+      static_cast<uint4 *>(dst), words / 4, static_cast<uint32_t *>(dst) + (words / 4) * 4,
+      (int)(words & 3), value);
+  lc.end();
+  return hipGetLastError();
+}
+
+}  // namespace
+
+size_t voxelizeWorkspaceBytes(const VoxelizeShape &s, size_t library_bytes) {
+  return carve(nullptr, s, library_bytes).total;
+}
+
+hipError_t libraryWorkspaceBytes(const VoxelizeShape &s, hipStream_t stream, size_t *bytes) {
+  const uint32_t cap = tableSlots(s.num_points);
+  size_t sort_bytes = 0, scan_bytes = 0;
+  uint32_t *u = nullptr;
+  hipError_t e = rocprim::radix_sort_pairs(nullptr, sort_bytes, u, u, u, u, (size_t)s.num_points, 0,
+                                           bitsFor(cap), stream);
+  if (e != hipSuccess) return e;
+  e = rocprim::exclusive_scan(nullptr, scan_bytes, u, u, 0u, (size_t)s.num_points,
+                              rocprim::plus<uint32_t>(), stream);
+  if (e != hipSuccess) return e;
+  *bytes = sort_bytes > scan_bytes ? sort_bytes : scan_bytes;
+  return hipSuccess;
+}
+
+hipError_t launchVoxelize(const LaunchCtx &lc, const VoxelizeShape &s, const float *points,
+                          const float *voxel_size, const float *coors_range, void *workspace,
+                          size_t workspace_bytes, float *voxels, int32_t *coors,
+                          int32_t *num_points_per_voxel, int32_t *voxel_num) {
+  const int64_t n = s.num_points;
+  const uint32_t cap = tableSlots(n);
+  size_t library_bytes = 0;
+  hipError_t e = libraryWorkspaceBytes(s, lc.stream, &library_bytes);
+  if (e != hipSuccess) return e;
+  const Workspace w = carve(workspace, s, library_bytes);
+  if (w.total > workspace_bytes) return hipErrorInvalidValue;
+
+  // outputs start from zero (reference kernels/voxelization/voxelization.cpp:283-309)
+  e = fillWords(lc, "voxFill16", voxels, (size_t)s.max_voxels * s.max_points * s.num_features, 0u);
+  if (e != hipSuccess) return e;
+  e = fillWords(lc, "voxFill16", coors, (size_t)s.max_voxels * 3, 0u);
+  if (e != hipSuccess) return e;
+  e = fillWords(lc, "voxFill16", num_points_per_voxel, (size_t)s.max_voxels, 0u);
+  if (e != hipSuccess) return e;
+  e = fillWords(lc, "voxFill16", w.keys, (size_t)cap * 2, 0xffffffffu);
+  if (e != hipSuccess) return e;
+
+  const int blocks = gridFor((size_t)n);
+  lc.begin("voxCellSlots");
+  voxCellSlots<<<blocks, kBlock, 0, lc.stream>>>(points, voxel_size, coors_range, n,
+                                                  s.num_features, w.keys, cap, w.cell_zyx,
+                                                  w.slot_of, w.point_of);
+  lc.end();
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+
+  lc.begin("radixSortPairs");
+  size_t lib = library_bytes;
+  e = rocprim::radix_sort_pairs(w.library, lib, w.slot_of, w.slot_sorted, w.point_of,
+                                w.point_sorted, (size_t)n, 0, bitsFor(cap), lc.stream);
+  lc.end();
+  if (e != hipSuccess) return e;
+
+  lc.begin("voxHeads");
+  voxHeads<<<blocks, kBlock, 0, lc.stream>>>(w.slot_sorted, n, cap, w.head);
+  lc.end();
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+
+  // the unsorted pair arrays are free again: they take rank and first point
+  int32_t *rank = reinterpret_cast<int32_t *>(w.slot_of);
+  int32_t *first = reinterpret_cast<int32_t *>(w.point_of);
+  lc.begin("voxRanks");
+  voxRanks<<<blocks, kBlock, 0, lc.stream>>>(w.slot_sorted, w.point_sorted, w.head, n, cap, rank,
+                                              first, w.is_first);
+  lc.end();
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+
+  lc.begin("exclusiveScan");
+  lib = library_bytes;
+  e = rocprim::exclusive_scan(w.library, lib, w.is_first, w.voxel_of_first, 0u, (size_t)n,
+                              rocprim::plus<uint32_t>(), lc.stream);
+  lc.end();
+  if (e != hipSuccess) return e;
+
+  lc.begin("voxAssign");
+  voxAssign<<<blocks, kBlock, 0, lc.stream>>>(points, w.cell_zyx, rank, first, w.is_first,
+                                               w.voxel_of_first, n, s.num_features, s.max_points,
+                                               s.max_voxels, voxels, coors, num_points_per_voxel,
+                                               voxel_num);
+  lc.end();
+  return hipGetLastError();
+}
+
+}  // namespace voxelization
+}  // namespace mluop

@@ -102,6 +102,12 @@ SIGNATURES = {
     "mluOpIndiceConvolutionBackwardFilter": (
         ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64p, ctypes.c_int64, ctypes.c_int64,
                        _vp, ctypes.c_size_t, _vp, _vp]),
+    "mluOpGetVoxelizationWorkspaceSize": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_bool,
+                       _vp, _vp, _vp, _vp, _szp]),
+    "mluOpVoxelization": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                       ctypes.c_bool, _vp, ctypes.c_size_t, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     # mlu_op_ext.h
     "mluOpExtSetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int]),
     "mluOpExtGetKernelTimingCount": (ctypes.c_int, [_vp, _ip]),
@@ -390,3 +396,37 @@ def indice_conv_backward_filter(handle, features, output_grad, indice_pairs, ind
         indice_pairs.data_ptr(), counts, inverse, int(sub_m), ws.data_ptr(), size.value, d_dw.ptr,
         dw.data_ptr()), "mluOpIndiceConvolutionBackwardFilter")
     return dw
+
+
+def voxelization(handle, points, voxel_size, coors_range, max_points, max_voxels, deterministic=True):
+    """Hard voxelization of `points` [N, F] (float32 device tensor; x, y, z first).
+
+    voxel_size [3] and coors_range [6] are float32 device tensors.  Returns (voxels
+    [max_voxels, max_points, F], coors [max_voxels, 3] int32 (z, y, x), num_points_per_voxel
+    [max_voxels] int32, voxel_num [1] int32), all on the device."""
+    torch = _torch()
+    n, f = points.shape
+    dev = points.device
+    voxels = torch.empty((max_voxels, max_points, f), dtype=torch.float32, device=dev)
+    coors = torch.empty((max_voxels, 3), dtype=torch.int32, device=dev)
+    npv = torch.empty((max_voxels,), dtype=torch.int32, device=dev)
+    voxel_num = torch.zeros((1,), dtype=torch.int32, device=dev)
+    d_points = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, f])
+    d_vs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [3])
+    d_cr = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [6])
+    d_voxels = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [max_voxels, max_points, f])
+    d_coors = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [max_voxels, 3])
+    d_npv = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [max_voxels])
+    d_num = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [1])
+    size = ctypes.c_size_t(0)
+    check(lib().mluOpGetVoxelizationWorkspaceSize(
+        handle.ptr, d_points.ptr, d_vs.ptr, d_cr.ptr, max_points, max_voxels, 3, bool(deterministic),
+        d_voxels.ptr, d_coors.ptr, d_npv.ptr, d_num.ptr, ctypes.byref(size)),
+        "mluOpGetVoxelizationWorkspaceSize")
+    ws = _workspace(size.value, dev)
+    check(lib().mluOpVoxelization(
+        handle.ptr, d_points.ptr, points.data_ptr(), d_vs.ptr, voxel_size.data_ptr(), d_cr.ptr,
+        coors_range.data_ptr(), max_points, max_voxels, 3, bool(deterministic), ws.data_ptr(), size.value,
+        d_voxels.ptr, voxels.data_ptr(), d_coors.ptr, coors.data_ptr(), d_npv.ptr, npv.data_ptr(), d_num.ptr,
+        voxel_num.data_ptr()), "mluOpVoxelization")
+    return voxels, coors, npv, voxel_num
