@@ -57,13 +57,33 @@ int bitsFor(uint32_t cap) {  // slot numbers 0..cap (cap itself marks "no cell")
   return b;
 }
 
-__global__ __launch_bounds__(kBlock) void voxFill16(uint4 *dst, size_t quads, uint32_t *tail,
-                                                    int tail_words, uint32_t value) {
-  const uint4 v = make_uint4(value, value, value, value);
-  for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < quads;
-       i += (size_t)gridDim.x * kBlock)
-    dst[i] = v;
-  if (blockIdx.x == 0 && (int)threadIdx.x < tail_words) tail[threadIdx.x] = value;
+// Up to four regions of 32-bit words filled by one launch.
+struct FillRegions {
+  uint32_t *base[4];
+  size_t words[4];
+  uint32_t value[4];
+};
+
+__global__ __launch_bounds__(kBlock) void voxFillRegions(FillRegions r) {
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    // words in front of the first 16-byte boundary, 16-byte stores, words behind the last
+    size_t head = ((16 - (reinterpret_cast<uintptr_t>(r.base[g]) & 15)) & 15) / 4;
+    head = head < r.words[g] ? head : r.words[g];
+    uint32_t *body = r.base[g] + head;
+    const size_t body_words = r.words[g] - head;
+    const size_t quads = body_words / 4;
+    const uint32_t value = r.value[g];
+    const uint4 v = make_uint4(value, value, value, value);
+    uint4 *dst = reinterpret_cast<uint4 *>(body);
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < quads;
+         i += (size_t)gridDim.x * kBlock)
+      dst[i] = v;
+    if (blockIdx.x == 0) {
+      if (threadIdx.x < head) r.base[g][threadIdx.x] = value;
+      if (threadIdx.x < (body_words & 3)) body[quads * 4 + threadIdx.x] = value;
+    }
+  }
 }
 
 // Cells along one axis: the float quotient rounded half away from zero.
@@ -116,11 +136,25 @@ __global__ __launch_bounds__(kBlock) void voxCellSlots(
   const unsigned long long key =
       ((unsigned long long)cz * (unsigned long long)gy + cy) * (unsigned long long)gx + cx;
   uint32_t slot = mix64(key) & (cap - 1);
-  // at most half of the slots are ever taken, so an empty one is always reached
-  while (true) {
-    const unsigned long long seen = atomicCAS(&keys[slot], kEmptyKey, key);
-    if (seen == kEmptyKey || seen == key) break;
-    slot = (slot + 1) & (cap - 1);
+  // At most half of the slots are ever taken, so an empty one is always reached.
+  // A grid of fewer than 2^32 - 1 cells (the same for every thread) keeps 32-bit
+  // keys in the first half of the table: 32-bit compare-and-swap is several times
+  // faster than the 64-bit one.
+  const unsigned long long cells = (unsigned long long)gz * (unsigned long long)gy * gx;
+  if (cells < 0xffffffffull) {
+    uint32_t *keys32 = reinterpret_cast<uint32_t *>(keys);
+    const uint32_t key32 = (uint32_t)key;
+    while (true) {
+      const uint32_t seen = atomicCAS(&keys32[slot], 0xffffffffu, key32);
+      if (seen == 0xffffffffu || seen == key32) break;
+      slot = (slot + 1) & (cap - 1);
+    }
+  } else {
+    while (true) {
+      const unsigned long long seen = atomicCAS(&keys[slot], kEmptyKey, key);
+      if (seen == kEmptyKey || seen == key) break;
+      slot = (slot + 1) & (cap - 1);
+    }
   }
   slot_of[i] = slot;
 }
@@ -215,16 +249,6 @@ Workspace carve(void *base, const VoxelizeShape &s, size_t library_bytes) {
   return w;
 }
 
-hipError_t fillWords(const LaunchCtx &lc, const char *name, void *dst, size_t words,
-                     uint32_t value) {
-  if (words == 0) return hipSuccess;
-  lc.begin(name);
-  voxFill16<<<gridFor(words / 4 + 1, 4096), kBlock, 0, lc.stream>>>(
-      static_cast<uint4 *>(dst), words / 4, static_cast<uint32_t *>(dst) + (words / 4) * 4,
-      (int)(words & 3), value);
-  lc.end();
-  return hipGetLastError();
-}
 
 }  // namespace
 
@@ -259,14 +283,25 @@ hipError_t launchVoxelize(const LaunchCtx &lc, const VoxelizeShape &s, const flo
   if (w.total > workspace_bytes) return hipErrorInvalidValue;
 
   // outputs start from zero (reference kernels/voxelization/voxelization.cpp:283-309)
-  e = fillWords(lc, "voxFill16", voxels, (size_t)s.max_voxels * s.max_points * s.num_features, 0u);
-  if (e != hipSuccess) return e;
-  e = fillWords(lc, "voxFill16", coors, (size_t)s.max_voxels * 3, 0u);
-  if (e != hipSuccess) return e;
-  e = fillWords(lc, "voxFill16", num_points_per_voxel, (size_t)s.max_voxels, 0u);
-  if (e != hipSuccess) return e;
-  e = fillWords(lc, "voxFill16", w.keys, (size_t)cap * 2, 0xffffffffu);
-  if (e != hipSuccess) return e;
+  // and the cell table from "empty"
+  FillRegions fr;
+  fr.base[0] = reinterpret_cast<uint32_t *>(voxels);
+  fr.words[0] = (size_t)s.max_voxels * s.max_points * s.num_features;
+  fr.base[1] = reinterpret_cast<uint32_t *>(coors);
+  fr.words[1] = (size_t)s.max_voxels * 3;
+  fr.base[2] = reinterpret_cast<uint32_t *>(num_points_per_voxel);
+  fr.words[2] = (size_t)s.max_voxels;
+  fr.base[3] = reinterpret_cast<uint32_t *>(w.keys);
+  fr.words[3] = (size_t)cap * 2;
+  size_t most = 0;
+  for (int g = 0; g < 4; ++g) {
+    fr.value[g] = g == 3 ? 0xffffffffu : 0u;
+    most = fr.words[g] > most ? fr.words[g] : most;
+  }
+  lc.begin("voxFillRegions");
+  voxFillRegions<<<gridFor(most / 4 + 1, 4096), kBlock, 0, lc.stream>>>(fr);
+  lc.end();
+  if ((e = hipGetLastError()) != hipSuccess) return e;
 
   const int blocks = gridFor((size_t)n);
   lc.begin("voxCellSlots");

@@ -16,7 +16,7 @@ import math
 import torch
 
 from . import (LAYOUT_ARRAY, get_indice_pairs, indice_conv_backward_data, indice_conv_backward_filter,
-               indice_conv_forward, make_handle_on_current_stream, regular_output_space)
+               indice_conv_forward, make_handle_on_current_stream, regular_output_space, voxelization)
 
 _handles = {}
 
@@ -159,3 +159,39 @@ class SparseConv3d(_ConvBase):
                  indice_key=None):
         super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, False, bias,
                          indice_key)
+
+
+class Voxelization(torch.nn.Module):
+    """Hard voxelization of one point cloud [N, F] (x, y, z first), the module mmcv puts in front of
+    its sparse encoder: returns (voxels [V, max_num_points, F], coors [V, 3] as (z, y, x),
+    num_points_per_voxel [V]) cut to the V voxels found.  Reading V costs one device-to-host copy."""
+
+    def __init__(self, voxel_size, point_cloud_range, max_num_points, max_voxels):
+        super().__init__()
+        self.register_buffer("voxel_size", torch.tensor(voxel_size, dtype=torch.float32))
+        self.register_buffer("point_cloud_range", torch.tensor(point_cloud_range, dtype=torch.float32))
+        self.max_num_points = int(max_num_points)
+        self.max_voxels = int(max_voxels)
+
+    def grid_shape(self):
+        """(D, H, W) = cells along (z, y, x), the spatial shape of the sparse tensor."""
+        r, s = self.point_cloud_range.tolist(), self.voxel_size.tolist()
+        return tuple(int(math.floor((r[3 + a] - r[a]) / s[a] + 0.5)) for a in (2, 1, 0))
+
+    @torch.no_grad()
+    def forward(self, points):
+        voxels, coors, npv, num = voxelization(_handle(), points.contiguous().float(), self.voxel_size,
+                                               self.point_cloud_range, self.max_num_points, self.max_voxels)
+        v = int(num.item())
+        return voxels[:v], coors[:v], npv[:v]
+
+
+def mean_voxel_features(voxels, num_points_per_voxel):
+    """Mean of the points of every voxel (mmcv's HardSimpleVFE): [V, max_points, F] -> [V, F]."""
+    return voxels.sum(dim=1) / num_points_per_voxel.clamp(min=1).to(voxels.dtype).unsqueeze(1)
+
+
+def sparse_tensor_from_voxels(features, coors, spatial_shape, batch_index=0, batch_size=1):
+    """SparseTensor of one cloud's voxels: indices (n, z, y, x) with n = batch_index."""
+    n = torch.full((coors.shape[0], 1), int(batch_index), dtype=torch.int32, device=coors.device)
+    return SparseTensor(features, torch.cat([n, coors.to(torch.int32)], dim=1), spatial_shape, batch_size)

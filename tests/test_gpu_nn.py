@@ -100,3 +100,38 @@ def test_half_precision_layer_runs_mfma_path(gpu_handle):
         np.add.at(ref, pairs[k, 1, :n], f64[pairs[k, 0, :n]] @ w[k])
     d1 = np.abs(y - ref).sum() / (np.abs(ref).sum() + 1e-9)
     assert d1 <= 3e-3, d1
+
+
+def test_points_to_voxels_to_submanifold_layer(gpu_handle):
+    """points -> Voxelization -> mean features -> SparseTensor -> SubMConv3d: voxel coordinates are
+    distinct cells of the grid, and the layer's output equals the dense convolution of the voxel
+    grid at those cells."""
+    import torch
+    import torch.nn.functional as F
+    from mluop_hip import nn as spnn
+    rng = np.random.default_rng(23)
+    pts = np.empty((4000, 4), np.float32)
+    pts[:, 0] = rng.uniform(0, 6.4, 4000)
+    pts[:, 1] = rng.uniform(-3.2, 3.2, 4000)
+    pts[:, 2] = rng.uniform(-1, 1, 4000)
+    pts[:, 3] = rng.uniform(0, 1, 4000)
+    vox = spnn.Voxelization([0.4, 0.4, 0.5], [0, -3.2, -1, 6.4, 3.2, 1], max_num_points=8, max_voxels=5000).cuda()
+    space = vox.grid_shape()
+    assert space == (4, 16, 16)
+    voxels, coors, npv = vox(torch.from_numpy(pts).cuda())
+    V = voxels.shape[0]
+    c = coors.cpu().numpy()
+    assert V == len({tuple(r) for r in c.tolist()}) and (c >= 0).all() and (c < np.array(space)).all()
+    assert int(npv.sum().item()) <= 4000 and int(npv.min().item()) >= 1
+    feats = spnn.mean_voxel_features(voxels, npv)
+    st = spnn.sparse_tensor_from_voxels(feats, coors, space)
+    torch.manual_seed(5)
+    layer = spnn.SubMConv3d(4, 16, 3).cuda()
+    y = layer(st).features.detach().cpu().double()
+    dense = torch.zeros((1, 4) + space, dtype=torch.float64)
+    ci = torch.from_numpy(c.astype(np.int64))
+    dense[0, :, ci[:, 0], ci[:, 1], ci[:, 2]] = feats.cpu().double().t()
+    w = layer.weight.detach().cpu().double().permute(4, 3, 0, 1, 2)
+    ref = F.conv3d(dense, w, padding=1)[0][:, ci[:, 0], ci[:, 1], ci[:, 2]].t()
+    d1 = (y - ref).abs().sum() / ref.abs().sum()
+    assert d1 <= 1e-5, float(d1)
