@@ -451,6 +451,55 @@ mluOpVoxelization(mluOpHandle_t handle,
                   const mluOpTensorDescriptor_t voxel_num_desc,
                   void *voxel_num);
 
+/* ---------------------------------------------------------------------------
+ * Dynamic point-to-voxel scatter (forward): the other upstream step, which groups
+ * points by their voxel coordinate and reduces their features.
+ * ------------------------------------------------------------------------- */
+
+/* reference mlu_op.h:361-365 */
+typedef enum {
+  MLUOP_REDUCE_DSUM  = 0, /* not accepted by mluOpDynamicPointToVoxelForward */
+  MLUOP_REDUCE_DMEAN = 1,
+  MLUOP_REDUCE_DMAX  = 2,
+} mluOpReduceMode_t;
+
+/* reference mlu_op.h:3767-3771 (kernels/dynamic_point_to_voxel/
+ * dynamic_point_to_voxel_forward/dynamic_point_to_voxel_forward.cpp:195-232). */
+mluOpStatus_t MLUOP_WIN_API
+mluOpGetDynamicPointToVoxelForwardWorkspaceSize(mluOpHandle_t handle,
+                                                const mluOpTensorDescriptor_t feats_desc,
+                                                const mluOpTensorDescriptor_t coors_desc,
+                                                size_t *workspace_size);
+
+/* reference mlu_op.h:3865-3883 (same file :234-380).  feats [N, C] float, coors
+ * [N, 3] int32 (rows with a negative coordinate are rewritten to -1,-1,-1 in
+ * place and belong to no voxel).  Outputs with M <= N rows: voxel_feats [M, C]
+ * (max or mean over the points of a voxel; rows past voxel_num hold -inf for
+ * max and 0 for mean), voxel_coors [M, 3] (distinct triples in ascending
+ * order), point2voxel_map [N] (voxel of every point, -1 for none),
+ * voxel_points_count [M], voxel_num [1].  reduce_type: MLUOP_REDUCE_DMAX or
+ * MLUOP_REDUCE_DMEAN (BAD_PARAM otherwise).  The call synchronises the stream
+ * once (it reads the largest coordinate back to size its sorts). */
+mluOpStatus_t MLUOP_WIN_API
+mluOpDynamicPointToVoxelForward(const mluOpHandle_t handle,
+                                const mluOpReduceMode_t reduce_type,
+                                const mluOpTensorDescriptor_t feats_desc,
+                                const void *feats,
+                                const mluOpTensorDescriptor_t coors_desc,
+                                void *coors,
+                                void *workspace,
+                                const size_t workspace_size,
+                                const mluOpTensorDescriptor_t voxel_feats_desc,
+                                void *voxel_feats,
+                                const mluOpTensorDescriptor_t voxel_coors_desc,
+                                void *voxel_coors,
+                                const mluOpTensorDescriptor_t point2voxel_map_desc,
+                                void *point2voxel_map,
+                                const mluOpTensorDescriptor_t voxel_points_count_desc,
+                                void *voxel_points_count,
+                                const mluOpTensorDescriptor_t voxel_num_desc,
+                                void *voxel_num);
+
 #if defined(__cplusplus)
 }
 #endif

@@ -1,0 +1,310 @@
+// Dynamic point-to-voxel scatter, forward: points that share a coordinate
+// triple form a voxel; voxels are numbered in ascending (lexicographic) order
+// of their triples; the features of a voxel's points are reduced by max or
+// mean.  The reference delegates the grouping to a vendor "unique" routine
+// (kernels/dynamic_point_to_voxel/dynamic_point_to_voxel_forward/
+//  dynamic_point_to_voxel_forward.cpp:300-340) and reduces with atomics.
+//
+// Here:
+//   1 dpvPrepare   rows with a negative coordinate become (-1,-1,-1) in place;
+//                  the largest coordinate of every axis is collected so that
+//                  the sorts run over as few bits as the data needs
+//   2 three stable radix sorts of (coordinate + 1, point index), last axis
+//                  first: the points end up in ascending triple order, equal
+//                  triples in point order
+//   3 dpvHeads + inclusive scan: number of the triple each sorted point has
+//   4 dpvEmit      point2voxel_map, voxel_coors, first sorted position of
+//                  every voxel, voxel_num
+//   5 dpvReduce    one thread per (voxel, feature) walks the voxel's points in
+//                  point order: max, or the sum of feats / count in exactly
+//                  the order the sequential definition adds them, so the mean
+//                  has the same bits on every run
+#include <hip/hip_runtime.h>
+#include <cstring>
+
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
+
+#include "dynamic_point_to_voxel/scatter_points.h"
+
+namespace mluop {
+namespace dynamic_point_to_voxel {
+namespace {
+
+constexpr int kBlock = 256;
+
+inline int gridFor(size_t n, int cap = 1 << 20) {
+  size_t b = (n + kBlock - 1) / kBlock;
+  if (b < 1) b = 1;
+  return (int)(b > (size_t)cap ? (size_t)cap : b);
+}
+
+size_t alignUp(size_t v) { return (v + 255) & ~(size_t)255; }
+
+__global__ __launch_bounds__(kBlock) void dpvFill(float *voxel_feats, size_t feat_words,
+                                                  float fill, int32_t *voxel_coors,
+                                                  int32_t *voxel_points_count, int rows,
+                                                  int32_t *axis_max) {
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  for (size_t i = t; i < feat_words; i += stride) voxel_feats[i] = fill;
+  for (size_t i = t; i < (size_t)rows * 3; i += stride) voxel_coors[i] = 0;
+  for (size_t i = t; i < (size_t)rows; i += stride) voxel_points_count[i] = 0;
+  if (t < 3) axis_max[t] = -1;
+}
+
+__global__ __launch_bounds__(kBlock) void dpvPrepare(int32_t *coors, int n, uint32_t *keys,
+                                                     uint32_t *points, int32_t *axis_max) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  int c0 = -1, c1 = -1, c2 = -1;
+  if (i < n) {
+    c0 = coors[3 * (size_t)i];
+    c1 = coors[3 * (size_t)i + 1];
+    c2 = coors[3 * (size_t)i + 2];
+    if (c0 < 0 || c1 < 0 || c2 < 0) {
+      c0 = c1 = c2 = -1;
+      coors[3 * (size_t)i] = -1;
+      coors[3 * (size_t)i + 1] = -1;
+      coors[3 * (size_t)i + 2] = -1;
+    }
+    keys[i] = (uint32_t)(c2 + 1);  // the last axis is sorted first
+    points[i] = (uint32_t)i;
+  }
+  // block maxima, then one atomic per axis and block
+  __shared__ int s_max[3][kBlock / 64];
+  int m0 = c0, m1 = c1, m2 = c2;
+  for (int off = 32; off > 0; off >>= 1) {
+    m0 = max(m0, __shfl_xor(m0, off, 64));
+    m1 = max(m1, __shfl_xor(m1, off, 64));
+    m2 = max(m2, __shfl_xor(m2, off, 64));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_max[0][threadIdx.x >> 6] = m0;
+    s_max[1][threadIdx.x >> 6] = m1;
+    s_max[2][threadIdx.x >> 6] = m2;
+  }
+  __syncthreads();
+  if (threadIdx.x < 3) {
+    int m = s_max[threadIdx.x][0];
+    for (int w = 1; w < kBlock / 64; ++w) m = max(m, s_max[threadIdx.x][w]);
+    if (m >= 0) atomicMax(&axis_max[threadIdx.x], m);
+  }
+}
+
+// keys[p] = coordinate `axis` of the point at sorted position p, plus one
+__global__ __launch_bounds__(kBlock) void dpvGatherKeys(const int32_t *__restrict__ coors,
+                                                        const uint32_t *__restrict__ points, int n,
+                                                        int axis, uint32_t *keys) {
+  const int p = blockIdx.x * kBlock + threadIdx.x;
+  if (p < n) keys[p] = (uint32_t)(coors[3 * (size_t)points[p] + axis] + 1);
+}
+
+__global__ __launch_bounds__(kBlock) void dpvHeads(const int32_t *__restrict__ coors,
+                                                   const uint32_t *__restrict__ points, int n,
+                                                   uint32_t *head) {
+  const int p = blockIdx.x * kBlock + threadIdx.x;
+  if (p >= n) return;
+  if (p == 0) {
+    head[0] = 1;
+    return;
+  }
+  const int32_t *a = coors + 3 * (size_t)points[p];
+  const int32_t *b = coors + 3 * (size_t)points[p - 1];
+  head[p] = (a[0] != b[0] || a[1] != b[1] || a[2] != b[2]) ? 1u : 0u;
+}
+
+__global__ __launch_bounds__(kBlock) void dpvEmit(const int32_t *__restrict__ coors,
+                                                  const uint32_t *__restrict__ points,
+                                                  const uint32_t *__restrict__ head,
+                                                  const uint32_t *__restrict__ triple_count, int n,
+                                                  int rows, int32_t *point2voxel_map,
+                                                  int32_t *voxel_coors, int32_t *first_pos,
+                                                  int32_t *voxel_num) {
+  const int p = blockIdx.x * kBlock + threadIdx.x;
+  if (p >= n) return;
+  // the (-1,-1,-1) triple sorts first and is not a voxel
+  const int skipped = coors[3 * (size_t)points[0]] == -1 ? 1 : 0;
+  const int v = (int)triple_count[p] - 1 - skipped;
+  const uint32_t i = points[p];
+  point2voxel_map[i] = v;
+  if (head[p] && v >= 0 && v <= rows) {
+    first_pos[v] = p;  // one past the last stored voxel included: it ends that voxel
+    if (v < rows) {
+      voxel_coors[3 * (size_t)v] = coors[3 * (size_t)i];
+      voxel_coors[3 * (size_t)v + 1] = coors[3 * (size_t)i + 1];
+      voxel_coors[3 * (size_t)v + 2] = coors[3 * (size_t)i + 2];
+    }
+  }
+  if (p == n - 1) *voxel_num = v + 1;
+}
+
+__global__ __launch_bounds__(kBlock) void dpvReduce(const float *__restrict__ feats,
+                                                    const uint32_t *__restrict__ points,
+                                                    const int32_t *__restrict__ first_pos,
+                                                    const int32_t *__restrict__ voxel_num, int n,
+                                                    int num_features, int rows, bool reduce_max,
+                                                    float *voxel_feats,
+                                                    int32_t *voxel_points_count) {
+  const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  const int voxels = min(*voxel_num, rows);
+  if (t >= (size_t)voxels * num_features) return;
+  const int v = (int)(t / num_features);
+  const int f = (int)(t % num_features);
+  const int begin = first_pos[v];
+  // dpvEmit stores the first position of voxel `rows` too, when there is one
+  const int stop = v + 1 < *voxel_num ? first_pos[v + 1] : n;
+  const int count = stop - begin;
+  if (f == 0) voxel_points_count[v] = count;
+  if (reduce_max) {
+    float best = -INFINITY;
+    for (int p = begin; p < stop; ++p) {
+      const float x = feats[(size_t)points[p] * num_features + f];
+      if (x >= best) best = x;
+    }
+    voxel_feats[t] = best;
+  } else {
+    float sum = 0.f;
+    const float fcount = (float)count;
+    for (int p = begin; p < stop; ++p)
+      sum = __fadd_rn(sum, __fdiv_rn(feats[(size_t)points[p] * num_features + f], fcount));
+    voxel_feats[t] = sum;
+  }
+}
+
+struct Workspace {
+  uint32_t *keys_a, *keys_b, *points_a, *points_b, *head, *triple_count;
+  int32_t *first_pos, *axis_max;
+  void *library;
+  size_t total;
+};
+
+Workspace carve(void *base, const ScatterShape &s, size_t library_bytes) {
+  const size_t n = (size_t)s.num_points;
+  char *p = static_cast<char *>(base);
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    char *q = p + off;
+    off += alignUp(bytes);
+    return q;
+  };
+  Workspace w;
+  w.keys_a = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.keys_b = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.points_a = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.points_b = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.head = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.triple_count = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.first_pos = reinterpret_cast<int32_t *>(take(4 * (n + 1)));
+  w.axis_max = reinterpret_cast<int32_t *>(take(16));
+  w.library = take(library_bytes);
+  w.total = off;
+  return w;
+}
+
+int bitsFor(int32_t max_coordinate) {  // keys are coordinate + 1, 0 for the -1 triple
+  const uint32_t top = (uint32_t)(max_coordinate + 1);
+  int b = 1;
+  while (b < 32 && (top >> b) != 0) ++b;
+  return b;
+}
+
+}  // namespace
+
+size_t scatterWorkspaceBytes(const ScatterShape &s, size_t library_bytes) {
+  return carve(nullptr, s, library_bytes).total;
+}
+
+hipError_t libraryWorkspaceBytes(const ScatterShape &s, hipStream_t stream, size_t *bytes) {
+  size_t sort_bytes = 0, scan_bytes = 0;
+  uint32_t *u = nullptr;
+  hipError_t e = rocprim::radix_sort_pairs(nullptr, sort_bytes, u, u, u, u, (size_t)s.num_points, 0,
+                                           32, stream);
+  if (e != hipSuccess) return e;
+  e = rocprim::inclusive_scan(nullptr, scan_bytes, u, u, (size_t)s.num_points,
+                              rocprim::plus<uint32_t>(), stream);
+  if (e != hipSuccess) return e;
+  *bytes = sort_bytes > scan_bytes ? sort_bytes : scan_bytes;
+  return hipSuccess;
+}
+
+hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const float *feats,
+                               int32_t *coors, void *workspace, size_t workspace_bytes,
+                               int32_t *pinned_host, float *voxel_feats, int32_t *voxel_coors,
+                               int32_t *point2voxel_map, int32_t *voxel_points_count,
+                               int32_t *voxel_num) {
+  const int n = s.num_points;
+  size_t library_bytes = 0;
+  hipError_t e = libraryWorkspaceBytes(s, lc.stream, &library_bytes);
+  if (e != hipSuccess) return e;
+  const Workspace w = carve(workspace, s, library_bytes);
+  if (w.total > workspace_bytes) return hipErrorInvalidValue;
+  const int blocks = gridFor((size_t)n);
+
+  const size_t feat_words = (size_t)s.voxel_rows * s.num_features;
+  lc.begin("dpvFill");
+  dpvFill<<<gridFor(feat_words > (size_t)n ? feat_words : (size_t)n, 4096), kBlock, 0, lc.stream>>>(
+      voxel_feats, feat_words, s.reduce_max ? -INFINITY : 0.f, voxel_coors, voxel_points_count,
+      s.voxel_rows, w.axis_max);
+  lc.end();
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+
+  lc.begin("dpvPrepare");
+  dpvPrepare<<<blocks, kBlock, 0, lc.stream>>>(coors, n, w.keys_a, w.points_a, w.axis_max);
+  lc.end();
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+  e = hipMemcpyAsync(pinned_host, w.axis_max, 3 * sizeof(int32_t), hipMemcpyDeviceToHost,
+                     lc.stream);
+  if (e != hipSuccess) return e;
+  if ((e = hipStreamSynchronize(lc.stream)) != hipSuccess) return e;
+  const int bits[3] = {bitsFor(pinned_host[0]), bitsFor(pinned_host[1]), bitsFor(pinned_host[2])};
+
+  // last axis first; every pass is stable, so the final order is lexicographic
+  // with equal triples in point order
+  uint32_t *pts_in = w.points_a, *pts_out = w.points_b;
+  for (int axis = 2; axis >= 0; --axis) {
+    if (axis != 2) {
+      lc.begin("dpvGatherKeys");
+      dpvGatherKeys<<<blocks, kBlock, 0, lc.stream>>>(coors, pts_in, n, axis, w.keys_a);
+      lc.end();
+      if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
+    lc.begin("radixSortPairs");
+    size_t lib = library_bytes;
+    e = rocprim::radix_sort_pairs(w.library, lib, w.keys_a, w.keys_b, pts_in, pts_out, (size_t)n,
+                                  0, bits[axis], lc.stream);
+    lc.end();
+    if (e != hipSuccess) return e;
+    uint32_t *t = pts_in;
+    pts_in = pts_out;
+    pts_out = t;
+  }
+  const uint32_t *sorted_points = pts_in;
+
+  lc.begin("dpvHeads");
+  dpvHeads<<<blocks, kBlock, 0, lc.stream>>>(coors, sorted_points, n, w.head);
+  lc.end();
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+  lc.begin("inclusiveScan");
+  size_t lib = library_bytes;
+  e = rocprim::inclusive_scan(w.library, lib, w.head, w.triple_count, (size_t)n,
+                              rocprim::plus<uint32_t>(), lc.stream);
+  lc.end();
+  if (e != hipSuccess) return e;
+
+  lc.begin("dpvEmit");
+  dpvEmit<<<blocks, kBlock, 0, lc.stream>>>(coors, sorted_points, w.head, w.triple_count, n,
+                                             s.voxel_rows, point2voxel_map, voxel_coors,
+                                             w.first_pos, voxel_num);
+  lc.end();
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+
+  lc.begin("dpvReduce");
+  dpvReduce<<<gridFor(feat_words), kBlock, 0, lc.stream>>>(
+      feats, sorted_points, w.first_pos, voxel_num, n, s.num_features, s.voxel_rows, s.reduce_max,
+      voxel_feats, voxel_points_count);
+  lc.end();
+  return hipGetLastError();
+}
+
+}  // namespace dynamic_point_to_voxel
+}  // namespace mluop

@@ -41,6 +41,7 @@ DTYPE_UINT32, DTYPE_UINT64, DTYPE_UINT16, DTYPE_DOUBLE = 11, 12, 13, 14
 DTYPE_COMPLEX_HALF, DTYPE_COMPLEX_FLOAT, DTYPE_BFLOAT16 = 15, 16, 17
 
 ATOMICS_NOT_ALLOWED, ATOMICS_ALLOWED = 1, 2
+REDUCE_DSUM, REDUCE_DMEAN, REDUCE_DMAX = 0, 1, 2
 POINTER_MODE_HOST, POINTER_MODE_DEVICE = 0, 1
 
 _vp = ctypes.c_void_p
@@ -108,6 +109,10 @@ SIGNATURES = {
     "mluOpVoxelization": (
         ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
                        ctypes.c_bool, _vp, ctypes.c_size_t, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "mluOpGetDynamicPointToVoxelForwardWorkspaceSize": (ctypes.c_int, [_vp, _vp, _vp, _szp]),
+    "mluOpDynamicPointToVoxelForward": (
+        ctypes.c_int, [_vp, ctypes.c_int, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t, _vp, _vp, _vp, _vp,
+                       _vp, _vp, _vp, _vp, _vp, _vp]),
     # mlu_op_ext.h
     "mluOpExtSetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int]),
     "mluOpExtGetKernelTimingCount": (ctypes.c_int, [_vp, _ip]),
@@ -430,3 +435,39 @@ def voxelization(handle, points, voxel_size, coors_range, max_points, max_voxels
         d_voxels.ptr, voxels.data_ptr(), d_coors.ptr, coors.data_ptr(), d_npv.ptr, npv.data_ptr(), d_num.ptr,
         voxel_num.data_ptr()), "mluOpVoxelization")
     return voxels, coors, npv, voxel_num
+
+
+def dynamic_point_to_voxel_forward(handle, feats, coors, reduce_type="max", rows=None):
+    """Groups points by coordinate triple and reduces their features ("max" or "mean").
+
+    feats [N, C] float32 and coors [N, 3] int32 are device tensors; coors is modified in place
+    (rows with a negative coordinate become -1,-1,-1).  Returns (voxel_feats [rows, C], voxel_coors
+    [rows, 3], point2voxel_map [N], voxel_points_count [rows], voxel_num [1]); rows defaults to N."""
+    torch = _torch()
+    n, c = feats.shape
+    m = n if rows is None else int(rows)
+    dev = feats.device
+    voxel_feats = torch.empty((m, c), dtype=torch.float32, device=dev)
+    voxel_coors = torch.empty((m, 3), dtype=torch.int32, device=dev)
+    p2v = torch.empty((n,), dtype=torch.int32, device=dev)
+    count = torch.empty((m,), dtype=torch.int32, device=dev)
+    voxel_num = torch.zeros((1,), dtype=torch.int32, device=dev)
+    mode = {"max": REDUCE_DMAX, "mean": REDUCE_DMEAN, "sum": REDUCE_DSUM}[reduce_type]
+    d_feats = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
+    d_coors = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [n, 3])
+    d_vf = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [m, c])
+    d_vc = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [m, 3])
+    d_p2v = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [n])
+    d_cnt = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [m])
+    d_num = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [1])
+    size = ctypes.c_size_t(0)
+    check(lib().mluOpGetDynamicPointToVoxelForwardWorkspaceSize(handle.ptr, d_feats.ptr, d_coors.ptr,
+                                                                ctypes.byref(size)),
+          "mluOpGetDynamicPointToVoxelForwardWorkspaceSize")
+    ws = _workspace(size.value, dev)
+    check(lib().mluOpDynamicPointToVoxelForward(
+        handle.ptr, mode, d_feats.ptr, feats.data_ptr(), d_coors.ptr, coors.data_ptr(), ws.data_ptr(),
+        size.value, d_vf.ptr, voxel_feats.data_ptr(), d_vc.ptr, voxel_coors.data_ptr(), d_p2v.ptr,
+        p2v.data_ptr(), d_cnt.ptr, count.data_ptr(), d_num.ptr, voxel_num.data_ptr()),
+        "mluOpDynamicPointToVoxelForward")
+    return voxel_feats, voxel_coors, p2v, count, voxel_num

@@ -230,7 +230,16 @@ class CaseTensor:
             if msg.has(field):
                 vals = np.array(msg.all(field), dtype=np.int64)
                 assert vals.size == n, "%s: %d values for %d elements" % (self.id, vals.size, n)
-                return (vals.astype(np.int32) if int_like else vals.astype(np.float32)).reshape(self.shape)
+                if int_like:
+                    return vals.astype(np.int32).reshape(self.shape)
+                # value_i of a floating tensor holds the elements' bit patterns (parser.cpp:568-578)
+                if self.dtype_name == "float32":
+                    out = vals.astype(np.int32).view(np.float32)
+                elif self.dtype_name == "float16":
+                    out = vals.astype(np.int16).view(np.float16).astype(np.float32)
+                else:
+                    out = bf16_bits_to_f32(vals.astype(np.int16).view(np.uint16))
+                return out.reshape(self.shape)
         if msg.has("value_f"):
             vals = np.array(msg.all("value_f"), dtype=np.float32)
             assert vals.size == n
@@ -429,6 +438,16 @@ def diff2(got, want):
 _ERROR_FUNCS = {"DIFF1": diff1, "DIFF2": diff2}
 
 
+def criteria(node):
+    """(error function names, thresholds): `test_param`, or the older node-level
+    `evaluation_criterion` / `evaluation_threshold` fields (parser.cpp:129-196)."""
+    tp = node.get("test_param")
+    if tp is not None and tp.has("error_func"):
+        return [str(f) for f in tp.all("error_func")], [float(t) for t in tp.all("error_threshold")]
+    return ([str(f) for f in node.all("evaluation_criterion")],
+            [float(t) for t in node.all("evaluation_threshold")])
+
+
 class Replay:
     """Outputs of one replayed case: `outputs` (name -> numpy array), `errors` (list of
     (output name, error_func, value, threshold)) and `passed`."""
@@ -508,9 +527,7 @@ def replay(path_or_text, handle):
     else:
         raise ValueError("case file names operator %r: only the sparse-convolution operators are built" % op)
 
-    tp = node.get("test_param", Message())
-    funcs = [str(f) for f in tp.all("error_func")]
-    thresholds = [float(t) for t in tp.all("error_threshold")]
+    funcs, thresholds = criteria(node)
     for t in outs:
         if t.values is None:
             continue

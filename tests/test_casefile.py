@@ -73,6 +73,23 @@ def test_value_kinds_decode(tmp_path):
         cf.CaseTensor(cf.parse("shape { dims: 3 } dtype: DTYPE_INT32 value_i: 1"))
 
 
+def test_value_i_of_float_tensors_holds_bit_patterns():
+    """The reference's own case files store float tensors as value_i bit patterns."""
+    cf = casefile()
+    node, _ = cf.load(os.path.join(GOLDEN, "dynamic_point_to_voxel_forward", "case_0.prototxt"))
+    assert node.get("op_name") == "dynamic_point_to_voxel_forward" and node.get("device") == "CPU"
+    feats = cf.CaseTensor(node.all("input")[0])
+    assert feats.values.shape == (6, 6) and feats.values.dtype == np.float32
+    assert np.all(np.abs(feats.values) <= 100.0)             # drawn from U(-100, 100)
+    assert feats.values[0, 0] == np.array([-1031791637], np.int32).view(np.float32)[0]
+    coors = cf.CaseTensor(node.all("input")[1])
+    assert coors.values.dtype == np.int32 and coors.values[3].tolist() == [-1, 18, 7]
+    assert cf.criteria(node) == (["DIFF1", "DIFF2"], [0.003, 0.003])
+    assert node.get("dynamic_point_to_voxel_forward_param").get("reduce_type") == "REDUCE_MODE_MEAN"
+    half = cf.CaseTensor(cf.parse("shape { dims: 2 } dtype: DTYPE_HALF value_i: 15360 value_i: -16384"))
+    assert half.values.tolist() == [1.0, -2.0]
+
+
 def test_bf16_rounding_matches_the_oracle():
     cf = casefile()
     x = np.random.default_rng(0).standard_normal(4096).astype(np.float32)

@@ -1,0 +1,105 @@
+"""mluOpDynamicPointToVoxelForward through the C ABI: the two case files the reference ships
+(replayed from their own values), the CPU oracle bit for bit (max and mean: the kernel adds
+feats / count in point order, as the sequential definition does), and a full-size cloud."""
+import os
+
+import numpy as np
+import pytest
+
+import dynamic_point_to_voxel_oracle as dpv
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "dynamic_point_to_voxel_forward")
+
+
+def run_gpu(handle, mode, feats, coors, rows=None):
+    import torch
+    import mluop_hip
+    c = torch.from_numpy(np.ascontiguousarray(coors, dtype=np.int32)).cuda()
+    out = mluop_hip.dynamic_point_to_voxel_forward(handle, torch.from_numpy(feats).cuda(), c, mode, rows)
+    torch.cuda.synchronize()
+    return [t.cpu().numpy() for t in out[:4]] + [int(out[4].item()), c.cpu().numpy()]
+
+
+def assert_same(got, want):
+    names = ("voxel_feats", "voxel_coors", "point2voxel_map", "voxel_points_count", "voxel_num", "coors")
+    for g, w, name in zip(got, want, names):
+        assert np.array_equal(g, w), name
+
+
+@pytest.mark.parametrize("name", ["case_0.prototxt", "case_1.prototxt"])
+def test_reference_case_files(gpu_handle, name):
+    from mluop_hip import casefile as cf
+    node, _ = cf.load(os.path.join(GOLDEN, name))
+    ins = [cf.CaseTensor(t) for t in node.all("input")]
+    outs = [cf.CaseTensor(t) for t in node.all("output")]
+    mode = {"REDUCE_MODE_MAX": "max", "REDUCE_MODE_MEAN": "mean"}[
+        str(node.get("dynamic_point_to_voxel_forward_param").get("reduce_type"))]
+    got = run_gpu(gpu_handle, mode, ins[0].values, ins[1].values, rows=outs[0].shape[0])
+    num = int(outs[4].values[0])
+    assert got[4] == num
+    assert np.array_equal(got[2], outs[2].values)
+    assert np.array_equal(got[1][:num], outs[1].values[:num])
+    assert np.array_equal(got[3][:num], outs[3].values[:num])
+    funcs, thresholds = cf.criteria(node)
+    for f, thr in zip(funcs, thresholds):
+        err = {"DIFF1": cf.diff1, "DIFF2": cf.diff2}[f](got[0][:num], outs[0].values[:num])
+        assert err <= min(thr, 1e-6), (f, err)
+
+
+CASES = [(1, 1, 1, 1, 0.0), (2, 50, 3, 3, 0.1), (3, 5000, 5, 6, 0.05), (4, 5000, 4, 40, 0.0), (5, 300, 1, 2, 0.5),
+         (6, 20000, 9, 12, 0.02)]
+
+
+@pytest.mark.parametrize("mode", ["max", "mean"])
+@pytest.mark.parametrize("case", CASES)
+def test_matches_oracle(gpu_handle, mode, case):
+    seed, n, c, span, neg = case
+    print("dynamic_point_to_voxel case", case, mode, flush=True)
+    rng = np.random.default_rng(seed)
+    feats = rng.uniform(-100, 100, (n, c)).astype(np.float32)
+    coors = rng.integers(0, span, (n, 3)).astype(np.int32)
+    k = int(n * neg)
+    if k:
+        coors[rng.choice(n, k, replace=False), rng.integers(0, 3, k)] = -rng.integers(1, 5, k)
+    assert_same(run_gpu(gpu_handle, mode, feats, coors), dpv.forward(mode, feats, coors))
+
+
+def test_fewer_output_rows_than_voxels_and_all_invalid(gpu_handle):
+    rng = np.random.default_rng(7)
+    feats = rng.uniform(-1, 1, (400, 3)).astype(np.float32)
+    coors = rng.integers(0, 5, (400, 3)).astype(np.int32)
+    for mode in ("max", "mean"):
+        assert_same(run_gpu(gpu_handle, mode, feats, coors, rows=20), dpv.forward(mode, feats, coors, rows=20))
+    bad = -np.ones((64, 3), np.int32)
+    got = run_gpu(gpu_handle, "mean", feats[:64], bad)
+    assert got[4] == 0 and (got[2] == -1).all() and not got[0].any()
+
+
+def test_large_coordinates(gpu_handle):
+    """Coordinates up to 2^31 - 1 need all 32 key bits."""
+    rng = np.random.default_rng(8)
+    feats = rng.uniform(-1, 1, (3000, 2)).astype(np.float32)
+    coors = rng.choice(np.array([0, 1, 70000, 2 ** 31 - 1], dtype=np.int64), size=(3000, 3)).astype(np.int32)
+    assert_same(run_gpu(gpu_handle, "max", feats, coors), dpv.forward("max", feats, coors))
+
+
+def test_full_size_cloud(gpu_handle):
+    rng = np.random.default_rng(9)
+    n = 1000000
+    feats = rng.uniform(-100, 100, (n, 4)).astype(np.float32)
+    coors = np.stack([rng.integers(0, 40, n), rng.integers(0, 1600, n), rng.integers(0, 1408, n)], axis=1).astype(
+        np.int32)
+    coors[rng.choice(n, n // 20, replace=False), 0] = -1
+    for mode in ("max", "mean"):
+        assert_same(run_gpu(gpu_handle, mode, feats, coors), dpv.forward(mode, feats, coors))
+
+
+def test_statuses(gpu_handle):
+    import torch
+    import mluop_hip
+    feats = torch.zeros((8, 2), device="cuda")
+    coors = torch.zeros((8, 3), dtype=torch.int32, device="cuda")
+    with pytest.raises(mluop_hip.MluOpError) as e:
+        mluop_hip.dynamic_point_to_voxel_forward(gpu_handle, feats, coors, "sum")
+    assert e.value.status == mluop_hip.STATUS_BAD_PARAM
