@@ -23,6 +23,9 @@ OPS = {
         "indice_convolution_backward_data/indice_convolution_backward_data_general.cpp",
     "indice_convolution_backward_filter":
         "indice_convolution_backward_filter/indice_convolution_backward_filter_general.cpp",
+    "voxelization": "voxelization/voxelization_general.cpp",
+    "dynamic_point_to_voxel_forward":
+        "dynamic_point_to_voxel_forward/dynamic_point_to_voxel_forward_general.cpp",
 }
 
 TOKEN = re.compile(r"\s*([A-Za-z_][A-Za-z_0-9:<> ]*[A-Za-z_0-9>]|[A-Za-z_]|-?\d+|[(){},])")
@@ -121,6 +124,9 @@ def main():
                 assert values["call"] == "testing::Values"
                 axes.append([simplify(a) for a in values["args"]])
             for idx, combo in enumerate(itertools.product(*axes)):
+                last = combo[-1]
+                if isinstance(last, list) and len(last) == 2 and str(last[1]).startswith("MLUOP_STATUS"):
+                    combo = tuple(combo[:-1]) + (last[0], last[1])  # PublicParam{device, status}
                 cases.append({"name": "%s/%d" % (name, idx), "params": list(combo[:-2]),
                               "device": combo[-2], "expected": combo[-1]})
         out[op] = {"source": "test/mlu_op_gtest/api_gtest/src/gtest/" + rel, "cases": cases}

@@ -268,6 +268,87 @@ def test_indice_convolution_backward_filter_null_arguments(handle):
 
 # --- descriptors, handle, exports ------------------------------------------------------------------
 
+REDUCE = {"MLUOP_REDUCE_DSUM": 0, "MLUOP_REDUCE_DMEAN": 1, "MLUOP_REDUCE_DMAX": 2}
+
+
+@pytest.mark.parametrize("case", cases("voxelization"))
+def test_voxelization_table(handle, case):
+    """api_gtest/src/gtest/voxelization/voxelization_general.cpp: workspace query, then the operator."""
+    lib = m.lib()
+    p_points, p_vs, p_cr, (max_points, max_voxels, ndim, det), p_vox, p_coors, p_npv, p_num = case["params"]
+    descs = [make_desc(p) for p in (p_points, p_vs, p_cr, p_vox, p_coors, p_npv, p_num)]
+    det = det in ("true", 1, True)
+    try:
+        size = ctypes.c_size_t(0)
+        st = lib.mluOpGetVoxelizationWorkspaceSize(handle.ptr, descs[0], descs[1], descs[2], max_points,
+                                                   max_voxels, ndim, det, descs[3], descs[4], descs[5], descs[6],
+                                                   ctypes.byref(size))
+        if st != 0:
+            assert st == STATUS[case["expected"]]
+            return
+        st = lib.mluOpVoxelization(handle.ptr, descs[0], FAKE, descs[1], FAKE, descs[2], FAKE, max_points,
+                                   max_voxels, ndim, det, FAKE, size.value, descs[3], FAKE, descs[4], FAKE,
+                                   descs[5], FAKE, descs[6], FAKE)
+        assert st in launch_ok(case["expected"])
+    finally:
+        free_descs(*descs)
+
+
+@pytest.mark.parametrize("case", cases("dynamic_point_to_voxel_forward"))
+def test_dynamic_point_to_voxel_forward_table(handle, case):
+    """api_gtest/src/gtest/dynamic_point_to_voxel_forward/dynamic_point_to_voxel_forward_general.cpp."""
+    lib = m.lib()
+    *tensors, reduce_type = case["params"]
+    descs = [make_desc(p) for p in tensors]
+    try:
+        st = lib.mluOpDynamicPointToVoxelForward(handle.ptr, REDUCE[reduce_type], descs[0], FAKE, descs[1], FAKE,
+                                                 FAKE, 1 << 30, descs[2], FAKE, descs[3], FAKE, descs[4], FAKE,
+                                                 descs[5], FAKE, descs[6], FAKE)
+        assert st in launch_ok(case["expected"])
+    finally:
+        free_descs(*descs)
+
+
+def test_voxelization_null_arguments(handle):
+    """api_gtest/src/gtest/voxelization/voxelization.cpp:255-413 and voxelization_workspace.cpp:162-242."""
+    lib = m.lib()
+    f, i = "MLUOP_DTYPE_FLOAT", "MLUOP_DTYPE_INT32"
+    descs = [make_desc(T("MLUOP_LAYOUT_ARRAY", dt, d)) for dt, d in
+             ((f, [20, 4]), (f, [3]), (f, [6]), (f, [5, 3, 4]), (i, [5, 3]), (i, [5]), (i, [1]))]
+    size = ctypes.c_size_t(0)
+    ws_args = [handle.ptr, descs[0], descs[1], descs[2], 3, 5, 3, True, descs[3], descs[4], descs[5], descs[6],
+               ctypes.byref(size)]
+    null_sweep(lib.mluOpGetVoxelizationWorkspaceSize, ws_args, [0, 1, 2, 3, 8, 9, 10, 11, 12])
+    assert lib.mluOpGetVoxelizationWorkspaceSize(*ws_args) == 0 and size.value > 0
+    args = [handle.ptr, descs[0], FAKE, descs[1], FAKE, descs[2], FAKE, 3, 5, 3, True, FAKE, size.value, descs[3],
+            FAKE, descs[4], FAKE, descs[5], FAKE, descs[6], FAKE]
+    null_sweep(lib.mluOpVoxelization, args, [0, 1, 2, 3, 4, 5, 6, 11, 13, 14, 15, 16, 17, 18, 19, 20])
+    assert lib.mluOpVoxelization(*args) == STATUS["MLUOP_STATUS_EXECUTION_FAILED"]  # host-only handle
+    args[10] = False        # non-deterministic mode does not exist (voxelization.cpp:166-170)
+    assert lib.mluOpVoxelization(*args) == STATUS["MLUOP_STATUS_BAD_PARAM"]
+    free_descs(*descs)
+
+
+def test_dynamic_point_to_voxel_forward_null_arguments(handle):
+    """api_gtest/src/gtest/dynamic_point_to_voxel_forward/dynamic_point_to_voxel_forward.cpp:326-500 and
+    dynamic_point_to_voxel_forward_workspace.cpp:101-140."""
+    lib = m.lib()
+    f, i = "MLUOP_DTYPE_FLOAT", "MLUOP_DTYPE_INT32"
+    descs = [make_desc(T("MLUOP_LAYOUT_ARRAY", dt, d)) for dt, d in
+             ((f, [20, 4]), (i, [20, 3]), (f, [20, 4]), (i, [20, 3]), (i, [20]), (i, [20]), (i, [1]))]
+    size = ctypes.c_size_t(0)
+    ws_args = [handle.ptr, descs[0], descs[1], ctypes.byref(size)]
+    null_sweep(lib.mluOpGetDynamicPointToVoxelForwardWorkspaceSize, ws_args, range(4))
+    assert lib.mluOpGetDynamicPointToVoxelForwardWorkspaceSize(*ws_args) == 0 and size.value > 0
+    args = [handle.ptr, REDUCE["MLUOP_REDUCE_DMAX"], descs[0], FAKE, descs[1], FAKE, FAKE, size.value, descs[2],
+            FAKE, descs[3], FAKE, descs[4], FAKE, descs[5], FAKE, descs[6], FAKE]
+    null_sweep(lib.mluOpDynamicPointToVoxelForward, args, [0, 2, 3, 4, 5, 6, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17])
+    assert lib.mluOpDynamicPointToVoxelForward(*args) == STATUS["MLUOP_STATUS_EXECUTION_FAILED"]
+    args[1] = REDUCE["MLUOP_REDUCE_DSUM"]
+    assert lib.mluOpDynamicPointToVoxelForward(*args) == STATUS["MLUOP_STATUS_BAD_PARAM"]
+    free_descs(*descs)
+
+
 def test_sparse_conv_descriptor_status_codes():
     """get_indice_pairs_structs.cpp:31-134: NULL create -> NOT_INITIALIZED, NULL destroy -> EXECUTION_FAILED."""
     lib = m.lib()
