@@ -150,3 +150,16 @@ def test_config3_regular_rulebook_full_size(gpu_handle):
     import mluop_hip
     idx = mluop_hip.datagen.clustered_voxels((4, 41, 1600, 1408), 30000, seed=3)
     compare(gpu_handle, idx, 4, (41, 1600, 1408), (3, 3, 3), [1, 1, 1], [2, 2, 2], [1, 1, 1], False)
+
+
+@pytest.mark.timeout(600)
+def test_largest_accepted_input_one_million_rows(gpu_handle):
+    """L = 1 000 000, the most rows the API accepts (INDICE_IN_LARGE_TENSOR_NUM), submanifold and
+    regular stride 2, in a grid of 2 x 48 x 512 x 512 cells (density 4 %)."""
+    rng = np.random.default_rng(77)
+    space = (48, 512, 512)
+    idx = random_voxels(rng, 2, space, 1000000)
+    print("subm 1M", flush=True)
+    compare(gpu_handle, idx, 2, space, (3, 3, 3), [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+    print("regular 1M", flush=True)
+    compare(gpu_handle, idx, 2, space, (2, 2, 2), [0, 0, 0], [2, 2, 2], [1, 1, 1], False)
