@@ -225,12 +225,78 @@ def measured_traffic(workload, kernel):
         return None
 
 
+UPSTREAM = {
+    # the operators in front of the sparse convolutions: 1.2 M points on a 1408 x 1600 x 40 grid
+    "voxelization": "hard voxelization, 1 200 000 points (4 features), voxel 0.05 x 0.05 x 0.1 in "
+                    "[0,70.4]x[-40,40]x[-3,1], max_points 5, max_voxels 150000",
+    "dynamic_point_to_voxel": "dynamic point-to-voxel scatter (mean), 1 000 000 points (4 features), "
+                              "coordinates in 40 x 1600 x 1408, 5 % invalid",
+}
+
+
+def run_upstream(args, torch, m, handle):
+    """Times one of the upstream operators (not the headline metric): prints its own JSON line."""
+    import numpy as np
+    rng = np.random.default_rng(10)
+    if args.workload == "voxelization":
+        n = 1200000
+        pts = np.empty((n, 4), np.float32)
+        pts[:, 0] = rng.uniform(0.0, 70.4, n)
+        pts[:, 1] = rng.uniform(-40.0, 40.0, n)
+        pts[:, 2] = rng.uniform(-3.0, 1.0, n)
+        pts[:, 3] = rng.uniform(0.0, 1.0, n)
+        far = rng.choice(n, n // 20, replace=False)
+        pts[far, :3] += 200.0
+        points = torch.from_numpy(pts).cuda()
+        vs = torch.tensor([0.05, 0.05, 0.1], device="cuda")
+        cr = torch.tensor([0.0, -40.0, -3.0, 70.4, 40.0, 1.0], device="cuda")
+        op = lambda: m.voxelization(handle, points, vs, cr, 5, 150000)
+        # points read, voxels/coors/counts zero-filled and written
+        algorithmic = n * 16 + 150000 * (5 * 16 + 12 + 4) * 2
+    else:
+        n = 1000000
+        feats = torch.from_numpy(rng.uniform(-100, 100, (n, 4)).astype(np.float32)).cuda()
+        c = np.stack([rng.integers(0, 40, n), rng.integers(0, 1600, n), rng.integers(0, 1408, n)], axis=1)
+        c[rng.choice(n, n // 20, replace=False), 0] = -1
+        coors = torch.from_numpy(c.astype(np.int32)).cuda()
+        op = lambda: m.dynamic_point_to_voxel_forward(handle, feats, coors, "mean")
+        # feats + coors read; per-point map and (at most N) voxel rows written
+        algorithmic = n * (16 + 12 + 4) + n * (16 + 12 + 4)
+    for _ in range(args.warmup):
+        op()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        op()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    result = {"metric": args.workload + " Mpoints/s", "value": n / (ms * 1e-3) / 1e6, "unit": "Mpoints/s",
+              "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+              "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32/int32",
+              "data": "synthetic", "config": {"workload": UPSTREAM[args.workload], "points": n}}
+    if not args.only_step:
+        handle.set_kernel_timing(True)
+        op()
+        torch.cuda.synchronize()
+        agg = {}
+        for name, t in handle.kernel_timings():
+            agg[name] = agg.get(name, 0.0) + t * 1e3
+        handle.set_kernel_timing(False)
+        result["kernels_us_per_call"] = agg
+        result["roofline"] = {"bound": "hbm", "achieved": algorithmic / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                              "unit": "GB/s", "frac": algorithmic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                              "traffic": None, "kernel": "whole operator", "algorithmic_bytes": algorithmic}
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="config4", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="config4", choices=sorted(WORKLOADS) + sorted(UPSTREAM))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only-step", action="store_true",
                     help="run just warmup + timed steps (for profiler runs)")
@@ -250,6 +316,9 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     handle = m.make_handle_on_current_stream()
+    if args.workload in UPSTREAM:
+        run_upstream(args, torch, m, handle)
+        return
     wl = WORKLOADS[args.workload]
     step = Step(handle, wl)
     step_ops = [("get_indice_pairs", step.rulebook), ("forward", step.forward)]

@@ -9,9 +9,11 @@
 //   1 dpvPrepare   rows with a negative coordinate become (-1,-1,-1) in place;
 //                  the largest coordinate of every axis is collected so that
 //                  the sorts run over as few bits as the data needs
-//   2 three stable radix sorts of (coordinate + 1, point index), last axis
-//                  first: the points end up in ascending triple order, equal
-//                  triples in point order
+//   2 one stable radix sort of (packed triple, point index) when the three
+//                  coordinates (+1) fit 64 bits together, which they do up to
+//                  2^21 cells per axis; otherwise three stable sorts, last
+//                  axis first.  Either way the points end up in ascending
+//                  triple order, equal triples in point order
 //   3 dpvHeads + inclusive scan: number of the triple each sorted point has
 //   4 dpvEmit      point2voxel_map, voxel_coors, first sorted position of
 //                  every voxel, voxel_num
@@ -55,24 +57,26 @@ __global__ __launch_bounds__(kBlock) void dpvFill(float *voxel_feats, size_t fea
 
 __global__ __launch_bounds__(kBlock) void dpvPrepare(int32_t *coors, int n, uint32_t *keys,
                                                      uint32_t *points, int32_t *axis_max) {
-  const int i = blockIdx.x * kBlock + threadIdx.x;
-  int c0 = -1, c1 = -1, c2 = -1;
-  if (i < n) {
-    c0 = coors[3 * (size_t)i];
-    c1 = coors[3 * (size_t)i + 1];
-    c2 = coors[3 * (size_t)i + 2];
+  // grid-stride: a few hundred blocks, so that the three atomics per block stay cheap
+  int m0 = -1, m1 = -1, m2 = -1;
+  for (int i = blockIdx.x * kBlock + threadIdx.x; i < n; i += gridDim.x * kBlock) {
+    int c0 = coors[3 * (size_t)i];
+    int c1 = coors[3 * (size_t)i + 1];
+    int c2 = coors[3 * (size_t)i + 2];
     if (c0 < 0 || c1 < 0 || c2 < 0) {
       c0 = c1 = c2 = -1;
       coors[3 * (size_t)i] = -1;
       coors[3 * (size_t)i + 1] = -1;
       coors[3 * (size_t)i + 2] = -1;
     }
-    keys[i] = (uint32_t)(c2 + 1);  // the last axis is sorted first
+    keys[i] = (uint32_t)(c2 + 1);  // the last axis is sorted first (three-sort path)
     points[i] = (uint32_t)i;
+    m0 = max(m0, c0);
+    m1 = max(m1, c1);
+    m2 = max(m2, c2);
   }
   // block maxima, then one atomic per axis and block
   __shared__ int s_max[3][kBlock / 64];
-  int m0 = c0, m1 = c1, m2 = c2;
   for (int off = 32; off > 0; off >>= 1) {
     m0 = max(m0, __shfl_xor(m0, off, 64));
     m1 = max(m1, __shfl_xor(m1, off, 64));
@@ -91,12 +95,33 @@ __global__ __launch_bounds__(kBlock) void dpvPrepare(int32_t *coors, int n, uint
   }
 }
 
+// key = (c0+1, c1+1, c2+1) packed most significant first; rows are already masked
+template <typename KeyT>
+__global__ __launch_bounds__(kBlock) void dpvPackKeys(const int32_t *__restrict__ coors, int n,
+                                                      int bits1, int bits2, KeyT *keys) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const KeyT k0 = (KeyT)(uint32_t)(coors[3 * (size_t)i] + 1);
+  const KeyT k1 = (KeyT)(uint32_t)(coors[3 * (size_t)i + 1] + 1);
+  const KeyT k2 = (KeyT)(uint32_t)(coors[3 * (size_t)i + 2] + 1);
+  keys[i] = (k0 << (bits1 + bits2)) | (k1 << bits2) | k2;
+}
+
 // keys[p] = coordinate `axis` of the point at sorted position p, plus one
 __global__ __launch_bounds__(kBlock) void dpvGatherKeys(const int32_t *__restrict__ coors,
                                                         const uint32_t *__restrict__ points, int n,
                                                         int axis, uint32_t *keys) {
   const int p = blockIdx.x * kBlock + threadIdx.x;
   if (p < n) keys[p] = (uint32_t)(coors[3 * (size_t)points[p] + axis] + 1);
+}
+
+// head[p] = 1 where the sorted packed key changes
+template <typename KeyT>
+__global__ __launch_bounds__(kBlock) void dpvHeadsFromKeys(const KeyT *__restrict__ sorted_keys,
+                                                           int n, uint32_t *head) {
+  const int p = blockIdx.x * kBlock + threadIdx.x;
+  if (p >= n) return;
+  head[p] = (p == 0 || sorted_keys[p] != sorted_keys[p - 1]) ? 1u : 0u;
 }
 
 __global__ __launch_bounds__(kBlock) void dpvHeads(const int32_t *__restrict__ coors,
@@ -188,8 +213,8 @@ Workspace carve(void *base, const ScatterShape &s, size_t library_bytes) {
     return q;
   };
   Workspace w;
-  w.keys_a = reinterpret_cast<uint32_t *>(take(4 * n));
-  w.keys_b = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.keys_a = reinterpret_cast<uint32_t *>(take(8 * n));  // 64-bit packed keys at most
+  w.keys_b = reinterpret_cast<uint32_t *>(take(8 * n));
   w.points_a = reinterpret_cast<uint32_t *>(take(4 * n));
   w.points_b = reinterpret_cast<uint32_t *>(take(4 * n));
   w.head = reinterpret_cast<uint32_t *>(take(4 * n));
@@ -220,9 +245,15 @@ hipError_t libraryWorkspaceBytes(const ScatterShape &s, hipStream_t stream, size
   hipError_t e = rocprim::radix_sort_pairs(nullptr, sort_bytes, u, u, u, u, (size_t)s.num_points, 0,
                                            32, stream);
   if (e != hipSuccess) return e;
+  size_t sort64_bytes = 0;
+  unsigned long long *u64 = nullptr;
+  e = rocprim::radix_sort_pairs(nullptr, sort64_bytes, u64, u64, u, u, (size_t)s.num_points, 0, 64,
+                                stream);
+  if (e != hipSuccess) return e;
   e = rocprim::inclusive_scan(nullptr, scan_bytes, u, u, (size_t)s.num_points,
                               rocprim::plus<uint32_t>(), stream);
   if (e != hipSuccess) return e;
+  sort_bytes = sort_bytes > sort64_bytes ? sort_bytes : sort64_bytes;
   *bytes = sort_bytes > scan_bytes ? sort_bytes : scan_bytes;
   return hipSuccess;
 }
@@ -249,7 +280,8 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
   if ((e = hipGetLastError()) != hipSuccess) return e;
 
   lc.begin("dpvPrepare");
-  dpvPrepare<<<blocks, kBlock, 0, lc.stream>>>(coors, n, w.keys_a, w.points_a, w.axis_max);
+  dpvPrepare<<<gridFor((size_t)n, 512), kBlock, 0, lc.stream>>>(coors, n, w.keys_a, w.points_a,
+                                                                w.axis_max);
   lc.end();
   if ((e = hipGetLastError()) != hipSuccess) return e;
   e = hipMemcpyAsync(pinned_host, w.axis_max, 3 * sizeof(int32_t), hipMemcpyDeviceToHost,
@@ -258,32 +290,72 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
   if ((e = hipStreamSynchronize(lc.stream)) != hipSuccess) return e;
   const int bits[3] = {bitsFor(pinned_host[0]), bitsFor(pinned_host[1]), bitsFor(pinned_host[2])};
 
-  // last axis first; every pass is stable, so the final order is lexicographic
-  // with equal triples in point order
   uint32_t *pts_in = w.points_a, *pts_out = w.points_b;
-  for (int axis = 2; axis >= 0; --axis) {
-    if (axis != 2) {
-      lc.begin("dpvGatherKeys");
-      dpvGatherKeys<<<blocks, kBlock, 0, lc.stream>>>(coors, pts_in, n, axis, w.keys_a);
+  bool packed = false;
+  const int total_bits = bits[0] + bits[1] + bits[2];
+  if (total_bits <= 64) {
+    size_t lib = library_bytes;
+    if (total_bits <= 32) {
+      lc.begin("dpvPackKeys");
+      dpvPackKeys<uint32_t><<<blocks, kBlock, 0, lc.stream>>>(coors, n, bits[1], bits[2], w.keys_a);
       lc.end();
       if ((e = hipGetLastError()) != hipSuccess) return e;
+      lc.begin("radixSortPairs");
+      e = rocprim::radix_sort_pairs(w.library, lib, w.keys_a, w.keys_b, pts_in, pts_out, (size_t)n,
+                                    0, total_bits, lc.stream);
+      lc.end();
+      if (e != hipSuccess) return e;
+      lc.begin("dpvHeads");
+      dpvHeadsFromKeys<uint32_t><<<blocks, kBlock, 0, lc.stream>>>(w.keys_b, n, w.head);
+      lc.end();
+    } else {
+      unsigned long long *ka = reinterpret_cast<unsigned long long *>(w.keys_a);
+      unsigned long long *kb = reinterpret_cast<unsigned long long *>(w.keys_b);
+      lc.begin("dpvPackKeys");
+      dpvPackKeys<unsigned long long><<<blocks, kBlock, 0, lc.stream>>>(coors, n, bits[1], bits[2], ka);
+      lc.end();
+      if ((e = hipGetLastError()) != hipSuccess) return e;
+      lc.begin("radixSortPairs");
+      e = rocprim::radix_sort_pairs(w.library, lib, ka, kb, pts_in, pts_out, (size_t)n, 0,
+                                    total_bits, lc.stream);
+      lc.end();
+      if (e != hipSuccess) return e;
+      lc.begin("dpvHeads");
+      dpvHeadsFromKeys<unsigned long long><<<blocks, kBlock, 0, lc.stream>>>(kb, n, w.head);
+      lc.end();
     }
-    lc.begin("radixSortPairs");
-    size_t lib = library_bytes;
-    e = rocprim::radix_sort_pairs(w.library, lib, w.keys_a, w.keys_b, pts_in, pts_out, (size_t)n,
-                                  0, bits[axis], lc.stream);
-    lc.end();
-    if (e != hipSuccess) return e;
-    uint32_t *t = pts_in;
+    if ((e = hipGetLastError()) != hipSuccess) return e;
     pts_in = pts_out;
-    pts_out = t;
+    packed = true;
+  } else {
+    // last axis first; every pass is stable, so the final order is lexicographic
+    // with equal triples in point order
+    for (int axis = 2; axis >= 0; --axis) {
+      if (axis != 2) {
+        lc.begin("dpvGatherKeys");
+        dpvGatherKeys<<<blocks, kBlock, 0, lc.stream>>>(coors, pts_in, n, axis, w.keys_a);
+        lc.end();
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+      }
+      lc.begin("radixSortPairs");
+      size_t lib = library_bytes;
+      e = rocprim::radix_sort_pairs(w.library, lib, w.keys_a, w.keys_b, pts_in, pts_out, (size_t)n,
+                                    0, bits[axis], lc.stream);
+      lc.end();
+      if (e != hipSuccess) return e;
+      uint32_t *t = pts_in;
+      pts_in = pts_out;
+      pts_out = t;
+    }
   }
   const uint32_t *sorted_points = pts_in;
 
-  lc.begin("dpvHeads");
-  dpvHeads<<<blocks, kBlock, 0, lc.stream>>>(coors, sorted_points, n, w.head);
-  lc.end();
-  if ((e = hipGetLastError()) != hipSuccess) return e;
+  if (!packed) {
+    lc.begin("dpvHeads");
+    dpvHeads<<<blocks, kBlock, 0, lc.stream>>>(coors, sorted_points, n, w.head);
+    lc.end();
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+  }
   lc.begin("inclusiveScan");
   size_t lib = library_bytes;
   e = rocprim::inclusive_scan(w.library, lib, w.head, w.triple_count, (size_t)n,

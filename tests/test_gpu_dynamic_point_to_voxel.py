@@ -77,11 +77,14 @@ def test_fewer_output_rows_than_voxels_and_all_invalid(gpu_handle):
 
 
 def test_large_coordinates(gpu_handle):
-    """Coordinates up to 2^31 - 1 need all 32 key bits."""
+    """The three key widths: triples packed in 32 bits, in 64 bits (17 bits per axis), and three
+    separate sorts (coordinates up to 2^31 - 1 need all 32 key bits each)."""
     rng = np.random.default_rng(8)
     feats = rng.uniform(-1, 1, (3000, 2)).astype(np.float32)
-    coors = rng.choice(np.array([0, 1, 70000, 2 ** 31 - 1], dtype=np.int64), size=(3000, 3)).astype(np.int32)
-    assert_same(run_gpu(gpu_handle, "max", feats, coors), dpv.forward("max", feats, coors))
+    for values in ([0, 1, 2, 900], [0, 1, 70000], [0, 1, 70000, 2 ** 31 - 1]):
+        coors = rng.choice(np.array(values, dtype=np.int64), size=(3000, 3)).astype(np.int32)
+        coors[::50, 1] = -7
+        assert_same(run_gpu(gpu_handle, "max", feats, coors), dpv.forward("max", feats, coors))
 
 
 def test_full_size_cloud(gpu_handle):
