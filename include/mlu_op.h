@@ -500,6 +500,44 @@ mluOpDynamicPointToVoxelForward(const mluOpHandle_t handle,
                                 const mluOpTensorDescriptor_t voxel_num_desc,
                                 void *voxel_num);
 
+/* reference mlu_op.h:3750 region, mluOpGetDynamicPointToVoxelBackwardWorkspaceSize
+ * (kernels/dynamic_point_to_voxel/dynamic_point_to_voxel_backward/
+ * dynamic_point_to_voxel_backward.cpp:336-364): N * C ints. */
+mluOpStatus_t MLUOP_WIN_API
+mluOpGetDynamicPointToVoxelBackwardWorkspaceSize(const mluOpHandle_t handle,
+                                                 const mluOpReduceMode_t reduce_type,
+                                                 const mluOpTensorDescriptor_t grad_voxel_feats_desc,
+                                                 const mluOpTensorDescriptor_t feats_desc,
+                                                 const mluOpTensorDescriptor_t voxel_feats_desc,
+                                                 const mluOpTensorDescriptor_t point2voxel_map_desc,
+                                                 const mluOpTensorDescriptor_t voxel_points_count_desc,
+                                                 const mluOpTensorDescriptor_t voxel_num_desc,
+                                                 size_t *workspace_size);
+
+/* reference mlu_op.h:3707-3725 (same file :177-334).  Gradient of the max
+ * reduction (MLUOP_REDUCE_DMAX only, BAD_PARAM otherwise): grad_feats [N, C] is
+ * zero except that, for every voxel and feature, the first point whose feature
+ * equals the voxel's maximum receives grad_voxel_feats[voxel, feature]. */
+mluOpStatus_t MLUOP_WIN_API
+mluOpDynamicPointToVoxelBackward(const mluOpHandle_t handle,
+                                 const mluOpReduceMode_t reduce_type,
+                                 const mluOpTensorDescriptor_t grad_voxel_feats_desc,
+                                 const void *grad_voxel_feats,
+                                 const mluOpTensorDescriptor_t feats_desc,
+                                 const void *feats,
+                                 const mluOpTensorDescriptor_t voxel_feats_desc,
+                                 const void *voxel_feats,
+                                 const mluOpTensorDescriptor_t point2voxel_map_desc,
+                                 const void *point2voxel_map,
+                                 const mluOpTensorDescriptor_t voxel_points_count_desc,
+                                 const void *voxel_points_count,
+                                 const mluOpTensorDescriptor_t voxel_num_desc,
+                                 const void *voxel_num,
+                                 void *workspace,
+                                 const size_t workspace_size,
+                                 const mluOpTensorDescriptor_t grad_feats_desc,
+                                 void *grad_feats);
+
 #if defined(__cplusplus)
 }
 #endif

@@ -33,6 +33,13 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
                                int32_t *point2voxel_map, int32_t *voxel_points_count,
                                int32_t *voxel_num);
 
+// Backward of the max reduction: `from` is [voxel_rows, num_features] ints of workspace.
+hipError_t launchScatterPointsBackward(const LaunchCtx &lc, int num_points, int num_features,
+                                       int voxel_rows, const float *grad_voxel_feats,
+                                       const float *feats, const float *voxel_feats,
+                                       const int32_t *point2voxel_map, const int32_t *voxel_num,
+                                       int32_t *from, float *grad_feats);
+
 }  // namespace dynamic_point_to_voxel
 }  // namespace mluop
 

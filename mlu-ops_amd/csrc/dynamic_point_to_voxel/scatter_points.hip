@@ -196,6 +196,41 @@ __global__ __launch_bounds__(kBlock) void dpvReduce(const float *__restrict__ fe
   }
 }
 
+// ---- backward of the max reduction ----
+
+__global__ __launch_bounds__(kBlock) void dpvBackwardInit(float *grad_feats, size_t grad_words,
+                                                          int32_t *from, size_t from_words,
+                                                          int32_t none) {
+  const size_t stride = (size_t)gridDim.x * kBlock;
+  const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  for (size_t i = t; i < grad_words; i += stride) grad_feats[i] = 0.f;
+  for (size_t i = t; i < from_words; i += stride) from[i] = none;
+}
+
+// from[v, c] = lowest point index whose feature equals the voxel's maximum
+__global__ __launch_bounds__(kBlock) void dpvBackwardFindSource(
+    const float *__restrict__ feats, const float *__restrict__ voxel_feats,
+    const int32_t *__restrict__ point2voxel_map, int n, int num_features, int rows, int32_t *from) {
+  const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (t >= (size_t)n * num_features) return;
+  const int x = (int)(t / num_features);
+  const int c = (int)(t % num_features);
+  const int v = point2voxel_map[x];
+  if (v < 0 || v >= rows) return;
+  if (feats[t] == voxel_feats[(size_t)v * num_features + c])
+    atomicMin(&from[(size_t)v * num_features + c], x);
+}
+
+__global__ __launch_bounds__(kBlock) void dpvBackwardScatter(
+    const float *__restrict__ grad_voxel_feats, const int32_t *__restrict__ from,
+    const int32_t *__restrict__ voxel_num, int n, int num_features, int rows, float *grad_feats) {
+  const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  const int voxels = min(*voxel_num, rows);
+  if (t >= (size_t)voxels * num_features) return;
+  const int x = from[t];
+  if (x < n) grad_feats[(size_t)x * num_features + t % num_features] = grad_voxel_feats[t];
+}
+
 struct Workspace {
   uint32_t *keys_a, *keys_b, *points_a, *points_b, *head, *triple_count;
   int32_t *first_pos, *axis_max;
@@ -374,6 +409,31 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
   dpvReduce<<<gridFor(feat_words), kBlock, 0, lc.stream>>>(
       feats, sorted_points, w.first_pos, voxel_num, n, s.num_features, s.voxel_rows, s.reduce_max,
       voxel_feats, voxel_points_count);
+  lc.end();
+  return hipGetLastError();
+}
+
+hipError_t launchScatterPointsBackward(const LaunchCtx &lc, int num_points, int num_features,
+                                       int voxel_rows, const float *grad_voxel_feats,
+                                       const float *feats, const float *voxel_feats,
+                                       const int32_t *point2voxel_map, const int32_t *voxel_num,
+                                       int32_t *from, float *grad_feats) {
+  const size_t grad_words = (size_t)num_points * num_features;
+  const size_t from_words = (size_t)voxel_rows * num_features;
+  lc.begin("dpvBackwardInit");
+  dpvBackwardInit<<<gridFor(grad_words, 4096), kBlock, 0, lc.stream>>>(grad_feats, grad_words, from,
+                                                                       from_words, num_points);
+  lc.end();
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || from_words == 0) return e;
+  lc.begin("dpvBackwardFindSource");
+  dpvBackwardFindSource<<<gridFor(grad_words), kBlock, 0, lc.stream>>>(
+      feats, voxel_feats, point2voxel_map, num_points, num_features, voxel_rows, from);
+  lc.end();
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+  lc.begin("dpvBackwardScatter");
+  dpvBackwardScatter<<<gridFor(from_words), kBlock, 0, lc.stream>>>(
+      grad_voxel_feats, from, voxel_num, num_points, num_features, voxel_rows, grad_feats);
   lc.end();
   return hipGetLastError();
 }

@@ -113,6 +113,11 @@ SIGNATURES = {
     "mluOpDynamicPointToVoxelForward": (
         ctypes.c_int, [_vp, ctypes.c_int, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t, _vp, _vp, _vp, _vp,
                        _vp, _vp, _vp, _vp, _vp, _vp]),
+    "mluOpGetDynamicPointToVoxelBackwardWorkspaceSize": (
+        ctypes.c_int, [_vp, ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _szp]),
+    "mluOpDynamicPointToVoxelBackward": (
+        ctypes.c_int, [_vp, ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                       ctypes.c_size_t, _vp, _vp]),
     # mlu_op_ext.h
     "mluOpExtSetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int]),
     "mluOpExtGetKernelTimingCount": (ctypes.c_int, [_vp, _ip]),
@@ -471,3 +476,31 @@ def dynamic_point_to_voxel_forward(handle, feats, coors, reduce_type="max", rows
         p2v.data_ptr(), d_cnt.ptr, count.data_ptr(), d_num.ptr, voxel_num.data_ptr()),
         "mluOpDynamicPointToVoxelForward")
     return voxel_feats, voxel_coors, p2v, count, voxel_num
+
+
+def dynamic_point_to_voxel_backward(handle, grad_voxel_feats, feats, voxel_feats, point2voxel_map,
+                                    voxel_points_count, voxel_num, reduce_type="max"):
+    """Gradient of `dynamic_point_to_voxel_forward(..., "max")` with respect to feats: [N, C]."""
+    torch = _torch()
+    n, c = feats.shape
+    m = grad_voxel_feats.shape[0]
+    grad_feats = torch.empty((n, c), dtype=torch.float32, device=feats.device)
+    mode = {"max": REDUCE_DMAX, "mean": REDUCE_DMEAN, "sum": REDUCE_DSUM}[reduce_type]
+    d_g = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [m, c])
+    d_feats = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
+    d_vf = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [m, c])
+    d_p2v = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [n])
+    d_cnt = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [m])
+    d_num = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [1])
+    d_out = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
+    size = ctypes.c_size_t(0)
+    check(lib().mluOpGetDynamicPointToVoxelBackwardWorkspaceSize(
+        handle.ptr, mode, d_g.ptr, d_feats.ptr, d_vf.ptr, d_p2v.ptr, d_cnt.ptr, d_num.ptr, ctypes.byref(size)),
+        "mluOpGetDynamicPointToVoxelBackwardWorkspaceSize")
+    ws = _workspace(size.value, feats.device)
+    check(lib().mluOpDynamicPointToVoxelBackward(
+        handle.ptr, mode, d_g.ptr, grad_voxel_feats.data_ptr(), d_feats.ptr, feats.data_ptr(), d_vf.ptr,
+        voxel_feats.data_ptr(), d_p2v.ptr, point2voxel_map.data_ptr(), d_cnt.ptr,
+        voxel_points_count.data_ptr(), d_num.ptr, voxel_num.data_ptr(), ws.data_ptr(), size.value, d_out.ptr,
+        grad_feats.data_ptr()), "mluOpDynamicPointToVoxelBackward")
+    return grad_feats

@@ -19,6 +19,13 @@
  * files the reference ships for this operator (tests/golden/
  * dynamic_point_to_voxel_forward/case_0.prototxt, case_1.prototxt) and an
  * independent numpy.unique formulation.
+ *
+ * oracle_dynamic_point_to_voxel_backward restates the backward executor
+ * (test/mlu_op_gtest/pb_gtest/src/zoo/dynamic_point_to_voxel_backward/
+ *  dynamic_point_to_voxel_backward.cpp:108-166, max reduction only) and is
+ * pinned by the reference's case file for it (tests/golden/
+ * dynamic_point_to_voxel_backward/case_1.prototxt) and by round trips through
+ * the forward oracle.
  */
 #include <math.h>
 #include <stdint.h>
@@ -94,5 +101,38 @@ int32_t oracle_dynamic_point_to_voxel_forward(int32_t reduce_max, const float *f
       for (int32_t j = 0; j < c; ++j) dst[j] += src[j] / count;
     }
   }
+  return 0;
+}
+
+/* The gradient of a voxel's maximum goes to the first point (lowest index) whose
+ * feature equals it; everything else is zero.  A (voxel, feature) no point of
+ * which matches gives its gradient to nobody: the operator's scatter drops the
+ * out-of-range index it leaves there
+ * (kernels/dynamic_point_to_voxel/dynamic_point_to_voxel_backward/
+ *  dynamic_point_to_voxel_backward.cpp:272-330), where the gtest body would write
+ * past the end of grad_feats.  voxel rows: `m` in the tensors, `voxel_num` used. */
+int32_t oracle_dynamic_point_to_voxel_backward(const float *grad_voxel_feats, const float *feats,
+                                               const float *voxel_feats,
+                                               const int32_t *point2voxel_map, int32_t voxel_num,
+                                               int32_t n, int32_t c, int32_t m, float *grad_feats) {
+  memset(grad_feats, 0, sizeof(float) * (size_t)n * c);
+  if (voxel_num > m) voxel_num = m;
+  if (n == 0 || c == 0 || voxel_num <= 0) return 0;
+  int32_t *from = (int32_t *)malloc(sizeof(int32_t) * (size_t)voxel_num * c);
+  if (!from) return -1;
+  for (size_t i = 0; i < (size_t)voxel_num * c; ++i) from[i] = n;
+  for (int32_t x = 0; x < n; ++x) {
+    const int32_t v = point2voxel_map[x];
+    if (v < 0 || v >= voxel_num) continue;
+    for (int32_t j = 0; j < c; ++j)
+      if (feats[(size_t)x * c + j] == voxel_feats[(size_t)v * c + j] && x < from[(size_t)v * c + j])
+        from[(size_t)v * c + j] = x;
+  }
+  for (int32_t v = 0; v < voxel_num; ++v)
+    for (int32_t j = 0; j < c; ++j) {
+      const int32_t x = from[(size_t)v * c + j];
+      if (x < n) grad_feats[(size_t)x * c + j] = grad_voxel_feats[(size_t)v * c + j];
+    }
+  free(from);
   return 0;
 }

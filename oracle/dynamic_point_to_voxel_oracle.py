@@ -20,6 +20,7 @@ def lib():
             subprocess.check_call(["make", "-C", _HERE, "-s"])
         _lib = ctypes.CDLL(_LIB_PATH)
         _lib.oracle_dynamic_point_to_voxel_forward.restype = ctypes.c_int32
+        _lib.oracle_dynamic_point_to_voxel_backward.restype = ctypes.c_int32
     return _lib
 
 
@@ -44,3 +45,20 @@ def forward(reduce_type, feats, coors, rows=None):
     if rc != 0:
         raise MemoryError("oracle_dynamic_point_to_voxel_forward")
     return vf, vc, p2v, cnt, int(num[0]), coors
+
+
+def backward(grad_voxel_feats, feats, voxel_feats, point2voxel_map, voxel_num):
+    """Gradient of the max reduction with respect to feats: [N, C]."""
+    g = np.ascontiguousarray(grad_voxel_feats, dtype=np.float32)
+    feats = np.ascontiguousarray(feats, dtype=np.float32)
+    vf = np.ascontiguousarray(voxel_feats, dtype=np.float32)
+    p2v = np.ascontiguousarray(point2voxel_map, dtype=np.int32)
+    n, c = feats.shape
+    out = np.empty((n, c), np.float32)
+    rc = lib().oracle_dynamic_point_to_voxel_backward(
+        g.ctypes.data_as(_f32p), feats.ctypes.data_as(_f32p), vf.ctypes.data_as(_f32p),
+        p2v.ctypes.data_as(_i32p), ctypes.c_int32(int(voxel_num)), ctypes.c_int32(n), ctypes.c_int32(c),
+        ctypes.c_int32(g.shape[0]), out.ctypes.data_as(_f32p))
+    if rc != 0:
+        raise MemoryError("oracle_dynamic_point_to_voxel_backward")
+    return out

@@ -26,6 +26,8 @@ OPS = {
     "voxelization": "voxelization/voxelization_general.cpp",
     "dynamic_point_to_voxel_forward":
         "dynamic_point_to_voxel_forward/dynamic_point_to_voxel_forward_general.cpp",
+    "dynamic_point_to_voxel_backward":
+        "dynamic_point_to_voxel_backward/dynamic_point_to_voxel_backward_general.cpp",
 }
 
 TOKEN = re.compile(r"\s*([A-Za-z_][A-Za-z_0-9:<> ]*[A-Za-z_0-9>]|[A-Za-z_]|-?\d+|[(){},])")

@@ -309,6 +309,40 @@ def test_dynamic_point_to_voxel_forward_table(handle, case):
         free_descs(*descs)
 
 
+@pytest.mark.parametrize("case", cases("dynamic_point_to_voxel_backward"))
+def test_dynamic_point_to_voxel_backward_table(handle, case):
+    """api_gtest/src/gtest/dynamic_point_to_voxel_backward/dynamic_point_to_voxel_backward_general.cpp."""
+    lib = m.lib()
+    reduce_type, *tensors = case["params"]
+    descs = [make_desc(p) for p in tensors]
+    try:
+        st = lib.mluOpDynamicPointToVoxelBackward(handle.ptr, REDUCE[reduce_type], descs[0], FAKE, descs[1], FAKE,
+                                                  descs[2], FAKE, descs[3], FAKE, descs[4], FAKE, descs[5], FAKE,
+                                                  FAKE, 1 << 30, descs[6], FAKE)
+        assert st in launch_ok(case["expected"])
+    finally:
+        free_descs(*descs)
+
+
+def test_dynamic_point_to_voxel_backward_null_arguments(handle):
+    """api_gtest/src/gtest/dynamic_point_to_voxel_backward/dynamic_point_to_voxel_backward.cpp and
+    dynamic_point_to_voxel_backward_workspace.cpp: one NULL argument at a time."""
+    lib = m.lib()
+    f, i = "MLUOP_DTYPE_FLOAT", "MLUOP_DTYPE_INT32"
+    descs = [make_desc(T("MLUOP_LAYOUT_ARRAY", dt, d)) for dt, d in
+             ((f, [4, 3]), (f, [6, 3]), (f, [4, 3]), (i, [6]), (i, [4]), (i, [1]), (f, [6, 3]))]
+    size = ctypes.c_size_t(0)
+    mx = REDUCE["MLUOP_REDUCE_DMAX"]
+    ws_args = [handle.ptr, mx, descs[0], descs[1], descs[2], descs[3], descs[4], descs[5], ctypes.byref(size)]
+    null_sweep(lib.mluOpGetDynamicPointToVoxelBackwardWorkspaceSize, ws_args, [0, 2, 3, 4, 5, 6, 7, 8])
+    assert lib.mluOpGetDynamicPointToVoxelBackwardWorkspaceSize(*ws_args) == 0 and size.value == 6 * 3 * 4
+    args = [handle.ptr, mx, descs[0], FAKE, descs[1], FAKE, descs[2], FAKE, descs[3], FAKE, descs[4], FAKE,
+            descs[5], FAKE, FAKE, size.value, descs[6], FAKE]
+    null_sweep(lib.mluOpDynamicPointToVoxelBackward, args, [0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 16, 17])
+    assert lib.mluOpDynamicPointToVoxelBackward(*args) == STATUS["MLUOP_STATUS_EXECUTION_FAILED"]
+    free_descs(*descs)
+
+
 def test_voxelization_null_arguments(handle):
     """api_gtest/src/gtest/voxelization/voxelization.cpp:255-413 and voxelization_workspace.cpp:162-242."""
     lib = m.lib()

@@ -106,3 +106,56 @@ def test_statuses(gpu_handle):
     with pytest.raises(mluop_hip.MluOpError) as e:
         mluop_hip.dynamic_point_to_voxel_forward(gpu_handle, feats, coors, "sum")
     assert e.value.status == mluop_hip.STATUS_BAD_PARAM
+
+
+def backward_case_inputs(cf, node):
+    """The case file stores grad_voxel_feats [34, 5] with the 150 values of its 30 real voxels only:
+    the rows past voxel_num are padded with zeros here."""
+    msgs = node.all("input")
+    bits = np.array(msgs[0].all("value_i"), dtype=np.int64).astype(np.int32).view(np.float32)
+    grad = np.zeros((34, 5), np.float32)
+    grad.reshape(-1)[:bits.size] = bits
+    return [grad] + [cf.CaseTensor(t).values for t in msgs[1:]]
+
+
+def test_backward_reference_case_file(gpu_handle):
+    import torch
+    import mluop_hip
+    from mluop_hip import casefile as cf
+    node, _ = cf.load(os.path.join(os.path.dirname(GOLDEN), "dynamic_point_to_voxel_backward", "case_1.prototxt"))
+    ins = backward_case_inputs(cf, node)
+    want = cf.CaseTensor(node.all("output")[0]).values
+    dev = [torch.from_numpy(np.ascontiguousarray(t)).cuda() for t in ins]
+    got = mluop_hip.dynamic_point_to_voxel_backward(gpu_handle, *dev)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("case", [(1, 200, 4, 3), (2, 5000, 6, 8), (3, 500, 1, 2), (4, 300000, 5, 30)])
+def test_backward_matches_oracle_after_gpu_forward(gpu_handle, case):
+    """Forward (max) and backward chained on the GPU; ties everywhere (integer features)."""
+    import torch
+    import mluop_hip
+    seed, n, c, span = case
+    print("dynamic_point_to_voxel backward case", case, flush=True)
+    rng = np.random.default_rng(seed)
+    feats = rng.integers(-3, 4, (n, c)).astype(np.float32)
+    coors = rng.integers(0, span, (n, 3)).astype(np.int32)
+    coors[rng.choice(n, n // 10, replace=False), 0] = -1
+    g = rng.standard_normal((n, c)).astype(np.float32)
+    tf, tc = torch.from_numpy(feats).cuda(), torch.from_numpy(coors).cuda()
+    vf, vc, p2v, cnt, num = mluop_hip.dynamic_point_to_voxel_forward(gpu_handle, tf, tc, "max")
+    grad = mluop_hip.dynamic_point_to_voxel_backward(gpu_handle, torch.from_numpy(g).cuda(), tf, vf, p2v, cnt, num)
+    torch.cuda.synchronize()
+    want = dpv.backward(g, feats, vf.cpu().numpy(), p2v.cpu().numpy(), int(num.item()))
+    assert np.array_equal(grad.cpu().numpy(), want)
+
+
+def test_backward_mean_is_rejected_like_the_reference(gpu_handle):
+    import torch
+    import mluop_hip
+    z = torch.zeros((4, 3), device="cuda")
+    i4 = torch.zeros((4,), dtype=torch.int32, device="cuda")
+    with pytest.raises(mluop_hip.MluOpError) as e:
+        mluop_hip.dynamic_point_to_voxel_backward(gpu_handle, z, z, z, i4, i4, i4[:1], "mean")
+    assert e.value.status == mluop_hip.STATUS_BAD_PARAM

@@ -88,3 +88,47 @@ def test_all_points_invalid_and_empty():
     vf, vc, p2v, cnt, num, _ = dpv.forward("mean", feats, coors)
     assert num == 0 and p2v.tolist() == [-1, -1, -1, -1] and not vf.any()
     assert dpv.forward("max", np.zeros((0, 3), np.float32), np.zeros((0, 3), np.int32))[4] == 0
+
+
+def backward_case_inputs(cf, node):
+    """The case file stores grad_voxel_feats [34, 5] with the 150 values of its 30 real voxels only:
+    the rows past voxel_num are padded with zeros here."""
+    msgs = node.all("input")
+    bits = np.array(msgs[0].all("value_i"), dtype=np.int64).astype(np.int32).view(np.float32)
+    grad = np.zeros((34, 5), np.float32)
+    grad.reshape(-1)[:bits.size] = bits
+    return [grad] + [cf.CaseTensor(t).values for t in msgs[1:]]
+
+
+def test_backward_reference_case_file():
+    """tests/golden/dynamic_point_to_voxel_backward/case_1.prototxt: 34 points, 5 features, bit-exact."""
+    from mluop_hip import casefile as cf
+    node, _ = cf.load(os.path.join(os.path.dirname(GOLDEN), "dynamic_point_to_voxel_backward", "case_1.prototxt"))
+    ins = backward_case_inputs(cf, node)
+    want = cf.CaseTensor(node.all("output")[0]).values
+    got = dpv.backward(ins[0], ins[1], ins[2], ins[3], int(ins[5][0]))
+    assert np.array_equal(got, want)
+    assert np.count_nonzero(want) > 0
+
+
+@pytest.mark.parametrize("seed,n,c,span", [(1, 200, 4, 3), (2, 3000, 6, 8), (3, 500, 1, 2)])
+def test_backward_round_trip_through_forward(seed, n, c, span):
+    """Every (voxel, feature) hands its gradient to exactly one of the voxel's points, the first one
+    that attains the maximum; summing grad_feats over a voxel's points gives grad_voxel_feats back."""
+    rng = np.random.default_rng(seed)
+    feats = rng.integers(-3, 4, (n, c)).astype(np.float32)          # many ties
+    coors = rng.integers(0, span, (n, 3)).astype(np.int32)
+    coors[rng.choice(n, n // 10, replace=False), 0] = -1
+    vf, vc, p2v, cnt, num, _ = dpv.forward("max", feats, coors)
+    g = rng.standard_normal((n, c)).astype(np.float32)
+    grad = dpv.backward(g, feats, vf, p2v, num)
+    assert not grad[p2v < 0].any()
+    back = np.zeros((num, c), np.float32)
+    np.add.at(back, p2v[p2v >= 0], grad[p2v >= 0])
+    assert np.array_equal(back, g[:num])
+    # first point attaining the maximum, found independently
+    for v in range(0, num, max(1, num // 50)):
+        pts = np.nonzero(p2v == v)[0]
+        for j in range(c):
+            first = pts[np.argmax(feats[pts, j] == vf[v, j])]
+            assert grad[first, j] == g[v, j]
