@@ -340,7 +340,12 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool fetcher = wave >= WAVES;
   const int ftid = tid - 64 * WAVES;            // thread index among the fetching waves
-  const int r0 = blockIdx.x * TR;
+  // Workgroups go to the eight XCDs round robin; giving XCD x the x-th eighth of the
+  // tiles keeps neighbouring tiles, which gather many of the same rows, on one L2.
+  const int tiles_per_xcd = gridDim.x >> 3;
+  const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
+  const int r0 = tile * TR;
+  if (r0 >= R) return;
   const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
   for (int i = tid; i < (TR + 1) * ACC_STRIDE; i += NT) s_acc[i] = 0.f;
@@ -987,7 +992,7 @@ void launchMfmaInstance(const LaunchCtx &lc, const void *A, const void *packed,
                         const int32_t *map, int R, int K, int ldc, void *result) {
   constexpr int NT = mfmaThreads(C);
   constexpr int TR = mfmaTileRows(C);
-  const dim3 grid((R + TR - 1) / TR, ldc / C);
+  const dim3 grid(((R + TR - 1) / TR + 7) / 8 * 8, ldc / C);  // a multiple of the XCD count
   lc.begin("gatherConvMfma");
   gatherConvMfma<E, Q, C><<<grid, NT, 0, lc.stream>>>(
       static_cast<const typename E::storage *>(A),
