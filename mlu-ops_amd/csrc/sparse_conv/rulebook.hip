@@ -37,6 +37,28 @@ constexpr int kGroup = 8;                    // offsets resolved together per la
 constexpr int kMaxInlineOffsets = 128;       // kernel volumes with an in-argument offset table
 constexpr int kWordsPerBlock = 1024;  // bitmap words (64 cells each) per block
 
+// Division of a non-negative int by a divisor fixed for the launch:
+// n / d = (n * mul) >> (31 + shift) for every 0 <= n < 2^31, with shift = ceil(log2 d)
+// and mul = ceil(2^(31 + shift) / d) < 2^32.  (n * mul exceeds n / d * 2^(31+shift)
+// by less than 2^(31+shift) / d, too little to reach the next quotient.)
+struct FastDiv {
+  uint32_t mul;
+  int shift;
+};
+
+inline FastDiv makeFastDiv(int d) {
+  FastDiv f;
+  f.shift = 0;
+  while ((1ll << f.shift) < (long long)d) ++f.shift;
+  const unsigned long long p = 1ull << (31 + f.shift);
+  f.mul = (uint32_t)((p + (unsigned long long)d - 1) / (unsigned long long)d);
+  return f;
+}
+
+__device__ __forceinline__ int fastDiv(int n, FastDiv f) {
+  return (int)(((unsigned long long)(uint32_t)n * f.mul) >> (31 + f.shift));
+}
+
 struct GeomDev {
   int batch;
   int out[3];
@@ -46,6 +68,10 @@ struct GeomDev {
   int dil[3];
   int K;
   int L;
+  FastDiv by_stride[3];
+  FastDiv by_out_volume;  // out[0] * out[1] * out[2]
+  FastDiv by_out_plane;   // out[1] * out[2]
+  FastDiv by_out_width;   // out[2]
 };
 
 // Home slot of a cell (before masking): the run of 16 cells along W it belongs
@@ -73,12 +99,13 @@ __device__ __forceinline__ void storeCoord(int32_t *dst, int j, int4 v, bool ali
 }
 
 // Output coordinate along one axis; -1 when this (input, offset) has none.
-__device__ __forceinline__ int axisOut(int i, int pad, int kk, int dil, int stride, int osize) {
+__device__ __forceinline__ int axisOut(int i, int pad, int kk, int dil, int stride, FastDiv by_stride,
+                                       int osize) {
   int num = i + pad - kk * dil;
   if (num < 0) return -1;
   int o = num;
   if (stride != 1) {
-    o = num / stride;
+    o = fastDiv(num, by_stride);
     if (o * stride != num) return -1;
   }
   return o < osize ? o : -1;
@@ -181,9 +208,9 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
       if (k < k_hi) {
         int kd, kh, kw;
         decodeOffset(tab, g, k, &kd, &kh, &kw);
-        const int od = axisOut(c.y, g.pad[0], kd, g.dil[0], g.stride[0], g.out[0]);
-        const int oh = axisOut(c.z, g.pad[1], kh, g.dil[1], g.stride[1], g.out[1]);
-        const int ow = axisOut(c.w, g.pad[2], kw, g.dil[2], g.stride[2], g.out[2]);
+        const int od = axisOut(c.y, g.pad[0], kd, g.dil[0], g.stride[0], g.by_stride[0], g.out[0]);
+        const int oh = axisOut(c.z, g.pad[1], kh, g.dil[1], g.stride[1], g.by_stride[1], g.out[1]);
+        const int ow = axisOut(c.w, g.pad[2], kw, g.dil[2], g.stride[2], g.by_stride[2], g.out[2]);
         if (n_ok && (od | oh | ow) >= 0)
           cell[u] = (uint32_t)(((c.x * g.out[0] + od) * g.out[1] + oh) * g.out[2] + ow);
       }
@@ -628,50 +655,47 @@ __global__ __launch_bounds__(kBlock) void rbRankAndDecode(GeomDev g,
                                                           int32_t *out_indices, bool aligned,
                                                           int out_rows) {
   __shared__ int s_wsum[kBlock / kWave];
+  constexpr int kPerThread = kWordsPerBlock / kBlock;  // consecutive words of one thread
+  static_assert(kPerThread == 4, "one 32-byte load and one 16-byte rank store per thread");
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
-  const size_t base = (size_t)blockIdx.x * kWordsPerBlock;
-  int carry = block_excl[blockIdx.x];
+  const size_t w0 = (size_t)blockIdx.x * kWordsPerBlock + (size_t)threadIdx.x * kPerThread;
   const int hw = g.out[1] * g.out[2];
   const int vol = g.out[0] * hw;
-  for (int i = 0; i < kWordsPerBlock / kBlock; ++i) {
-    const size_t w = base + (size_t)i * kBlock + threadIdx.x;
-    unsigned long long bits = w < n_words ? bitmap[w] : 0ull;
-    const int v = __popcll(bits);
-    int incl = v;
+  unsigned long long bits[kPerThread];
+  int mine = 0;
 #pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      int t = __shfl_up(incl, off, kWave);
-      if (lane >= off) incl += t;
-    }
-    if (lane == kWave - 1) s_wsum[wave] = incl;
-    __syncthreads();
-    int woff = 0, total = 0;
+  for (int i = 0; i < kPerThread; ++i) {
+    bits[i] = w0 + i < n_words ? bitmap[w0 + i] : 0ull;
+    mine += __popcll(bits[i]);
+  }
+  const int incl = waveInclusiveScan(mine);
+  if (lane == kWave - 1) s_wsum[wave] = incl;
+  __syncthreads();
+  int rank = block_excl[blockIdx.x] + incl - mine;
 #pragma unroll
-    for (int x = 0; x < kBlock / kWave; ++x) {
-      if (x < wave) woff += s_wsum[x];
-      total += s_wsum[x];
-    }
-    int rank = carry + woff + incl - v;
-    if (w < n_words) word_rank[w] = (uint32_t)rank;
-    while (bits) {
-      const int bit = __ffsll((long long)bits) - 1;
-      bits &= bits - 1;
+  for (int x = 0; x < kBlock / kWave; ++x)
+    if (x < wave) rank += s_wsum[x];
+#pragma unroll
+  for (int i = 0; i < kPerThread; ++i) {
+    if (w0 + i < n_words) word_rank[w0 + i] = (uint32_t)rank;
+    unsigned long long b = bits[i];
+    while (b) {
+      const int bit = __ffsll((long long)b) - 1;
+      b &= b - 1;
       if (rank < out_rows) {
-        int cell = (int)(w * 64 + bit);
+        int cell = (int)((w0 + i) * 64 + bit);
         int4 o;
-        o.x = cell / vol;
+        o.x = fastDiv(cell, g.by_out_volume);
         cell -= o.x * vol;
-        o.y = cell / hw;
+        o.y = fastDiv(cell, g.by_out_plane);
         cell -= o.y * hw;
-        o.z = cell / g.out[2];
+        o.z = fastDiv(cell, g.by_out_width);
         o.w = cell - o.z * g.out[2];
         storeCoord(out_indices, rank, o, aligned);
       }
       ++rank;
     }
-    carry += total;
-    __syncthreads();
   }
   const int n_out = *num_act_out;
   const size_t gstride = (size_t)gridDim.x * kBlock;
@@ -769,7 +793,11 @@ GeomDev toDev(const RulebookGeom &g) {
     d.pad[a] = g.pad[a];
     d.stride[a] = g.stride[a];
     d.dil[a] = g.dilation[a];
+    d.by_stride[a] = makeFastDiv(g.stride[a]);
   }
+  d.by_out_volume = makeFastDiv(g.out_space[0] * g.out_space[1] * g.out_space[2]);
+  d.by_out_plane = makeFastDiv(g.out_space[1] * g.out_space[2]);
+  d.by_out_width = makeFastDiv(g.out_space[2]);
   d.K = g.K;
   d.L = g.L;
   return d;
