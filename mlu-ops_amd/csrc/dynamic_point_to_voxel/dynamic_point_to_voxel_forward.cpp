@@ -33,54 +33,48 @@ mluOpStatus_t paramCheck(const std::string &api, const mluOpHandle_t handle,
                          const mluOpTensorDescriptor_t voxel_num_desc, bool *zero_element) {
   PARAM_CHECK(api, handle != NULL);
   if (!archOk(api, handle)) return MLUOP_STATUS_ARCH_MISMATCH;
-  PARAM_CHECK(api, feats_desc != NULL);
-  PARAM_CHECK(api, coors_desc != NULL);
-  PARAM_CHECK(api, voxel_feats_desc != NULL);
-  PARAM_CHECK(api, voxel_coors_desc != NULL);
-  PARAM_CHECK(api, point2voxel_map_desc != NULL);
-  PARAM_CHECK(api, voxel_points_count_desc != NULL);
-  PARAM_CHECK(api, voxel_num_desc != NULL);
-  PARAM_CHECK(api, feats_desc->getDim() == 2);
-  PARAM_CHECK(api, coors_desc->getDim() == 2);
-  PARAM_CHECK(api, voxel_feats_desc->getDim() == 2);
-  PARAM_CHECK(api, voxel_coors_desc->getDim() == 2);
-  PARAM_CHECK(api, point2voxel_map_desc->getDim() == 1);
-  PARAM_CHECK(api, voxel_points_count_desc->getDim() == 1);
-  PARAM_CHECK(api, voxel_num_desc->getDim() == 1);
-  STRIDE_TENSOR_CHECK(api + ":", feats_desc, "feats_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api + ":", coors_desc, "coors_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api + ":", voxel_feats_desc, "voxel_feats_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api + ":", voxel_coors_desc, "voxel_coors_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api + ":", point2voxel_map_desc, "point2voxel_map_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api + ":", voxel_points_count_desc,
-                      "voxel_points_count_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api + ":", voxel_num_desc, "voxel_num_desc must be contiguous");
-  PARAM_CHECK_V2(api, (feats_desc->getDtype() == MLUOP_DTYPE_FLOAT),
-                 "Only float are supported in feats tensor, but the data type of tensor is "
-                     << mluop::getNameOfDataType(feats_desc->getDtype()) << ".");
-  PARAM_CHECK_V2(api, (coors_desc->getDtype() == MLUOP_DTYPE_INT32),
-                 "Only int32 are supported in coors tensor, but the data type of tensor is "
-                     << mluop::getNameOfDataType(coors_desc->getDtype()) << ".");
-  PARAM_CHECK_V2(api, (point2voxel_map_desc->getDtype() == MLUOP_DTYPE_INT32),
-                 "Only int32 are supported in point2voxel_map tensor, but the data type of tensor is "
-                     << mluop::getNameOfDataType(point2voxel_map_desc->getDtype()) << ".");
-  PARAM_CHECK(api, voxel_feats_desc->getDtype() == feats_desc->getDtype());
-  PARAM_CHECK(api, voxel_coors_desc->getDtype() == coors_desc->getDtype());
-  PARAM_CHECK(api, voxel_points_count_desc->getDtype() == point2voxel_map_desc->getDtype());
-  PARAM_CHECK(api, voxel_num_desc->getDtype() == point2voxel_map_desc->getDtype());
+
+  // The seven tensors in argument order, with the rank and element type each must have;
+  // the checks run in the reference's order: all descriptors, all ranks, all strides, all types.
+  struct Expect {
+    const mluOpTensorDescriptor_t desc;
+    const char *name;
+    int rank;
+    mluOpDataType_t dtype;
+  };
+  const Expect tensors[] = {
+      {feats_desc, "feats", 2, MLUOP_DTYPE_FLOAT},
+      {coors_desc, "coors", 2, MLUOP_DTYPE_INT32},
+      {voxel_feats_desc, "voxel_feats", 2, MLUOP_DTYPE_FLOAT},
+      {voxel_coors_desc, "voxel_coors", 2, MLUOP_DTYPE_INT32},
+      {point2voxel_map_desc, "point2voxel_map", 1, MLUOP_DTYPE_INT32},
+      {voxel_points_count_desc, "voxel_points_count", 1, MLUOP_DTYPE_INT32},
+      {voxel_num_desc, "voxel_num", 1, MLUOP_DTYPE_INT32},
+  };
+  for (const Expect &t : tensors)
+    PARAM_CHECK_V2(api, t.desc != NULL, "descriptor of " << t.name << " is NULL.");
+  for (const Expect &t : tensors)
+    PARAM_CHECK_V2(api, t.desc->getDim() == t.rank, t.name << " must have " << t.rank << " dimensions.");
+  for (const Expect &t : tensors)
+    STRIDE_TENSOR_CHECK(api + ":", t.desc, t.name << " must be contiguous");
+  for (const Expect &t : tensors)
+    PARAM_CHECK_V2(api, t.desc->getDtype() == t.dtype,
+                   t.name << " must be " << mluop::getNameOfDataType(t.dtype) << ", but is "
+                          << mluop::getNameOfDataType(t.desc->getDtype()) << ".");
   if (reduce_type != MLUOP_REDUCE_DMAX && reduce_type != MLUOP_REDUCE_DMEAN) {
-    MLUOP_LOG(ERROR) << api << " Only support max and mean. Please check reduce_type!";
+    MLUOP_LOG(ERROR) << api << " reduce_type must be max or mean.";
     return MLUOP_STATUS_BAD_PARAM;
   }
-  PARAM_CHECK(api, feats_desc->getDimIndex(0) == coors_desc->getDimIndex(0));
-  PARAM_CHECK(api, feats_desc->getDimIndex(0) == point2voxel_map_desc->getDimIndex(0));
-  PARAM_CHECK(api, voxel_feats_desc->getDimIndex(0) == voxel_coors_desc->getDimIndex(0));
-  PARAM_CHECK(api, voxel_feats_desc->getDimIndex(0) == voxel_points_count_desc->getDimIndex(0));
+
+  // N points, M voxel rows, C features, three coordinates
+  const int64_t n = feats_desc->getDimIndex(0), c = feats_desc->getDimIndex(1);
+  const int64_t m = voxel_feats_desc->getDimIndex(0);
+  PARAM_CHECK(api, coors_desc->getDimIndex(0) == n && point2voxel_map_desc->getDimIndex(0) == n);
+  PARAM_CHECK(api, voxel_coors_desc->getDimIndex(0) == m && voxel_points_count_desc->getDimIndex(0) == m);
   PARAM_CHECK(api, voxel_num_desc->getDimIndex(0) == 1);
-  PARAM_CHECK(api, feats_desc->getDimIndex(1) == voxel_feats_desc->getDimIndex(1));
-  PARAM_CHECK(api, coors_desc->getDimIndex(1) == voxel_coors_desc->getDimIndex(1));
-  PARAM_CHECK(api, coors_desc->getDimIndex(1) == 3);
-  PARAM_CHECK(api, feats_desc->getDimIndex(0) >= voxel_feats_desc->getDimIndex(0));
+  PARAM_CHECK(api, voxel_feats_desc->getDimIndex(1) == c);
+  PARAM_CHECK(api, coors_desc->getDimIndex(1) == 3 && voxel_coors_desc->getDimIndex(1) == 3);
+  PARAM_CHECK(api, n >= m);
 
   const size_t feats_element_num = mluOpGetTensorElementNum(feats_desc);
   const size_t coors_element_num = mluOpGetTensorElementNum(coors_desc);
@@ -93,13 +87,10 @@ mluOpStatus_t paramCheck(const std::string &api, const mluOpHandle_t handle,
   if (workspace_size > 0) {
     PARAM_CHECK(api, workspace != NULL);
   }
-  PARAM_CHECK(api, feats != NULL);
-  PARAM_CHECK(api, coors != NULL);
-  PARAM_CHECK(api, voxel_feats != NULL);
-  PARAM_CHECK(api, voxel_coors != NULL);
-  PARAM_CHECK(api, point2voxel_map != NULL);
-  PARAM_CHECK(api, voxel_points_count != NULL);
-  PARAM_CHECK(api, voxel_num != NULL);
+  const void *const data[] = {feats, coors, voxel_feats, voxel_coors, point2voxel_map, voxel_points_count,
+                              voxel_num};
+  for (size_t i = 0; i < sizeof(data) / sizeof(data[0]); ++i)
+    PARAM_CHECK_V2(api, data[i] != NULL, tensors[i].name << " is NULL.");
   return MLUOP_STATUS_SUCCESS;
 }
 
