@@ -29,40 +29,37 @@ mluOpStatus_t voxelizationParamCheck(const char *api, const mluOpHandle_t handle
     MLUOP_LOG(ERROR) << api << " Non-deterministic mode is not supported.";
     return MLUOP_STATUS_BAD_PARAM;
   }
-  PARAM_CHECK_EQ(api, points_desc->getDim(), 2);
-  PARAM_CHECK_EQ(api, voxel_size_desc->getDim(), 1);
-  PARAM_CHECK_EQ(api, voxel_size_desc->getDimIndex(0), 3);
-  PARAM_CHECK_EQ(api, coors_range_desc->getDim(), 1);
-  PARAM_CHECK_EQ(api, coors_range_desc->getDimIndex(0), 6);
-  PARAM_CHECK_EQ(api, voxels_desc->getDim(), 3);
-  PARAM_CHECK_EQ(api, voxels_desc->getDimIndex(0), max_voxels);
-  PARAM_CHECK_EQ(api, voxels_desc->getDimIndex(1), max_points);
-  PARAM_CHECK_EQ(api, voxels_desc->getDimIndex(2), points_desc->getDimIndex(1));
-  PARAM_CHECK_EQ(api, coors_desc->getDim(), 2);
-  PARAM_CHECK_EQ(api, coors_desc->getDimIndex(0), max_voxels);
-  PARAM_CHECK_EQ(api, coors_desc->getDimIndex(1), 3);
-  PARAM_CHECK_EQ(api, num_points_per_voxel_desc->getDim(), 1);
-  PARAM_CHECK_EQ(api, num_points_per_voxel_desc->getDimIndex(0), max_voxels);
-  PARAM_CHECK_EQ(api, voxel_num_desc->getDim(), 1);
-  PARAM_CHECK_EQ(api, voxel_num_desc->getDimIndex(0), 1);
+  // points [N, F]; voxel_size [3]; coors_range [6]; voxels [max_voxels, max_points, F];
+  // coors [max_voxels, 3]; num_points_per_voxel [max_voxels]; voxel_num [1].
+  // -1 in `dims` = "whatever the tensor says" (N and F come from points).
+  struct Expect {
+    const mluOpTensorDescriptor_t desc;
+    const char *name;
+    int rank;
+    int64_t dims[3];
+    mluOpDataType_t dtype;
+  };
+  const int64_t features = points_desc->getDim() == 2 ? points_desc->getDimIndex(1) : -1;
+  const Expect tensors[] = {
+      {points_desc, "points", 2, {-1, -1, 0}, MLUOP_DTYPE_FLOAT},
+      {voxel_size_desc, "voxel_size", 1, {3, 0, 0}, MLUOP_DTYPE_FLOAT},
+      {coors_range_desc, "coors_range", 1, {6, 0, 0}, MLUOP_DTYPE_FLOAT},
+      {voxels_desc, "voxels", 3, {max_voxels, max_points, features}, MLUOP_DTYPE_FLOAT},
+      {coors_desc, "coors", 2, {max_voxels, 3, 0}, MLUOP_DTYPE_INT32},
+      {num_points_per_voxel_desc, "num_points_per_voxel", 1, {max_voxels, 0, 0}, MLUOP_DTYPE_INT32},
+      {voxel_num_desc, "voxel_num", 1, {1, 0, 0}, MLUOP_DTYPE_INT32},
+  };
+  for (const Expect &t : tensors) {
+    PARAM_CHECK_V2(api, t.desc->getDim() == t.rank, t.name << " must have " << t.rank << " dimensions.");
+    for (int a = 0; a < t.rank; ++a)
+      PARAM_CHECK_V2(api, t.dims[a] < 0 || t.desc->getDimIndex(a) == t.dims[a],
+                     "dimension " << a << " of " << t.name << " must be " << t.dims[a] << ".");
+  }
   PARAM_CHECK_EQ(api, NDim, 3);
-
-  STRIDE_TENSOR_CHECK(api, points_desc, "points_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api, voxel_size_desc, "voxel_size_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api, coors_range_desc, "coors_range_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api, voxels_desc, "voxels_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api, coors_desc, "coors_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api, num_points_per_voxel_desc,
-                      "num_points_per_voxel_desc must be contiguous");
-  STRIDE_TENSOR_CHECK(api, voxel_num_desc, "voxel_num_desc must be contiguous");
-
-  PARAM_CHECK(api, points_desc->getDtype() == MLUOP_DTYPE_FLOAT);
-  PARAM_CHECK(api, voxel_size_desc->getDtype() == MLUOP_DTYPE_FLOAT);
-  PARAM_CHECK(api, coors_range_desc->getDtype() == MLUOP_DTYPE_FLOAT);
-  PARAM_CHECK(api, voxels_desc->getDtype() == MLUOP_DTYPE_FLOAT);
-  PARAM_CHECK(api, coors_desc->getDtype() == MLUOP_DTYPE_INT32);
-  PARAM_CHECK(api, num_points_per_voxel_desc->getDtype() == MLUOP_DTYPE_INT32);
-  PARAM_CHECK(api, voxel_num_desc->getDtype() == MLUOP_DTYPE_INT32);
+  for (const Expect &t : tensors) STRIDE_TENSOR_CHECK(api, t.desc, t.name << " must be contiguous");
+  for (const Expect &t : tensors)
+    PARAM_CHECK_V2(api, t.desc->getDtype() == t.dtype,
+                   t.name << " must be " << mluop::getNameOfDataType(t.dtype) << ".");
 
   const uint64_t points_num = mluOpGetTensorElementNum(points_desc);
   const uint64_t voxel_size_num = mluOpGetTensorElementNum(voxel_size_desc);
