@@ -671,10 +671,14 @@ constexpr int kFilterMaxSlices = 768;    // about three workgroups per CU
 
 // Both operands are needed with the pair index running along the MFMA's K
 // dimension, i.e. transposed relative to the row-major tensors: rows are
-// gathered with row-contiguous 16-byte loads and written to LDS transposed
-// ([channel][pair], element-sized stores), from where an operand fragment (8
-// consecutive pairs of one channel, 4 for float) is one 16-byte read.  Wave w multiplies the
-// 16-row blocks w, w+4, ... of dW[k] against all column blocks.
+// gathered with 16-byte loads and written to LDS transposed ([channel][pair],
+// element-sized stores), from where an operand fragment (8 consecutive pairs of
+// one channel, 4 for float) is one 16-byte read.  A wave stages 32 pairs x two
+// neighbouring 16-byte pieces at a time: every transposed store of the wave then
+// writes two runs of 32 consecutive pairs, which no two lanes share a bank in
+// (with a row's pieces spread over eight lanes the same stores hit 8 banks and
+// took 28 cycles each).  Wave w multiplies the 16-row blocks w, w+4, ... of dW[k]
+// against all column blocks.
 template <typename E, int CI, int CO>
 __global__ __launch_bounds__(256) void backwardFilterMfma(
     const typename E::storage *X, const typename E::storage *dY, const int32_t *pairs, int L,
@@ -688,6 +692,9 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
   constexpr int YP = SP * CO / EPP;
   constexpr int XT = XP / 256 > 0 ? XP / 256 : 1;
   constexpr int YT = YP / 256 > 0 ? YP / 256 : 1;
+  constexpr int XU = XP / 64;  // staging units (32 pairs x 2 pieces) of X per step
+  constexpr int YU = YP / 64;
+  static_assert(SP == 64 && (CI / EPP) % 2 == 0 && (CO / EPP) % 2 == 0, "unit = 32 pairs x 2 pieces");
   constexpr int CBW = (CI / 16 + 3) / 4;  // row blocks per wave
   constexpr int COB = CO / 16;
   static_assert(XP % 256 == 0 || XP < 256, "piece split");
@@ -721,31 +728,33 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
   auto fetch_step = [&](int local) {  // local = first pair of the step within the index chunk
 #pragma unroll
     for (int i = 0; i < XT; ++i) {
-      const int q = tid + i * 256;
+      const int u = wave + i * 4;  // unit: pairs 32*(u&1).., pieces 2*(u>>1)..
       xr[i] = u32x4{0u, 0u, 0u, 0u};
-      if (XP >= 256 || q < XP) {
-        const int row = s_in[local + q / (CI / EPP)];
+      if (XU >= 4 || u < XU) {
+        const int row = s_in[local + (u & 1) * 32 + (lane >> 1)];
         if (row >= 0)
-          xr[i] = *reinterpret_cast<const u32x4 *>(X + (size_t)row * CI + (q % (CI / EPP)) * EPP);
+          xr[i] = *reinterpret_cast<const u32x4 *>(X + (size_t)row * CI +
+                                                   ((u >> 1) * 2 + (lane & 1)) * EPP);
       }
     }
 #pragma unroll
     for (int i = 0; i < YT; ++i) {
-      const int q = tid + i * 256;
+      const int u = wave + i * 4;
       yr[i] = u32x4{0u, 0u, 0u, 0u};
-      if (YP >= 256 || q < YP) {
-        const int row = s_out[local + q / (CO / EPP)];
+      if (YU >= 4 || u < YU) {
+        const int row = s_out[local + (u & 1) * 32 + (lane >> 1)];
         if (row >= 0)
-          yr[i] = *reinterpret_cast<const u32x4 *>(dY + (size_t)row * CO + (q % (CO / EPP)) * EPP);
+          yr[i] = *reinterpret_cast<const u32x4 *>(dY + (size_t)row * CO +
+                                                   ((u >> 1) * 2 + (lane & 1)) * EPP);
       }
     }
   };
   auto store_step = [&]() {
 #pragma unroll
     for (int i = 0; i < XT; ++i) {
-      const int q = tid + i * 256;
-      if (XP >= 256 || q < XP) {
-        const int pr = q / (CI / EPP), c0 = (q % (CI / EPP)) * EPP;
+      const int u = wave + i * 4;
+      if (XU >= 4 || u < XU) {
+        const int pr = (u & 1) * 32 + (lane >> 1), c0 = ((u >> 1) * 2 + (lane & 1)) * EPP;
 #pragma unroll
         for (int e = 0; e < EPP; ++e) {
           if constexpr (sizeof(S) == 2)
@@ -758,9 +767,9 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
     }
 #pragma unroll
     for (int i = 0; i < YT; ++i) {
-      const int q = tid + i * 256;
-      if (YP >= 256 || q < YP) {
-        const int pr = q / (CO / EPP), c0 = (q % (CO / EPP)) * EPP;
+      const int u = wave + i * 4;
+      if (YU >= 4 || u < YU) {
+        const int pr = (u & 1) * 32 + (lane >> 1), c0 = ((u >> 1) * 2 + (lane & 1)) * EPP;
 #pragma unroll
         for (int e = 0; e < EPP; ++e) {
           if constexpr (sizeof(S) == 2)
@@ -829,10 +838,10 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
   }
 }
 
-// dW[k] = sum of the offset's partial tiles, rounded once.  A block adds 64
-// consecutive elements: wave g of 16 takes the slices g, g+16, ... in eight
-// independent running sums, the sums are combined pairwise in a fixed order,
-// so the result depends on the slice count only, never on timing.
+// dW[k] = sum of the offset's partial tiles, rounded once.  A block adds 256
+// consecutive elements (four per lane): wave g of 16 takes the slices g, g+16, ...
+// in eight independent running sums, the sums are combined pairwise in a fixed
+// order, so the result depends on the slice count only, never on timing.
 constexpr int kSliceSumWaves = 16;
 template <typename E>
 __global__ __launch_bounds__(64 * kSliceSumWaves) void sliceSum(const float *partial,
@@ -840,34 +849,37 @@ __global__ __launch_bounds__(64 * kSliceSumWaves) void sliceSum(const float *par
                                                                 int tile_elems,
                                                                 typename E::storage *dW) {
   constexpr int W = kSliceSumWaves;
-  __shared__ float s_part[W][64];
+  __shared__ float4v s_part[W][64];
   const int k = blockIdx.y;
   const int lane = threadIdx.x & 63;
   const int g = threadIdx.x >> 6;
-  const int e = blockIdx.x * 64 + lane;
+  const int e = (blockIdx.x * 64 + lane) * 4;  // tile_elems is a multiple of 256
   const int slices = (tab.n[k] + slice_len - 1) / slice_len;
-  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float4v acc[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) acc[u] = float4v{0.f, 0.f, 0.f, 0.f};
   if (e < tile_elems) {
     const float *src = partial + (size_t)tab.first[k] * tile_elems + e;
     for (int i0 = g; i0 < slices; i0 += 8 * W) {
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int i = i0 + W * u;
-        if (i < slices) acc[u] += src[(size_t)i * tile_elems];
+        if (i < slices) acc[u] += *reinterpret_cast<const float4v *>(src + (size_t)i * tile_elems);
       }
     }
   }
   s_part[g][lane] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
   __syncthreads();
   if (g == 0 && e < tile_elems) {
-    float t[W];
+    float4v t[W];
 #pragma unroll
     for (int i = 0; i < W; ++i) t[i] = s_part[i][lane];
 #pragma unroll
     for (int span = 1; span < W; span *= 2)
 #pragma unroll
       for (int i = 0; i < W; i += 2 * span) t[i] += t[i + span];
-    E::store(dW + (size_t)k * tile_elems + e, t[0]);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) E::store(dW + (size_t)k * tile_elems + e + v, t[0][v]);
   }
 }
 
@@ -1128,7 +1140,7 @@ void launchFilterMfmaInstance(const LaunchCtx &lc, const ConvProblem &p, const S
         p.L, p.L, p.num_out, p.K, tab, slice_len, partial);
   lc.end();
   lc.begin("sliceSum");
-  sliceSum<E><<<dim3((CI * CO + 63) / 64, p.K), 64 * kSliceSumWaves, 0, lc.stream>>>(
+  sliceSum<E><<<dim3(CI * CO / 256, p.K), 64 * kSliceSumWaves, 0, lc.stream>>>(
       partial, tab, slice_len, CI * CO, static_cast<S *>(filters_grad));
   lc.end();
 }
