@@ -1,0 +1,59 @@
+"""The submanifold rulebook and the three convolution operators enqueue kernels only (no stream
+synchronisation, no allocation, no memset nodes), so a caller can capture them into a HIP graph.
+One layer's step is captured once and replayed several times, with ordinary eager calls and
+synchronisations in between, and every replay must reproduce the eager results bit for bit."""
+import numpy as np
+import pytest
+
+from spconv_cases import random_voxels
+
+pytestmark = pytest.mark.gpu
+
+
+def test_captured_step_replays_bit_exactly():
+    import torch
+    import mluop_hip as m
+    rng = np.random.default_rng(31)
+    batch, space, L, ci, co, ks = 2, (12, 24, 24), 5000, 64, 64, (3, 3, 3)
+    idx = torch.from_numpy(random_voxels(rng, batch, space, L)).cuda()
+    feats = torch.from_numpy(rng.standard_normal((L, ci)).astype(np.float32)).cuda().half()
+    w = torch.from_numpy((rng.standard_normal(ks + (ci, co)) * 0.1).astype(np.float32)).cuda().half()
+    dy = torch.from_numpy(rng.standard_normal((L, co)).astype(np.float32)).cuda().half()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        handle = m.make_handle_on_current_stream()      # the handle's queue is the capture stream
+
+        def step(num_host):
+            pairs, out_idx, num, n_out = m.get_indice_pairs(handle, idx, batch, space, ks, list(space), [1, 1, 1],
+                                                            [1, 1, 1], [1, 1, 1], True)
+            out = m.indice_conv_forward(handle, feats, w, m.LAYOUT_ARRAY, pairs, num_host, L, True)
+            dx = m.indice_conv_backward_data(handle, dy, w, m.LAYOUT_ARRAY, pairs, num_host, True, ci)
+            dw = m.indice_conv_backward_filter(handle, feats, dy, pairs, num_host, ks, True)
+            return pairs, num, out, dx, dw
+
+        # eager reference (also the warm-up); indice_num goes to the host once, as a framework does
+        pairs0, num0, _, _, _ = step([L] * 27)
+        side.synchronize()
+        num_host = num0.cpu().tolist()
+        eager = [t.clone() for t in step(num_host)]
+        side.synchronize()
+
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            captured = step(num_host)
+        for replay in range(4):
+            for t in captured:
+                t.fill_(0)                               # eager work between the replays
+            extra = step(num_host)                       # and an eager step on the same stream
+            side.synchronize()
+            graph.replay()
+            side.synchronize()
+            for name, got, want in zip(("pairs", "indice_num", "forward", "backward_data", "backward_filter"),
+                                       captured, eager):
+                assert torch.equal(got, want), "replay %d: %s" % (replay, name)
+            for got, want in zip(extra, eager):
+                assert torch.equal(got, want)
+    torch.cuda.current_stream().wait_stream(side)
+    handle.close()
