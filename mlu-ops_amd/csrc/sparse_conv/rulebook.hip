@@ -76,7 +76,8 @@ struct GeomDev {
 
 // Home slot of a cell (before masking): the run of 16 cells along W it belongs
 // to is hashed, the position inside the run is kept.  Neighbours along W have
-// neighbouring home slots, so one 12-byte load answers three probes.
+// neighbouring home slots, so one window of consecutive keys answers the
+// probes of all kernel positions along W.
 __device__ __forceinline__ uint32_t hashCell(uint32_t key) {
   uint32_t h = (key >> 4) * 0x9E3779B1u;
   h ^= h >> 15;
