@@ -205,7 +205,8 @@ __global__ __launch_bounds__(256) void gatherConvSimt(const typename E::storage 
 // CHUNK reduction channels per fragment; 8 and 32 for the 2-byte types, 4 and 16
 // for float):
 // packed[(((k*(C/16) + nb)*(Q/CHUNK) + kb)*64 + lane)*VEC + e]
-//   = B(k, q = kb*CHUNK + VEC*(lane/16) + e, c = nb*16 + lane%16).
+//   = B(k, q = kb*CHUNK + VEC*(lane/16) + e, c = nb*16 + lane%16), zero for q >= Q
+// (16 reduction channels of a 2-byte type fill half a fragment).
 // One launch for the two independent preparations of the MFMA path: blocks
 // below fill_blocks set the row map to -1 (16-byte stores), the others repack
 // the filter.
@@ -226,20 +227,22 @@ __global__ __launch_bounds__(256) void fillMapPackFilter(int32_t *map, size_t ma
   }
   const int pack_blocks = gridDim.x - fill_blocks;
   constexpr int VEC = E::kVec, CHUNK = E::kChunk;
-  const size_t total = (size_t)K * (C / 16) * (Q / CHUNK) * 64;
+  const int chunks = (Q + CHUNK - 1) / CHUNK;  // Q below one fragment is padded with zeros
+  const size_t total = (size_t)K * (C / 16) * chunks * 64;
   for (size_t t = (size_t)(blockIdx.x - fill_blocks) * 256 + threadIdx.x; t < total;
        t += (size_t)pack_blocks * 256) {
     const int lane = (int)(t & 63);
     size_t rest = t >> 6;
-    const int kb = (int)(rest % (Q / CHUNK));
-    rest /= (Q / CHUNK);
+    const int kb = (int)(rest % chunks);
+    rest /= chunks;
     const int nb = (int)(rest % (C / 16));
     const int k = (int)(rest / (C / 16));
     const int c = nb * 16 + (lane & 15);
     const int qb = kb * CHUNK + VEC * (lane >> 4);
 #pragma unroll
     for (int e = 0; e < VEC; ++e)
-      packed[t * VEC + e] = W[(size_t)k * sK + (size_t)(qb + e) * sQ + (size_t)c * sC];
+      packed[t * VEC + e] =
+          qb + e < Q ? W[(size_t)k * sK + (size_t)(qb + e) * sQ + (size_t)c * sC] : typename E::storage(0);
   }
 }
 
@@ -265,7 +268,7 @@ constexpr int mfmaStageRows(int row_bytes) {
 // 16-pair blocks multiplied together; bounded by the registers the W fragments of two batches
 // take (16 bytes per lane for every 16-byte piece of a row and every 16 result columns).
 constexpr int mfmaBatchBlocks(int elem_bytes, int Q, int C) {
-  const int regs_per_block = (Q * elem_bytes / 64) * (C >= 128 ? 2 : 1) * 4;
+  const int regs_per_block = ((Q * elem_bytes + 63) / 64) * mfmaColBlocksPerWave(C) * 4;
   const int g = 32 / regs_per_block;
   return g < 1 ? 1 : (g > 4 ? 4 : g);
 }
@@ -310,7 +313,8 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   constexpr int NT = mfmaThreads(C);
   constexpr int TR = mfmaTileRows(C);
   constexpr int NSEG = TR / 64;
-  constexpr int KB = Q / E::kChunk;           // operand fragments per row
+  constexpr int KB = (Q + E::kChunk - 1) / E::kChunk;  // operand fragments per row
+  constexpr bool kPartialFragment = Q < E::kChunk;     // 16 channels of a 2-byte type: upper lanes are zero
   constexpr int KC = kOffsetChunk;
   constexpr int ALLW = NT / 64;                 // multiplying + fetching waves
   constexpr int FW = ALLW - WAVES;              // fetching waves
@@ -512,6 +516,11 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
 #pragma unroll
           for (int kb = 0; kb < KB; ++kb)
             afr[g][kb] = *reinterpret_cast<const vec8 *>(arow + kb * 64);
+          if constexpr (kPartialFragment) {
+            // the row ends after Q channels: the lanes of the upper quads would read the next
+            // staged row; they multiply zero filter fragments, and zero keeps a NaN there out
+            if (quad * E::kVec >= Q) afr[g][0] = vec8{};
+          }
         }
         float4v prod[G][NB];
 #pragma unroll
@@ -905,11 +914,10 @@ bool forceSimt() {
   return v != nullptr && v[0] == '1';
 }
 
-// fp16/bf16: 16x16x32 MFMA, reduction channels in {32, 64, 128}; float: 16x16x4 MFMA,
-// reduction channels in {16, 32, 64, 128}.
+// fp16/bf16: 16x16x32 MFMA; float: 16x16x4 MFMA; reduction channels in {16, 32, 64, 128}.
 bool mfmaShapeOk(ElemType t, int Q, int C) {
-  const bool q_ok = t == ElemType::kFloat ? (Q == 16 || Q == 32 || Q == 64 || Q == 128)
-                                          : (Q == 32 || Q == 64 || Q == 128);
+  (void)t;  // 16 channels of a 2-byte type run as half-filled fragments
+  const bool q_ok = (Q == 16 || Q == 32 || Q == 64 || Q == 128);
   const bool c_ok = (C == 16 || C == 32 || C == 64 || C == 128);
   return q_ok && c_ok;
 }
@@ -950,8 +958,12 @@ GatherWorkspace carveGather(const ConvProblem &p, const GatherDims &d, void *bas
   };
   if (p.K > kMaxInlineK) ws.dev_counts = reinterpret_cast<int32_t *>(take((size_t)p.K * 4));
   ws.map = reinterpret_cast<int32_t *>(take((size_t)p.K * d.R * 4));
-  if (mfmaShapeOk(p.dtype, d.Q, d.C))
-    ws.packed = take((size_t)p.K * d.Q * d.C * elemSize(p.dtype));
+  if (mfmaShapeOk(p.dtype, d.Q, d.C)) {
+    // reduction channels are padded to whole 16-byte fragments (32 for the 2-byte types)
+    const size_t chunk = 64 / elemSize(p.dtype);
+    const size_t q_padded = ((size_t)d.Q + chunk - 1) / chunk * chunk;
+    ws.packed = take((size_t)p.K * q_padded * d.C * elemSize(p.dtype));
+  }
   ws.bytes = off + kBaseAlign;
   return ws;
 }
@@ -1030,11 +1042,8 @@ void launchMfmaByC(const LaunchCtx &lc, int C, int tile_cols, const void *A, con
 template <typename E>
 void launchMfma(const LaunchCtx &lc, int Q, int C, int tile_cols, const void *A, const void *packed,
                 const int32_t *map, int R, int K, void *result) {
-  constexpr bool is_float = std::is_same<E, FloatElem>::value;
   switch (Q) {
-    case 16:
-      if constexpr (is_float) launchMfmaByC<E, 16>(lc, C, tile_cols, A, packed, map, R, K, result);
-      break;
+    case 16: launchMfmaByC<E, 16>(lc, C, tile_cols, A, packed, map, R, K, result); break;
     case 32: launchMfmaByC<E, 32>(lc, C, tile_cols, A, packed, map, R, K, result); break;
     case 64: launchMfmaByC<E, 64>(lc, C, tile_cols, A, packed, map, R, K, result); break;
     case 128: launchMfmaByC<E, 128>(lc, C, tile_cols, A, packed, map, R, K, result); break;
@@ -1062,7 +1071,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
   const int64_t sC = d.row_col == 1 ? f.stride_co : f.stride_ci;
   const size_t map_elems = (size_t)p.K * d.R;
   if (use_mfma) {
-    const size_t frags = (size_t)p.K * (d.C / 16) * (d.Q / E::kChunk) * 64;
+    const size_t frags = (size_t)p.K * (d.C / 16) * ((d.Q + E::kChunk - 1) / E::kChunk) * 64;
     const int fill_blocks = gridFor(map_elems / 4 + 1, 2048);
     const int pack_blocks = gridFor(frags, 512);
     lc.begin("fillMapPackFilter");

@@ -82,6 +82,8 @@ SHAPES = [
     # (batch, space, L, ks, ci, co, sub_m, stride)
     (1, (6, 6, 6), 50, (3, 3, 3), 16, 16, True, (1, 1, 1)),
     (2, (8, 9, 10), 400, (3, 3, 3), 32, 32, True, (1, 1, 1)),
+    (2, (8, 9, 10), 400, (3, 3, 3), 16, 32, True, (1, 1, 1)),     # 16 reduction channels: half-filled fragments for fp16/bf16
+    (1, (8, 8, 8), 300, (3, 3, 3), 32, 16, False, (2, 2, 2)),
     (1, (10, 12, 12), 900, (3, 3, 3), 64, 64, True, (1, 1, 1)),
     (2, (8, 10, 10), 500, (3, 3, 3), 64, 32, False, (2, 2, 2)),
     (1, (8, 8, 8), 300, (3, 3, 3), 32, 128, True, (1, 1, 1)),
