@@ -267,6 +267,58 @@ UPSTREAM = {
 }
 
 
+def run_backbone(args, torch, m):
+    """Forward + backward of a sparse encoder in the shape of SECOND / CenterPoint's (submanifold
+    pairs at four resolutions, strided convolutions between them) over the caller layer
+    (mluop_hip.nn): what a training step of the sparse part costs end to end, Python included."""
+    import numpy as np
+    from mluop_hip import nn as spnn
+    grid = (1, 41, 1600, 1408)
+    idx = m.datagen.clustered_voxels(grid, 120000, 4)
+    rng = np.random.default_rng(4)
+    feats = torch.from_numpy(rng.standard_normal((idx.shape[0], 5)).astype(np.float32)).cuda().half()
+    indices = torch.from_numpy(idx).cuda()
+    torch.manual_seed(0)
+    layers = [spnn.SubMConv3d(5, 16, 3, indice_key="s1"), spnn.SubMConv3d(16, 16, 3, indice_key="s1")]
+    c = 16
+    for stage, co in enumerate((32, 64, 128), start=2):
+        layers.append(spnn.SparseConv3d(c, co, 3, stride=2, padding=1))
+        layers += [spnn.SubMConv3d(co, co, 3, indice_key="s%d" % stage) for _ in range(2)]
+        c = co
+    net = torch.nn.ModuleList(layers).cuda().half()
+
+    def step():
+        x = spnn.SparseTensor(feats.clone().requires_grad_(True), indices, grid[1:], grid[0])
+        for layer in net:
+            x = layer(x)
+            x = x.replace_features(torch.relu(x.features))
+        x.features.float().square().mean().backward()
+        return x
+
+    for _ in range(max(args.warmup, 2)):
+        out = step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    rows = [int(idx.shape[0])]
+    x = spnn.SparseTensor(feats, indices, grid[1:], grid[0])
+    with torch.no_grad():
+        for layer in net:
+            x = layer(x)
+            if not layer.sub_m:
+                rows.append(int(x.features.shape[0]))
+    print(json.dumps({"metric": "sparse encoder forward+backward ms", "value": ms, "unit": "ms", "n_gpus": 1,
+                      "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+                      "config": {"workload": "11 sparse layers (5-16-16 | 32x3 | 64x3 | 128x3 channels, 3 strided), "
+                                             "120000 clustered voxels in 1x41x1600x1408, fp16, wall clock with "
+                                             "the Python caller layer", "rows_per_stage": rows},
+                      "output_rows": int(out.features.shape[0])}))
+
+
 def run_upstream(args, torch, m, handle):
     """Times one of the upstream operators (not the headline metric): prints its own JSON line."""
     import numpy as np
@@ -329,7 +381,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="config4", choices=sorted(WORKLOADS) + sorted(UPSTREAM))
+    ap.add_argument("--workload", default="config4", choices=sorted(WORKLOADS) + sorted(UPSTREAM) + ["backbone"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only-step", action="store_true",
                     help="run just warmup + timed steps (for profiler runs)")
@@ -348,6 +400,9 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.workload == "backbone":
+        run_backbone(args, torch, m)
+        return
     handle = m.make_handle_on_current_stream()
     if args.workload in UPSTREAM:
         run_upstream(args, torch, m, handle)

@@ -93,6 +93,14 @@ class _IndiceConv(torch.autograd.Function):
         return grad_features, grad_weight, None
 
 
+def _mfma_channels(c):
+    """The next channel count the matrix-core kernels take, or c itself beyond 128."""
+    for size in (16, 32, 64, 128):
+        if c <= size:
+            return size
+    return c
+
+
 def _triple(v):
     return [int(v)] * 3 if isinstance(v, int) else [int(x) for x in v]
 
@@ -134,7 +142,18 @@ class _ConvBase(torch.nn.Module):
 
     def forward(self, x):
         rb = self._rulebook(x)
-        feats = _IndiceConv.apply(x.features, self.weight.to(x.features.dtype), rb)
+        feats, weight = x.features, self.weight.to(x.features.dtype)
+        # Channel counts the matrix-core kernels take are 16, 32, 64 and 128; a smaller count (the
+        # 4 or 5 point features of a first layer) is padded with zero channels, which costs a few
+        # megabytes of traffic and saves the several times slower generic kernels.  autograd slices
+        # the gradients back.
+        ci, co = _mfma_channels(self.in_channels), _mfma_channels(self.out_channels)
+        if ci != self.in_channels or co != self.out_channels:
+            feats = torch.nn.functional.pad(feats, (0, ci - self.in_channels))
+            weight = torch.nn.functional.pad(weight, (0, co - self.out_channels, 0, ci - self.in_channels))
+        feats = _IndiceConv.apply(feats, weight, rb)
+        if co != self.out_channels:
+            feats = feats[:, :self.out_channels]
         if self.bias is not None:
             feats = feats + self.bias.to(feats.dtype)
         if self.sub_m:

@@ -135,3 +135,36 @@ def test_points_to_voxels_to_submanifold_layer(gpu_handle):
     ref = F.conv3d(dense, w, padding=1)[0][:, ci[:, 0], ci[:, 1], ci[:, 2]].t()
     d1 = (y - ref).abs().sum() / ref.abs().sum()
     assert d1 <= 1e-5, float(d1)
+
+
+def test_small_channel_counts_are_padded_for_the_matrix_cores(gpu_handle):
+    """5 -> 12 channels (padded to 16 -> 16 inside the layer): values and gradients against the
+    rulebook-driven float64 formula."""
+    import torch
+    from mluop_hip import nn as spnn
+    rng = np.random.default_rng(24)
+    batch, space, L = 1, (9, 10, 11), 400
+    idx = random_voxels(rng, batch, space, L)
+    feats = torch.from_numpy(rng.standard_normal((L, 5)).astype(np.float32)).cuda().requires_grad_(True)
+    torch.manual_seed(7)
+    layer = spnn.SubMConv3d(5, 12, 3).cuda()
+    st = spnn.SparseTensor(feats, torch.from_numpy(idx).cuda(), space, batch)
+    y = layer(st).features
+    assert tuple(y.shape) == (L, 12)
+    g = torch.from_numpy(rng.standard_normal((L, 12)).astype(np.float32)).cuda()
+    (y * g).sum().backward()
+    rb = layer._rulebook(st)
+    pairs = rb.pairs.cpu().numpy()
+    w = layer.weight.detach().cpu().double().numpy().reshape(27, 5, 12)
+    x64, g64 = feats.detach().cpu().double().numpy(), g.cpu().double().numpy()
+    ref, dx, dw = np.zeros((L, 12)), np.zeros((L, 5)), np.zeros((27, 5, 12))
+    for k in range(27):
+        n = rb.indice_num[k]
+        i, o = pairs[k, 0, :n], pairs[k, 1, :n]
+        np.add.at(ref, o, x64[i] @ w[k])
+        np.add.at(dx, i, g64[o] @ w[k].T)
+        dw[k] = x64[i].T @ g64[o]
+    for got, want, what in ((y.detach().cpu().numpy(), ref, "forward"), (feats.grad.cpu().numpy(), dx, "grad x"),
+                            (layer.weight.grad.cpu().numpy().reshape(27, 5, 12), dw, "grad w")):
+        d1 = np.abs(got - want).sum() / np.abs(want).sum()
+        assert d1 <= 1e-5, (what, d1)
