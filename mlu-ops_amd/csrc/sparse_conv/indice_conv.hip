@@ -468,17 +468,27 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
     } else if (nblk > 0) {
       vec8 wnext[G][KB][NB];
       uint32_t dnext[G];
+      int k_held[G];  // offset whose fragments slot g holds: a dense offset fills several
+                      // batches in a row and its fragments are fetched once
+#pragma unroll
+      for (int g = 0; g < G; ++g) k_held[g] = -1;
       auto fetch_batch = [&](int b0) {
         const uint32_t dv = s_blk[b0 + (lane & (G - 1))];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
           dnext[g] = (uint32_t)__builtin_amdgcn_readlane((int)dv, g);
-          const char *bk = b_base + (size_t)(kc + (int)(dnext[g] >> 24)) * kBytesPerOffset;
+          const int kk = (int)(dnext[g] >> 24);
+          // (single-block batches only: with several slots the branch costs the other
+          // instances more than the saved loads)
+          if (G > 1 || kk != k_held[g]) {
+            k_held[g] = kk;
+            const char *bk = b_base + (size_t)(kc + kk) * kBytesPerOffset;
 #pragma unroll
-          for (int kb = 0; kb < KB; ++kb)
+            for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-              wnext[g][kb][nb] = *reinterpret_cast<const vec8 *>(bk + (nb * KB + kb) * 1024);
+              for (int nb = 0; nb < NB; ++nb)
+                wnext[g][kb][nb] = *reinterpret_cast<const vec8 *>(bk + (nb * KB + kb) * 1024);
+          }
         }
       };
       fetch_batch(0);
