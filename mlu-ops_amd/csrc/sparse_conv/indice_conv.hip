@@ -572,6 +572,201 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   }
 }
 
+// ---- MFMA gather convolution for dense rulebooks -------------------------------
+//
+// When most rows of a tile have a partner at most offsets, compacting pairs buys
+// little and the fp32 accumulate in LDS (a 16-byte read-modify-write per lane and
+// 16 result columns, on arbitrary rows: bank conflicts) is what the kernel above
+// spends its time on.  Here a tile is 64 result rows = four groups of 16, the
+// partner rows of one offset are staged at their result-row position, and a wave
+// accumulates 32 result columns of two row groups in registers over all offsets:
+// no accumulator traffic at all.  A lane whose row has no partner at the
+// offset multiplies zeros; a row group none of whose rows has one is skipped.
+//
+// The partner rows travel from global memory straight into LDS (16-byte
+// `global_load_lds`: lane l of a wave-load writes bytes [16 l, 16 l + 16) of a
+// 1 KiB block, no registers involved), requested kDenseDepth - 1 offsets ahead by
+// the multiplying waves themselves: there are no fetching waves and one barrier
+// per offset.  Because those blocks are unpadded, a row's 16-byte pieces are
+// stored permuted (piece ^ f(row)) so that the 16 rows an operand read touches
+// fall into 16 different bank groups.
+constexpr int kDenseTileRows = 64;
+constexpr int kDenseChunk = 32;  // offsets whose row-map slice is resident in LDS at once
+constexpr int kDenseDepth = 4;   // stage buffers: offsets i .. i+3 are resident or in flight
+constexpr int kDenseRowSplit = 2;  // waves along the rows of a tile
+constexpr int denseThreads(int C) { return 64 * (C / 32) * kDenseRowSplit; }
+
+template <typename E, int Q, int C>
+__global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
+    const typename E::storage *A, const typename E::storage *packedW, const int32_t *map, int R,
+    int K, int ldc, typename E::storage *result) {
+  typedef typename E::vec8 vec8;
+  typedef typename E::storage S;
+  constexpr int NB = 2;                      // 16-column blocks per wave
+  constexpr int CW = C / 32;                 // waves along the columns
+  constexpr int RS = kDenseRowSplit;         // waves along the rows
+  constexpr int WAVES = CW * RS;
+  constexpr int GPW = kDenseTileRows / 16 / RS;  // row groups per wave
+  constexpr int TR = kDenseTileRows;
+  constexpr int KC = kDenseChunk;
+  constexpr int D = kDenseDepth;
+  constexpr int KB = Q / E::kChunk;
+  constexpr int ROW_BYTES = Q * (int)sizeof(S);
+  constexpr int PPR = ROW_BYTES / 16;        // 16-byte pieces per row
+  constexpr int RP256 = 256 / ROW_BYTES;     // rows per 256 bytes (one pass over all banks)
+  constexpr int LOADS = TR * PPR / 64;       // wave-loads per offset
+  constexpr int LPW = LOADS / WAVES;         // every wave issues at least this many of them
+  constexpr int LPW_MAX = (LOADS + WAVES - 1) / WAVES;
+  static_assert(Q % E::kChunk == 0 && C % 32 == 0, "whole fragments and column pairs");
+  static_assert(ROW_BYTES <= 256 && 256 % ROW_BYTES == 0, "rows of 32 to 256 bytes");
+  static_assert((D - 2) * (LPW + KB * NB) <= 63, "fits the load counter");
+
+  __shared__ __attribute__((aligned(1024))) char s_stage[D][TR * ROW_BYTES];
+  __shared__ int s_map[KC][TR];   // partner row of (offset in chunk, tile row) or -1
+  __shared__ int s_list[KC];      // offsets of the chunk that have a pair in this tile
+  __shared__ int s_has[KC];
+  __shared__ int s_count;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tiles_per_xcd = gridDim.x >> 3;  // neighbouring tiles on one XCD, as above
+  const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
+  const int r0 = tile * TR;
+  if (r0 >= R) return;
+  const int col_group = blockIdx.y;
+  const int pair = lane & 15;
+  const int quad = lane >> 4;
+  const char *a_bytes = reinterpret_cast<const char *>(A);
+  const int cw = wave % CW;                  // this wave's column pair
+  const int g0 = (wave / CW) * GPW;          // and its first row group
+  const char *b_base = reinterpret_cast<const char *>(packedW) +
+                       ((size_t)(col_group * (C / 16) + cw * NB) * KB * 64 + lane) * 16;
+  const uint32_t kBytesPerOffset = (uint32_t)(ldc / 16) * KB * 64 * 16;
+
+  float4v acc[GPW][NB];
+#pragma unroll
+  for (int g = 0; g < GPW; ++g)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[g][nb] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  for (int kc = 0; kc < K; kc += KC) {
+    const int kn = (K - kc) < KC ? (K - kc) : KC;
+    __syncthreads();  // the chunk before is finished with s_map and the stage
+    for (int kk = wave; kk < kn; kk += WAVES) {
+      const int r = r0 + lane;
+      const int v = r < R ? map[(size_t)(kc + kk) * R + r] : -1;
+      s_map[kk][lane] = v;
+      const unsigned long long any = __ballot(v >= 0);
+      if (lane == 0) s_has[kk] = any != 0ull;
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const bool has = lane < kn && s_has[lane < kn ? lane : 0] != 0;
+      const unsigned long long m = __ballot(has);
+      if (has) s_list[__popcll(m & ((1ull << lane) - 1ull))] = lane;
+      if (lane == 0) s_count = __popcll(m);
+    }
+    __syncthreads();
+    const int items = s_count;
+    if (items == 0) continue;
+
+    // Requests the rows of one offset into its stage buffer.  Position p (in 16-byte
+    // units) of the buffer holds piece (p % PPR) ^ f(row) of row p / PPR; a row
+    // without a partner fetches row 0, which nobody reads.
+    auto request = [&](int item) {
+      const int kk = s_list[item];
+      char *buf = s_stage[item & (D - 1)];
+#pragma unroll
+      for (int t = 0; t < LPW_MAX; ++t) {
+        const int wl = wave + t * WAVES;
+        if (wl >= LOADS) break;
+        const int p = wl * 64 + lane;
+        const int row = p / PPR;
+        const int piece = (p % PPR) ^ ((row / RP256) & (PPR - 1));
+        const int src = s_map[kk][row];
+        const char *g = a_bytes + (size_t)(src < 0 ? 0 : src) * ROW_BYTES + piece * 16;
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void *)g,
+            (__attribute__((address_space(3))) void *)(buf + wl * 1024), 16, 0, 0);
+      }
+    };
+    vec8 wnext[KB][NB];
+    auto fetch_w = [&](int item) {
+      const char *bk = b_base + (size_t)(kc + s_list[item]) * kBytesPerOffset;
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          wnext[kb][nb] = *reinterpret_cast<const vec8 *>(bk + (nb * KB + kb) * 1024);
+    };
+#pragma unroll
+    for (int j = 0; j < D - 1; ++j)
+      if (j < items) request(j);
+    fetch_w(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // item 0 (and whatever else has arrived) is staged
+
+    for (int i = 0; i < items; ++i) {
+      vec8 wcur[KB][NB];
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) wcur[kb][nb] = wnext[kb][nb];
+      if (i + 1 < items) fetch_w(i + 1);
+      // buffer (i + D - 1) % D held item i - 1, which every wave left at the last barrier
+      const bool more = i + D - 1 < items;
+      if (more) request(i + D - 1);
+
+      const int kk = s_list[i];
+      const char *stage = s_stage[i & (D - 1)];
+#pragma unroll
+      for (int g = 0; g < GPW; ++g) {
+        const int row = (g0 + g) * 16 + pair;
+        const bool mine = s_map[kk][row] >= 0;
+        if (__ballot(mine) == 0ull) continue;  // no row of the group has a partner here
+        const char *arow = stage + row * ROW_BYTES;
+        const int swz = (row / RP256) & (PPR - 1);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          vec8 afr = *reinterpret_cast<const vec8 *>(arow + (((kb * 4 + quad) ^ swz) * 16));
+          if (!mine) afr = vec8{};
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) acc[g][nb] = E::mfma(wcur[kb][nb], afr, acc[g][nb]);
+        }
+      }
+      // Item i + 1 must have landed before anybody reads it.  Loads complete in order, and
+      // the last D - 2 iterations (this one included) each issued at least LPW row requests
+      // and KB * NB filter fragments, all of them after the requests of item i + 1 (nothing
+      // moves across the barrier below), so that many loads may stay in flight.  Waiting for
+      // fewer would also wait for the filter fragments of item i + 1, requested a moment ago.
+      // Near the end of the list nothing newer is in flight and everything is awaited.
+      if (more)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((D - 2) * (LPW + KB * NB)) : "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    }
+  }
+  // lane holds result columns 16*nb + 4*quad + (0..3) of row 16*g + pair
+#pragma unroll
+  for (int g = 0; g < GPW; ++g) {
+    const int r = r0 + (g0 + g) * 16 + pair;
+    if (r >= R) continue;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      S *dst = result + (size_t)r * ldc + col_group * C + cw * 32 + nb * 16 + quad * 4;
+      S tmp[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) E::store(&tmp[e], acc[g][nb][e]);
+      if constexpr (sizeof(S) == 2)
+        *reinterpret_cast<uint2 *>(dst) = *reinterpret_cast<const uint2 *>(tmp);
+      else
+        *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(tmp);
+    }
+  }
+}
+
 // ---- backward filter -------------------------------------------------------------
 // One block = 32 x 64 tile of dW[k] over a contiguous slice of the offset's pairs.
 template <typename E>
@@ -1061,6 +1256,68 @@ void launchMfma(const LaunchCtx &lc, int Q, int C, int tile_cols, const void *A,
   }
 }
 
+// The register-accumulating kernel pays when a quarter or more of all (row, offset)
+// slots hold a pair (below that, most of its multiplies are zeros); it takes 64
+// or 128 result columns and reduction channels of whole fragments.
+bool denseShapeOk(ElemType t, int Q, int C) {
+  const int chunk = t == ElemType::kFloat ? 16 : 32;
+  // fp32 rows of 128 channels leave no room for the double-buffered stage and the fragments
+  if (t == ElemType::kFloat && Q > 64) return false;
+  return (C == 64 || C == 128) && Q % chunk == 0 && (Q == 16 || Q == 32 || Q == 64 || Q == 128);
+}
+
+bool useDenseKernel(const ConvProblem &p, const GatherDims &d) {
+  if (!denseShapeOk(p.dtype, d.Q, d.C)) return false;
+  // MLUOP_SPCONV_DENSE=1 / 0 forces the choice (the parity tests run both kernels on one shape)
+  if (const char *e = getenv("MLUOP_SPCONV_DENSE")) return e[0] == '1';
+  // measured: 128 result columns gain (128 -> 128 at 0.73 pairs per slot: 250 us against
+  // 305 us), 64 result columns tie with the pair-list kernel
+  if (d.C != 128) return false;
+  double pairs = 0;
+  for (int k = 0; k < p.K; ++k) pairs += (double)p.indice_num[k];
+  return pairs >= 0.25 * (double)d.R * p.K;
+}
+
+template <typename E, int Q, int C>
+void launchDenseInstance(const LaunchCtx &lc, const void *A, const void *packed, const int32_t *map,
+                         int R, int K, void *result) {
+  const dim3 grid(((R + kDenseTileRows - 1) / kDenseTileRows + 7) / 8 * 8, 1);
+  lc.begin("gatherConvDense");
+  gatherConvDense<E, Q, C><<<grid, denseThreads(C), 0, lc.stream>>>(
+      static_cast<const typename E::storage *>(A), static_cast<const typename E::storage *>(packed),
+      map, R, K, C, static_cast<typename E::storage *>(result));
+  lc.end();
+}
+
+template <typename E>
+void launchDense(const LaunchCtx &lc, int Q, int C, const void *A, const void *packed,
+                 const int32_t *map, int R, int K, void *result) {
+  constexpr bool is_float = std::is_same<E, FloatElem>::value;
+#define DENSE_CASE(q)                                                                      \
+  case q:                                                                                  \
+    if (C == 64) launchDenseInstance<E, q, 64>(lc, A, packed, map, R, K, result);          \
+    else launchDenseInstance<E, q, 128>(lc, A, packed, map, R, K, result);                 \
+    break;
+  switch (Q) {
+    case 16:
+      if constexpr (is_float) {
+        if (C == 64) launchDenseInstance<E, 16, 64>(lc, A, packed, map, R, K, result);
+        else launchDenseInstance<E, 16, 128>(lc, A, packed, map, R, K, result);
+      }
+      break;
+    DENSE_CASE(32)
+    DENSE_CASE(64)
+    case 128:
+      if constexpr (!is_float) {
+        if (C == 64) launchDenseInstance<E, 128, 64>(lc, A, packed, map, R, K, result);
+        else launchDenseInstance<E, 128, 128>(lc, A, packed, map, R, K, result);
+      }
+      break;
+    default: break;
+  }
+#undef DENSE_CASE
+}
+
 void launchScatterRowMap(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d,
                          const GatherWorkspace &ws, const OffsetCounts &inl, int max_count) {
   if (max_count <= 0) return;
@@ -1090,7 +1347,10 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
         d.Q, d.C, static_cast<S *>(ws.packed));
     lc.end();
     launchScatterRowMap(lc, p, d, ws, inl, max_count);
-    launchMfma<E>(lc, d.Q, d.C, mfmaTileCols(p, d), gathered, ws.packed, ws.map, d.R, p.K, result);
+    if (useDenseKernel(p, d))
+      launchDense<E>(lc, d.Q, d.C, gathered, ws.packed, ws.map, d.R, p.K, result);
+    else
+      launchMfma<E>(lc, d.Q, d.C, mfmaTileCols(p, d), gathered, ws.packed, ws.map, d.R, p.K, result);
     return;
   }
   lc.begin("fillInt32");

@@ -111,6 +111,32 @@ def test_simt_path_matches_oracle_on_mfma_shapes(gpu_handle, dtype_name):
     run_all_ops(gpu_handle, c, dtype_name, force_simt=True, check=("fwd", "bwd_data"))
 
 
+DENSE_SHAPES = [
+    # the register-accumulating kernel takes 64 or 128 result columns; (8, 8, 8) with 300 voxels is dense
+    (1, (8, 8, 8), 300, (3, 3, 3), 64, 64, True, (1, 1, 1)),
+    (1, (8, 8, 8), 300, (3, 3, 3), 128, 128, True, (1, 1, 1)),
+    (2, (8, 8, 8), 500, (3, 3, 3), 32, 128, True, (1, 1, 1)),
+    (1, (8, 8, 8), 300, (3, 3, 3), 128, 64, False, (1, 1, 1)),
+    (1, (6, 6, 6), 150, (5, 5, 7), 64, 128, True, (1, 1, 1)),     # K = 175: six chunks of offsets
+    (1, (20, 20, 20), 130, (3, 3, 3), 64, 64, True, (1, 1, 1)),    # sparse input through the dense kernel
+]
+
+
+@pytest.mark.parametrize("shape", DENSE_SHAPES)
+@pytest.mark.parametrize("dtype_name", ["float32", "float16", "bfloat16"])
+def test_dense_kernel_matches_oracle(gpu_handle, shape, dtype_name):
+    """The same operators with the dense-rulebook kernel forced on (and, for comparison, off)."""
+    batch, space, L, ks, ci, co, sub_m, stride = shape
+    print("dense conv case", shape, dtype_name, flush=True)
+    c = conv_case(12, batch, space, L, ks, ci, co, sub_m, stride)
+    for force in ("1", "0"):
+        os.environ["MLUOP_SPCONV_DENSE"] = force
+        try:
+            run_all_ops(gpu_handle, c, dtype_name, check=("fwd", "bwd_data"))
+        finally:
+            os.environ.pop("MLUOP_SPCONV_DENSE", None)
+
+
 @pytest.mark.parametrize("layout_name", ["NDHWC", "NCDHW", "ARRAY"])
 @pytest.mark.parametrize("dtype_name", ["float32", "float16"])
 def test_forward_filter_layouts(gpu_handle, layout_name, dtype_name):
