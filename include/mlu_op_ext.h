@@ -27,6 +27,24 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtGetKernelTimingCount(mluOpHandle_t handle, i
 mluOpStatus_t MLUOP_WIN_API mluOpExtGetKernelTiming(mluOpHandle_t handle, int index,
                                                     const char **name, float *milliseconds);
 
+/* Modes of the indice-convolution operators that the reference rejects
+ * (kernels/sparse_conv/indice_convolution_forward/indice_convolution_forward.cpp:74-78,
+ * indice_convolution_backward_data.cpp:129-132, indice_convolution_backward_filter.cpp:185).
+ * Off by default: a fresh handle answers them with the reference's status codes.
+ * With `enable` non-zero the three operators accept
+ *   - inverse = 1: the sparse inverse convolution of the PyTorch sparse-convolution
+ *     stacks (spconv / mmcv SparseInverseConv3d).  The operator runs the rulebook of
+ *     its partner layer backwards: input-side rows (features, input_grad) are taken
+ *     through pair column 1, output-side rows (features_out, output_grad) through
+ *     column 0, so indice_pairs.dim[2] must equal the row count of the output-side
+ *     tensor (num_act_out for the forward operator) and the filter stays
+ *     W(k, ci, co) of this layer;
+ *   - a filters_grad descriptor tagged NHWC / NDHWC ([Co, (kd,) kh, kw, Ci]) or
+ *     NCHW / NCDHW ([Co, Ci, (kd,) kh, kw]) in mluOpIndiceConvolutionBackwardFilter,
+ *     written in that layout (the reference reads the dimensions positionally as
+ *     (kd,) kh, kw, Ci, Co whatever the tag says). */
+mluOpStatus_t MLUOP_WIN_API mluOpExtSetSparseConvExtendedModes(mluOpHandle_t handle, int enable);
+
 #if defined(__cplusplus)
 }
 #endif

@@ -136,6 +136,13 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelTiming(mluOpHandle_t handle, int en
   return MLUOP_STATUS_SUCCESS;
 }
 
+mluOpStatus_t MLUOP_WIN_API mluOpExtSetSparseConvExtendedModes(mluOpHandle_t handle,
+                                                               int enable) {
+  PARAM_CHECK("[mluOpExtSetSparseConvExtendedModes]", handle != NULL);
+  handle->sparse_conv_extended = enable != 0;
+  return MLUOP_STATUS_SUCCESS;
+}
+
 mluOpStatus_t MLUOP_WIN_API mluOpExtGetKernelTimingCount(mluOpHandle_t handle, int *count) {
   PARAM_CHECK("[mluOpExtGetKernelTimingCount]", handle != NULL);
   PARAM_CHECK("[mluOpExtGetKernelTimingCount]", count != NULL);

@@ -34,6 +34,9 @@ struct mluOpContext {
   mluOpAtomicsMode_t atomics_mode = MLUOP_ATOMICS_NOT_ALLOWED;
   int32_t *pinned_scalar = nullptr;  // 64-byte pinned host slot for read-backs
   mluop::KernelTimer timer;          // per-kernel event timing, off by default
+  // Modes the reference rejects (inverse convolution, filters_grad written in its
+  // tagged layout): off unless mluOpExtSetSparseConvExtendedModes switched them on.
+  bool sparse_conv_extended = false;
 
   // What the kernel launchers need: the stream, and the timer while it is on.
   mluop::LaunchCtx launchCtx() { return mluop::LaunchCtx(queue, timer.enabled ? &timer : nullptr); }

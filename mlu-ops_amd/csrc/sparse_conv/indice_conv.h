@@ -30,12 +30,19 @@ struct FilterView {
 struct ConvProblem {
   ElemType dtype;
   int K;          // kernel volume = indice_pairs.dim[0]
-  int L;          // indice_pairs.dim[2] = rows of the input-side tensor
-  int num_out;    // rows of the output-side tensor
+  int L;          // indice_pairs.dim[2] = rows of the tensor pair column 0 indexes
+  int num_out;    // rows of the tensor pair column 1 indexes
   int Ci;
   int Co;
   const int32_t *indice_pairs;  // device [K, 2, L]
   const int64_t *indice_num;    // host [K]
+  // Inverse convolution: the rulebook of the partner layer read backwards.
+  // Pair column 0 then names rows of the output-side tensors (L of them) and
+  // column 1 rows of the input-side tensors (num_out of them).
+  bool inverse = false;
+  // Backward filter only: element strides of dW(k, ci, co) in filters_grad;
+  // all zero = the positional [K, Ci, Co].
+  int64_t grad_stride_k = 0, grad_stride_ci = 0, grad_stride_co = 0;
 };
 
 // Which of the two gather-GEMM directions a launch computes.

@@ -768,15 +768,23 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
 }
 
 // ---- backward filter -------------------------------------------------------------
+// Where dW(k, ci, co) goes in filters_grad (element strides).
+struct GradLayout {
+  int64_t stride_k, stride_ci, stride_co;
+};
+__device__ __forceinline__ size_t gradOffset(const GradLayout &g, int k, int ci, int co) {
+  return (size_t)(k * g.stride_k + ci * g.stride_ci + co * g.stride_co);
+}
+
 // One block = 32 x 64 tile of dW[k] over a contiguous slice of the offset's pairs.
 template <typename E>
 __global__ __launch_bounds__(256) void backwardFilterSimt(const typename E::storage *X,
                                                           const typename E::storage *dY,
-                                                          const int32_t *pairs, int L, int n_in,
-                                                          int n_out, int Ci, int Co,
-                                                          OffsetCounts inl,
+                                                          const int32_t *pairs, int L,
+                                                          int x_col, int n_in, int n_out, int Ci,
+                                                          int Co, OffsetCounts inl,
                                                           const int32_t *dev_counts, int splits,
-                                                          float *partial,
+                                                          float *partial, GradLayout lay,
                                                           typename E::storage *dW) {
   constexpr int TI = 32, TO = 64, PC = 32;
   __shared__ float Xs[PC][TI + 1];
@@ -796,8 +804,8 @@ __global__ __launch_bounds__(256) void backwardFilterSimt(const typename E::stor
   per = (per + PC - 1) / PC * PC;
   const int p_begin = s * per;
   const int p_end = (p_begin + per) < n ? (p_begin + per) : n;
-  const int32_t *in_col = pairs + (size_t)k * 2 * L;
-  const int32_t *out_col = in_col + L;
+  const int32_t *in_col = pairs + ((size_t)k * 2 + x_col) * L;
+  const int32_t *out_col = pairs + ((size_t)k * 2 + 1 - x_col) * L;
   float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
   for (int p0 = p_begin; p0 < p_end; p0 += PC) {
     if (tid < PC) {
@@ -849,7 +857,7 @@ __global__ __launch_bounds__(256) void backwardFilterSimt(const typename E::stor
       if (co >= Co) continue;
       const size_t e = ((size_t)k * Ci + ci) * Co + co;
       if (splits == 1) {
-        E::store(dW + e, acc[i][j]);
+        E::store(dW + gradOffset(lay, k, ci, co), acc[i][j]);
       } else {
         partial[(size_t)s * K * Ci * Co + e] = acc[i][j];
       }
@@ -860,12 +868,15 @@ __global__ __launch_bounds__(256) void backwardFilterSimt(const typename E::stor
 // dW[e] = sum over splits, in split order, rounded once.
 template <typename E>
 __global__ __launch_bounds__(256) void reduceFilterPartials(const float *partial, size_t n,
-                                                            int splits,
+                                                            int splits, int Ci, int Co,
+                                                            GradLayout lay,
                                                             typename E::storage *dW) {
   for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (size_t)gridDim.x * 256) {
     float s = 0.f;
     for (int i = 0; i < splits; ++i) s += partial[(size_t)i * n + e];
-    E::store(dW + e, s);
+    const int co = (int)(e % Co);
+    const size_t kc = e / Co;
+    E::store(dW + gradOffset(lay, (int)(kc / Ci), (int)(kc % Ci), co), s);
   }
 }
 
@@ -896,7 +907,7 @@ constexpr int kFilterMaxSlices = 768;    // about three workgroups per CU
 template <typename E, int CI, int CO>
 __global__ __launch_bounds__(256) void backwardFilterMfma(
     const typename E::storage *X, const typename E::storage *dY, const int32_t *pairs, int L,
-    int n_in, int n_out, int K, SliceTable tab, int slice_len, float *partial) {
+    int x_col, int n_in, int n_out, int K, SliceTable tab, int slice_len, float *partial) {
   typedef typename E::vec8 vec8;
   typedef typename E::storage S;
   constexpr int SP = kFilterStepPairs;
@@ -929,8 +940,8 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int32_t *in_col = pairs + (size_t)k * 2 * L;
-  const int32_t *out_col = in_col + L;
+  const int32_t *in_col = pairs + ((size_t)k * 2 + x_col) * L;
+  const int32_t *out_col = pairs + ((size_t)k * 2 + 1 - x_col) * L;
 
   float4v acc[CBW][COB];
 #pragma unroll
@@ -1060,7 +1071,8 @@ constexpr int kSliceSumWaves = 16;
 template <typename E>
 __global__ __launch_bounds__(64 * kSliceSumWaves) void sliceSum(const float *partial,
                                                                 SliceTable tab, int slice_len,
-                                                                int tile_elems,
+                                                                int tile_elems, int Co,
+                                                                GradLayout lay,
                                                                 typename E::storage *dW) {
   constexpr int W = kSliceSumWaves;
   __shared__ float4v s_part[W][64];
@@ -1093,7 +1105,8 @@ __global__ __launch_bounds__(64 * kSliceSumWaves) void sliceSum(const float *par
 #pragma unroll
       for (int i = 0; i < W; i += 2 * span) t[i] += t[i + span];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) E::store(dW + (size_t)k * tile_elems + e + v, t[0][v]);
+    for (int v = 0; v < 4; ++v)
+      E::store(dW + gradOffset(lay, k, (e + v) / Co, (e + v) % Co), t[0][v]);
   }
 }
 
@@ -1133,14 +1146,24 @@ struct GatherDims {
   int Q;       // reduction channels
   int C;       // result channels
   int row_col, src_col;
+  bool filter_forward;  // B(k, q, c) = W(k, ci = q, co = c); otherwise its transpose
 };
 
 GatherDims gatherDims(const ConvProblem &p, GatherDirection dir) {
   GatherDims d;
-  if (dir == GatherDirection::kForward) {
-    d.R = p.num_out; d.n_src = p.L; d.Q = p.Ci; d.C = p.Co; d.row_col = 1; d.src_col = 0;
+  d.filter_forward = dir == GatherDirection::kForward;
+  if (d.filter_forward) {
+    d.Q = p.Ci; d.C = p.Co;
   } else {
-    d.R = p.L; d.n_src = p.num_out; d.Q = p.Co; d.C = p.Ci; d.row_col = 0; d.src_col = 1;
+    d.Q = p.Co; d.C = p.Ci;
+  }
+  // The result rows are the pair column the operator writes through: column 1
+  // for forward, column 0 for backward data, and the other way round for an
+  // inverse convolution, which runs its partner's rulebook backwards.
+  if (d.filter_forward != p.inverse) {
+    d.R = p.num_out; d.n_src = p.L; d.row_col = 1; d.src_col = 0;
+  } else {
+    d.R = p.L; d.n_src = p.num_out; d.row_col = 0; d.src_col = 1;
   }
   return d;
 }
@@ -1334,8 +1357,8 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
                        const void *gathered, const FilterView &f, bool use_mfma, void *result) {
   typedef typename E::storage S;
   // B(k, q, c): forward q = ci, c = co; backward data q = co, c = ci.
-  const int64_t sQ = d.row_col == 1 ? f.stride_ci : f.stride_co;
-  const int64_t sC = d.row_col == 1 ? f.stride_co : f.stride_ci;
+  const int64_t sQ = d.filter_forward ? f.stride_ci : f.stride_co;
+  const int64_t sC = d.filter_forward ? f.stride_co : f.stride_ci;
   const size_t map_elems = (size_t)p.K * d.R;
   if (use_mfma) {
     const size_t frags = (size_t)p.K * (d.C / 16) * ((d.Q + E::kChunk - 1) / E::kChunk) * 64;
@@ -1407,6 +1430,17 @@ FilterGradWorkspace carveFilterGrad(const ConvProblem &p, void *base) {
   return ws;
 }
 
+// filters_grad is [K, Ci, Co] unless the caller asked for another layout.
+GradLayout gradLayout(const ConvProblem &p) {
+  GradLayout g;
+  if (p.grad_stride_k == 0 && p.grad_stride_ci == 0 && p.grad_stride_co == 0) {
+    g.stride_k = (int64_t)p.Ci * p.Co; g.stride_ci = p.Co; g.stride_co = 1;
+  } else {
+    g.stride_k = p.grad_stride_k; g.stride_ci = p.grad_stride_ci; g.stride_co = p.grad_stride_co;
+  }
+  return g;
+}
+
 template <typename E, int CI, int CO>
 void launchFilterMfmaInstance(const LaunchCtx &lc, const ConvProblem &p, const SliceTable &tab,
                               int slice_len, int total_slices, float *partial, const void *features,
@@ -1416,11 +1450,12 @@ void launchFilterMfmaInstance(const LaunchCtx &lc, const ConvProblem &p, const S
   if (total_slices > 0)
     backwardFilterMfma<E, CI, CO><<<total_slices, 256, 0, lc.stream>>>(
         static_cast<const S *>(features), static_cast<const S *>(output_grad), p.indice_pairs,
-        p.L, p.L, p.num_out, p.K, tab, slice_len, partial);
+        p.L, p.inverse ? 1 : 0, p.inverse ? p.num_out : p.L, p.inverse ? p.L : p.num_out, p.K,
+        tab, slice_len, partial);
   lc.end();
   lc.begin("sliceSum");
   sliceSum<E><<<dim3(CI * CO / 256, p.K), 64 * kSliceSumWaves, 0, lc.stream>>>(
-      partial, tab, slice_len, CI * CO, static_cast<S *>(filters_grad));
+      partial, tab, slice_len, CI * CO, CO, gradLayout(p), static_cast<S *>(filters_grad));
   lc.end();
 }
 
@@ -1485,14 +1520,14 @@ void launchFilterGradTyped(const LaunchCtx &lc, const ConvProblem &p,
   lc.begin("backwardFilterSimt");
   backwardFilterSimt<E><<<grid, 256, 0, lc.stream>>>(
       static_cast<const S *>(features), static_cast<const S *>(output_grad), p.indice_pairs, p.L,
-      p.L, p.num_out, p.Ci, p.Co, inl, ws.dev_counts, ws.splits, ws.partial,
-      static_cast<S *>(filters_grad));
+      p.inverse ? 1 : 0, p.inverse ? p.num_out : p.L, p.inverse ? p.L : p.num_out, p.Ci, p.Co, inl,
+      ws.dev_counts, ws.splits, ws.partial, gradLayout(p), static_cast<S *>(filters_grad));
   lc.end();
   if (ws.splits > 1) {
     const size_t n = (size_t)p.K * p.Ci * p.Co;
     lc.begin("reduceFilterPartials");
-    reduceFilterPartials<E><<<gridFor(n), 256, 0, lc.stream>>>(ws.partial, n, ws.splits,
-                                                            static_cast<S *>(filters_grad));
+    reduceFilterPartials<E><<<gridFor(n), 256, 0, lc.stream>>>(
+        ws.partial, n, ws.splits, p.Ci, p.Co, gradLayout(p), static_cast<S *>(filters_grad));
     lc.end();
   }
 }

@@ -116,10 +116,18 @@ mluOpStatus_t foolCheckNoPtr(mluOpHandle_t handle, const mluOpTensorDescriptor_t
   for (int64_t kk = 0; kk < K; ++kk) {
     PARAM_CHECK(api, indice_num[kk] >= 0);
   }
-  if (inverse == 1) {
+  // Rejected as in the reference unless the handle was switched to the extended
+  // modes (mluOpExtSetSparseConvExtendedModes).
+  if (inverse == 1 && !handle->sparse_conv_extended) {
     MLUOP_LOG(ERROR) << api << " Not support inverse == 1 yet.";
     return MLUOP_STATUS_NOT_SUPPORTED;
   }
+  // The tensor pair column 0 indexes has indice_pairs.dim[2] rows: input_grad,
+  // or output_grad of an inverse convolution.
+  const mluOpTensorDescriptor_t col0_desc = inverse == 1 ? output_grad_desc : input_grad_desc;
+  const mluOpTensorDescriptor_t col1_desc = inverse == 1 ? input_grad_desc : output_grad_desc;
+  const char *col0_name = inverse == 1 ? "output_grad" : "input_grad";
+  const char *col1_name = inverse == 1 ? "input_grad" : "output_grad";
 
   if (K != indice_pairs_desc->getDimIndex(0)) {
     MLUOP_LOG(ERROR) << api << " The dims[0] of indice_pairs should be equal to kd*kh*kw.";
@@ -133,9 +141,9 @@ mluOpStatus_t foolCheckNoPtr(mluOpHandle_t handle, const mluOpTensorDescriptor_t
     MLUOP_LOG(ERROR) << api << " The dims[1] of input_grad should be equal to dxc of filters.";
     return MLUOP_STATUS_BAD_PARAM;
   }
-  if (input_grad_desc->getDimIndex(0) != indice_pairs_desc->getDimIndex(2)) {
-    MLUOP_LOG(ERROR) << api << " The dims[0] of input_grad should be equal to the dims[2] of "
-                     << "indice_pairs.";
+  if (col0_desc->getDimIndex(0) != indice_pairs_desc->getDimIndex(2)) {
+    MLUOP_LOG(ERROR) << api << " The dims[0] of " << col0_name
+                     << " should be equal to the dims[2] of indice_pairs.";
     return MLUOP_STATUS_BAD_PARAM;
   }
   const int64_t max_indice_num = K > 0 ? maxCount(indice_num, K) : 0;
@@ -156,9 +164,9 @@ mluOpStatus_t foolCheckNoPtr(mluOpHandle_t handle, const mluOpTensorDescriptor_t
       return MLUOP_STATUS_BAD_PARAM;
     }
   }
-  if (output_grad_desc->getDimIndex(0) < max_indice_num) {
-    MLUOP_LOG(ERROR) << api << " The dims[0] of output_grad should be larger than or equal to "
-                     << "the maximum number of indice_num.";
+  if (col1_desc->getDimIndex(0) < max_indice_num) {
+    MLUOP_LOG(ERROR) << api << " The dims[0] of " << col1_name
+                     << " should be larger than or equal to the maximum number of indice_num.";
     return MLUOP_STATUS_BAD_PARAM;
   }
   if (sub_m == 1 && K % 2 == 0) {
@@ -191,13 +199,15 @@ mluOpStatus_t foolCheckNoPtr(mluOpHandle_t handle, const mluOpTensorDescriptor_t
 ConvProblem makeProblem(const mluOpTensorDescriptor_t output_grad_desc,
                         const mluOpTensorDescriptor_t filters_desc,
                         const mluOpTensorDescriptor_t indice_pairs_desc,
-                        const int64_t indice_num[], const void *indice_pairs) {
+                        const mluOpTensorDescriptor_t input_grad_desc, const int64_t indice_num[],
+                        int64_t inverse, const void *indice_pairs) {
   const FilterDims fd = filterDims(filters_desc);
   ConvProblem p;
   p.dtype = toElemType(filters_desc->getDtype());
   p.K = (int)indice_pairs_desc->getDimIndex(0);
   p.L = (int)indice_pairs_desc->getDimIndex(2);
-  p.num_out = (int)output_grad_desc->getDimIndex(0);
+  p.inverse = inverse != 0;
+  p.num_out = (int)(p.inverse ? input_grad_desc : output_grad_desc)->getDimIndex(0);
   p.Ci = (int)fd.dxc;
   p.Co = (int)fd.dyc;
   p.indice_pairs = static_cast<const int32_t *>(indice_pairs);
@@ -253,7 +263,8 @@ mluOpStatus_t MLUOP_WIN_API mluOpGetIndiceConvolutionBackwardDataWorkspaceSize(
   if (st != MLUOP_STATUS_SUCCESS) return st;
   if (is_zero) return MLUOP_STATUS_SUCCESS;
   const ConvProblem p =
-      makeProblem(output_grad_desc, filters_desc, indice_pairs_desc, indice_num, nullptr);
+      makeProblem(output_grad_desc, filters_desc, indice_pairs_desc, input_grad_desc, indice_num,
+                  inverse, nullptr);
   *workspace_size =
       mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kBackwardData);
   return MLUOP_STATUS_SUCCESS;
@@ -282,7 +293,8 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardData(
   }
 
   const ConvProblem p =
-      makeProblem(output_grad_desc, filters_desc, indice_pairs_desc, indice_num, indice_pairs);
+      makeProblem(output_grad_desc, filters_desc, indice_pairs_desc, input_grad_desc, indice_num,
+                  inverse, indice_pairs);
   const size_t need =
       mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kBackwardData);
   if (workspace_size < need || workspace == NULL) {

@@ -65,6 +65,38 @@ mluOpStatus_t dtypeValid(const std::string &api, const mluOpTensorDescriptor_t f
   return MLUOP_STATUS_SUCCESS;
 }
 
+// Extents and element strides of dW(k, ci, co) in filters_grad.  The reference takes the
+// dimensions positionally as (kd,) kh, kw, Ci, Co whatever the layout tag says
+// (indice_convolution_backward_filter.cpp:227-242); with the extended modes on,
+// a tensor tagged N(D)HWC is [Co, (kd,) kh, kw, Ci] and one tagged NC(D)HW is
+// [Co, Ci, (kd,) kh, kw], as the forward and backward-data operators read their filters.
+struct GradDims {
+  int64_t K, ci, co;
+  int64_t stride_k, stride_ci, stride_co;
+};
+
+GradDims gradDims(const mluOpTensorDescriptor_t desc, bool extended) {
+  const int n = desc->getDim();
+  auto volume = [&](int first) {
+    int64_t v = 1;
+    for (int i = first; i < first + n - 2; ++i) v *= desc->getDimIndex(i);
+    return v;
+  };
+  const mluOpTensorLayout_t layout = desc->getLayout();
+  GradDims g;
+  if (extended && (layout == MLUOP_LAYOUT_NHWC || layout == MLUOP_LAYOUT_NDHWC)) {
+    g.co = desc->getDimIndex(0); g.ci = desc->getDimIndex(n - 1); g.K = volume(1);
+    g.stride_k = g.ci; g.stride_ci = 1; g.stride_co = g.K * g.ci;
+  } else if (extended && (layout == MLUOP_LAYOUT_NCHW || layout == MLUOP_LAYOUT_NCDHW)) {
+    g.co = desc->getDimIndex(0); g.ci = desc->getDimIndex(1); g.K = volume(2);
+    g.stride_k = 1; g.stride_ci = g.K; g.stride_co = g.ci * g.K;
+  } else {
+    g.ci = desc->getDimIndex(n - 2); g.co = desc->getDimIndex(n - 1); g.K = volume(0);
+    g.stride_k = g.ci * g.co; g.stride_ci = g.co; g.stride_co = 1;
+  }
+  return g;
+}
+
 mluOpStatus_t baseParamCheck(const std::string &api, mluOpHandle_t handle,
                              const mluOpTensorDescriptor_t features_desc,
                              const mluOpTensorDescriptor_t output_grad_desc,
@@ -77,7 +109,9 @@ mluOpStatus_t baseParamCheck(const std::string &api, mluOpHandle_t handle,
   PARAM_CHECK(api, indice_pairs_desc != nullptr);
   PARAM_CHECK(api, filters_grad_desc != nullptr);
   PARAM_CHECK(api, indice_num != nullptr);
-  PARAM_CHECK(api, inverse == 0);
+  // inverse = 1 is a bad parameter in the reference, and here unless the handle was
+  // switched to the extended modes (mluOpExtSetSparseConvExtendedModes).
+  PARAM_CHECK(api, inverse == 0 || (inverse == 1 && handle->sparse_conv_extended));
 
   STRIDE_TENSOR_CHECK(api, features_desc, "features_desc must be contiguous");
   STRIDE_TENSOR_CHECK(api, output_grad_desc, "output_grad_desc must be contiguous");
@@ -108,17 +142,13 @@ mluOpStatus_t baseParamCheck(const std::string &api, mluOpHandle_t handle,
     shape_check = false;
   }
   if (shape_check) {
-    // filters_grad is (kd,)kh,kw,Ci,Co positionally, whatever its layout tag.
-    const int n = filters_grad_desc->getDim();
-    const int64_t ci = filters_grad_desc->getDimIndex(n - 2);
-    const int64_t co = filters_grad_desc->getDimIndex(n - 1);
-    const int64_t kd = n == 4 ? 1 : filters_grad_desc->getDimIndex(0);
-    const int64_t kh = n == 4 ? filters_grad_desc->getDimIndex(0) : filters_grad_desc->getDimIndex(1);
-    const int64_t kw = n == 4 ? filters_grad_desc->getDimIndex(1) : filters_grad_desc->getDimIndex(2);
-    if (ci != features_desc->getDimIndex(1) || co != output_grad_desc->getDimIndex(1) ||
-        features_desc->getDimIndex(0) != indice_pairs_desc->getDimIndex(2) ||
-        2 != indice_pairs_desc->getDimIndex(1) ||
-        kd * kh * kw != indice_pairs_desc->getDimIndex(0)) {
+    const GradDims g = gradDims(filters_grad_desc, handle->sparse_conv_extended);
+    // indice_pairs.dim[2] is the row count of the tensor pair column 0 indexes:
+    // features, or output_grad of an inverse convolution.
+    const mluOpTensorDescriptor_t col0_desc = inverse == 1 ? output_grad_desc : features_desc;
+    if (g.ci != features_desc->getDimIndex(1) || g.co != output_grad_desc->getDimIndex(1) ||
+        col0_desc->getDimIndex(0) != indice_pairs_desc->getDimIndex(2) ||
+        2 != indice_pairs_desc->getDimIndex(1) || g.K != indice_pairs_desc->getDimIndex(0)) {
       shape_check = false;
     }
     PARAM_CHECK_LE(api, indice_pairs_desc->getDimIndex(2), INDICE_IN_LARGE_TENSOR_NUM);
@@ -136,15 +166,21 @@ bool anyZeroElement(const mluOpTensorDescriptor_t a, const mluOpTensorDescriptor
          c->getTotalElementNum() == 0 || d->getTotalElementNum() == 0;
 }
 
-ConvProblem makeProblem(const mluOpTensorDescriptor_t features_desc,
+ConvProblem makeProblem(mluOpHandle_t handle, const mluOpTensorDescriptor_t features_desc,
                         const mluOpTensorDescriptor_t output_grad_desc,
                         const mluOpTensorDescriptor_t indice_pairs_desc,
-                        const int64_t indice_num[], const void *indice_pairs) {
+                        const mluOpTensorDescriptor_t filters_grad_desc,
+                        const int64_t indice_num[], int64_t inverse, const void *indice_pairs) {
   ConvProblem p;
   p.dtype = toElemType(features_desc->getDtype());
   p.K = (int)indice_pairs_desc->getDimIndex(0);
   p.L = (int)indice_pairs_desc->getDimIndex(2);
-  p.num_out = (int)output_grad_desc->getDimIndex(0);
+  p.inverse = inverse != 0;
+  p.num_out = (int)(p.inverse ? features_desc : output_grad_desc)->getDimIndex(0);
+  const GradDims g = gradDims(filters_grad_desc, handle->sparse_conv_extended);
+  p.grad_stride_k = g.stride_k;
+  p.grad_stride_ci = g.stride_ci;
+  p.grad_stride_co = g.stride_co;
   p.Ci = (int)features_desc->getDimIndex(1);
   p.Co = (int)output_grad_desc->getDimIndex(1);
   p.indice_pairs = static_cast<const int32_t *>(indice_pairs);
@@ -172,7 +208,8 @@ mluOpStatus_t MLUOP_WIN_API mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize
     return MLUOP_STATUS_SUCCESS;
   }
   const ConvProblem p =
-      makeProblem(features_desc, output_grad_desc, indice_pairs_desc, indice_num, nullptr);
+      makeProblem(handle, features_desc, output_grad_desc, indice_pairs_desc, filters_grad_desc,
+                  indice_num, inverse, nullptr);
   *size = mluop::sparse_conv::backwardFilterWorkspaceBytes(p);
   return MLUOP_STATUS_SUCCESS;
 }
@@ -199,7 +236,8 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardFilter(
     PARAM_CHECK(api, workspace != nullptr);
   }
   const ConvProblem p =
-      makeProblem(features_desc, output_grad_desc, indice_pairs_desc, indice_num, indice_pairs);
+      makeProblem(handle, features_desc, output_grad_desc, indice_pairs_desc, filters_grad_desc,
+                  indice_num, inverse, indice_pairs);
   const size_t need = mluop::sparse_conv::backwardFilterWorkspaceBytes(p);
   if (workspace_size < need || (need > 0 && workspace == nullptr)) {
     MLUOP_LOG(ERROR) << api << " workspace of " << workspace_size

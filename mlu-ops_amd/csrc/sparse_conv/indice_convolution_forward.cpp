@@ -71,7 +71,9 @@ mluOpStatus_t foolProof(const std::string &api, mluOpHandle_t handle,
 
   PARAM_CHECK(api, sub_m == 0 || sub_m == 1);
   PARAM_CHECK(api, inverse == 0 || inverse == 1);
-  if (inverse != 0) {
+  // The reference rejects inverse = 1; so does this library unless the handle
+  // was switched to the extended modes (mluOpExtSetSparseConvExtendedModes).
+  if (inverse != 0 && !handle->sparse_conv_extended) {
     MLUOP_LOG(ERROR) << api << " inverse is: " << inverse << ", which is not supported now.";
     return MLUOP_STATUS_NOT_SUPPORTED;
   }
@@ -114,7 +116,13 @@ mluOpStatus_t foolProof(const std::string &api, mluOpHandle_t handle,
   }
 
   const FilterDims fd = forwardFilterDims(filters_desc);
-  PARAM_CHECK(api, features_desc->getDimIndex(0) == indice_pairs_desc->getDimIndex(2));
+  // indice_pairs.dim[2] is the row count of the tensor pair column 0 indexes:
+  // the input features, or the output of an inverse convolution.
+  if (inverse == 0) {
+    PARAM_CHECK(api, features_desc->getDimIndex(0) == indice_pairs_desc->getDimIndex(2));
+  } else {
+    PARAM_CHECK(api, num_act_out == indice_pairs_desc->getDimIndex(2));
+  }
   PARAM_CHECK(api, features_desc->getDimIndex(1) == fd.ci);
   PARAM_CHECK(api, indice_pairs_desc->getDimIndex(0) == fd.num_filter);
   PARAM_CHECK(api, indice_pairs_desc->getDimIndex(1) == 2);
@@ -123,7 +131,9 @@ mluOpStatus_t foolProof(const std::string &api, mluOpHandle_t handle,
 
   for (int64_t i = 0; i < fd.num_filter; ++i) {
     std::string where = "i: " + std::to_string(i) + ".";
-    PARAM_CHECK_V2(api, indice_num[i] >= 0 && indice_num[i] <= features_desc->getDimIndex(0),
+    PARAM_CHECK_V2(api,
+                   indice_num[i] >= 0 && indice_num[i] <= indice_pairs_desc->getDimIndex(2) &&
+                       indice_num[i] <= features_desc->getDimIndex(0),
                    where);
   }
   return MLUOP_STATUS_SUCCESS;
@@ -138,14 +148,15 @@ bool anyZeroElement(const mluOpTensorDescriptor_t a, const mluOpTensorDescriptor
 ConvProblem makeProblem(const mluOpTensorDescriptor_t features_desc,
                         const mluOpTensorDescriptor_t filters_desc,
                         const mluOpTensorDescriptor_t indice_pairs_desc,
-                        const int64_t indice_num[], int64_t num_act_out,
+                        const int64_t indice_num[], int64_t num_act_out, int64_t inverse,
                         const void *indice_pairs) {
   const FilterDims fd = forwardFilterDims(filters_desc);
   ConvProblem p;
   p.dtype = toElemType(features_desc->getDtype());
   p.K = (int)indice_pairs_desc->getDimIndex(0);
   p.L = (int)indice_pairs_desc->getDimIndex(2);
-  p.num_out = (int)num_act_out;
+  p.inverse = inverse != 0;
+  p.num_out = p.inverse ? (int)features_desc->getDimIndex(0) : (int)num_act_out;
   p.Ci = (int)fd.ci;
   p.Co = (int)fd.co;
   p.indice_pairs = static_cast<const int32_t *>(indice_pairs);
@@ -197,7 +208,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpGetIndiceConvolutionForwardWorkspaceSize(
   }
   PARAM_CHECK(api, size != nullptr);
   const ConvProblem p = makeProblem(features_desc, filters_desc, indice_pairs_desc, indice_num,
-                                    num_act_out, nullptr);
+                                    num_act_out, inverse, nullptr);
   *size = mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kForward);
   return MLUOP_STATUS_SUCCESS;
 }
@@ -225,7 +236,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionForward(
   }
 
   const ConvProblem p = makeProblem(features_desc, filters_desc, indice_pairs_desc, indice_num,
-                                    num_act_out, indice_pairs);
+                                    num_act_out, inverse, indice_pairs);
   const size_t need = mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kForward);
   if (workspace_size < need || workspace == nullptr) {
     MLUOP_LOG(ERROR) << api << " workspace of " << workspace_size

@@ -120,6 +120,7 @@ SIGNATURES = {
                        ctypes.c_size_t, _vp, _vp]),
     # mlu_op_ext.h
     "mluOpExtSetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "mluOpExtSetSparseConvExtendedModes": (ctypes.c_int, [_vp, ctypes.c_int]),
     "mluOpExtGetKernelTimingCount": (ctypes.c_int, [_vp, _ip]),
     "mluOpExtGetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int, ctypes.POINTER(ctypes.c_char_p),
                                                ctypes.POINTER(ctypes.c_float)]),
@@ -176,6 +177,10 @@ class Handle:
 
     def set_kernel_timing(self, enable):
         check(lib().mluOpExtSetKernelTiming(self.ptr, 1 if enable else 0))
+
+    def set_extended_modes(self, enable):
+        """Accept inverse = 1 and tagged filters_grad layouts, which the reference rejects."""
+        check(lib().mluOpExtSetSparseConvExtendedModes(self.ptr, 1 if enable else 0))
 
     def kernel_timings(self):
         """[(kernel name, milliseconds)] per launch since timing was enabled (waits for the queue)."""
@@ -360,15 +365,17 @@ def indice_conv_forward(handle, features, filters, filters_layout, indice_pairs,
 
 
 def indice_conv_backward_data(handle, output_grad, filters, filters_layout, indice_pairs,
-                              indice_num_host, sub_m, ci, inverse=0):
+                              indice_num_host, sub_m, ci, inverse=0, rows=None):
+    """input_grad [rows, ci]; rows = indice_pairs.shape[2] unless the convolution is an inverse one."""
     torch = _torch()
     code = torch_dtype_code(output_grad.dtype)
     K, _, L = indice_pairs.shape
-    dx = torch.empty((L, ci), dtype=output_grad.dtype, device=output_grad.device)
+    rows = L if rows is None else int(rows)
+    dx = torch.empty((rows, ci), dtype=output_grad.dtype, device=output_grad.device)
     d_dy = TensorDescriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
     d_filt = TensorDescriptor(filters_layout, code, list(filters.shape))
     d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
-    d_dx = TensorDescriptor(LAYOUT_ARRAY, code, [L, ci])
+    d_dx = TensorDescriptor(LAYOUT_ARRAY, code, [rows, ci])
     counts = _host_counts(indice_num_host)
     size = ctypes.c_size_t(0)
     check(lib().mluOpGetIndiceConvolutionBackwardDataWorkspaceSize(
@@ -383,17 +390,25 @@ def indice_conv_backward_data(handle, output_grad, filters, filters_layout, indi
 
 
 def indice_conv_backward_filter(handle, features, output_grad, indice_pairs, indice_num_host,
-                                filter_space, sub_m, inverse=0, onchip_float=True):
-    """Returns filters_grad laid out [kd, kh, kw, Ci, Co]."""
+                                filter_space, sub_m, inverse=0, onchip_float=True,
+                                grad_layout=LAYOUT_ARRAY):
+    """Returns filters_grad laid out [kd, kh, kw, Ci, Co]; with the handle's extended modes on,
+    grad_layout NDHWC gives [Co, kd, kh, kw, Ci] and NCDHW [Co, Ci, kd, kh, kw]."""
     torch = _torch()
     code = torch_dtype_code(features.dtype)
     K, _, L = indice_pairs.shape
     ci, co = features.shape[1], output_grad.shape[1]
-    dw = torch.empty(tuple(filter_space) + (ci, co), dtype=features.dtype, device=features.device)
+    if grad_layout in (LAYOUT_NDHWC, LAYOUT_NHWC):
+        shape = (co,) + tuple(filter_space) + (ci,)
+    elif grad_layout in (LAYOUT_NCDHW, LAYOUT_NCHW):
+        shape = (co, ci) + tuple(filter_space)
+    else:
+        shape = tuple(filter_space) + (ci, co)
+    dw = torch.empty(shape, dtype=features.dtype, device=features.device)
     d_x = TensorDescriptor(LAYOUT_ARRAY, code, list(features.shape))
     d_dy = TensorDescriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
     d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
-    d_dw = TensorDescriptor(LAYOUT_ARRAY, code, list(dw.shape),
+    d_dw = TensorDescriptor(grad_layout, code, list(dw.shape),
                             onchip_dtype=DTYPE_FLOAT if onchip_float else None)
     counts = _host_counts(indice_num_host)
     size = ctypes.c_size_t(0)

@@ -1,7 +1,8 @@
 """PyTorch caller layer over the C API: the call sequence mmcv's sparse-conv ops run against
 mlu-ops (descriptor -> workspace size -> mluOpGetIndicePairs -> num_act_out -> device-to-host
 copy of indice_num -> the three indice-convolution operators), wrapped in an autograd function and
-two modules, `SubMConv3d` and `SparseConv3d`.
+the modules `SubMConv3d`, `SparseConv3d` and `SparseInverseConv3d` (the last one through the
+library's extended modes, which the reference does not have).
 
 A `SparseTensor` carries features [L, C], int32 indices [L, 4] = (n, d, h, w), the spatial shape
 and the batch size, plus a cache of rulebooks keyed by `indice_key`, so that stacked submanifold
@@ -26,13 +27,17 @@ def _handle():
     key = (torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream)
     if key not in _handles:
         _handles[key] = make_handle_on_current_stream()
+        _handles[key].set_extended_modes(True)  # SparseInverseConv3d runs the operators with inverse = 1
     return _handles[key]
 
 
 class Rulebook:
     """indice_pairs [K,2,L] (device), indice_num as host ints, out_indices, num_act_out."""
 
-    def __init__(self, pairs, out_indices, indice_num_host, num_act_out, filter_space, sub_m, out_space):
+    def __init__(self, pairs, out_indices, indice_num_host, num_act_out, filter_space, sub_m, out_space,
+                 in_indices=None, in_space=None):
+        self.in_indices = in_indices  # what an inverse convolution over this rulebook gives back
+        self.in_space = None if in_space is None else tuple(in_space)
         self.pairs = pairs
         self.out_indices = out_indices
         self.indice_num = indice_num_host
@@ -67,14 +72,20 @@ class SparseTensor:
 
 class _IndiceConv(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, features, weight, rulebook):
+    def forward(ctx, features, weight, rulebook, inverse=False):
         handle = _handle()
         features = features.contiguous()
         weight = weight.contiguous()
-        out = indice_conv_forward(handle, features, weight, LAYOUT_ARRAY, rulebook.pairs, rulebook.indice_num,
-                                  rulebook.num_act_out, rulebook.sub_m)
+        if inverse:
+            # the partner layer's rulebook backwards: one output row per input row of the partner
+            out = indice_conv_forward(handle, features, weight, LAYOUT_ARRAY, rulebook.pairs, rulebook.indice_num,
+                                      rulebook.pairs.shape[2], False, inverse=1)
+        else:
+            out = indice_conv_forward(handle, features, weight, LAYOUT_ARRAY, rulebook.pairs,
+                                      rulebook.indice_num, rulebook.num_act_out, rulebook.sub_m)
         ctx.save_for_backward(features, weight)
         ctx.rulebook = rulebook
+        ctx.inverse = inverse
         return out
 
     @staticmethod
@@ -84,13 +95,15 @@ class _IndiceConv(torch.autograd.Function):
         handle = _handle()
         grad_out = grad_out.contiguous()
         grad_features = grad_weight = None
+        inverse, sub_m = (1, False) if ctx.inverse else (0, rb.sub_m)
         if ctx.needs_input_grad[0]:
             grad_features = indice_conv_backward_data(handle, grad_out, weight, LAYOUT_ARRAY, rb.pairs,
-                                                      rb.indice_num, rb.sub_m, features.shape[1])
+                                                      rb.indice_num, sub_m, features.shape[1], inverse=inverse,
+                                                      rows=features.shape[0])
         if ctx.needs_input_grad[1]:
             grad_weight = indice_conv_backward_filter(handle, features, grad_out, rb.pairs, rb.indice_num,
-                                                      rb.filter_space, rb.sub_m)
-        return grad_features, grad_weight, None
+                                                      rb.filter_space, sub_m, inverse=inverse)
+        return grad_features, grad_weight, None, None
 
 
 def _mfma_channels(c):
@@ -106,6 +119,8 @@ def _triple(v):
 
 
 class _ConvBase(torch.nn.Module):
+    inverse = False
+
     def __init__(self, in_channels, out_channels, kernel_size, stride, padding, dilation, sub_m, bias,
                  indice_key):
         super().__init__()
@@ -135,10 +150,16 @@ class _ConvBase(torch.nn.Module):
             self.stride, self.dilation, self.sub_m)
         # the operators take indice_num as host int64: one device-to-host copy per rulebook
         rb = Rulebook(pairs, out_indices[:n_out], num.cpu().tolist(), n_out, self.kernel_size, self.sub_m,
-                      out_space)
+                      out_space, in_indices=x.indices, in_space=x.spatial_shape)
         if self.indice_key is not None:
             x.rulebooks[self.indice_key] = rb
         return rb
+
+    def _result(self, x, rb, feats):
+        if self.sub_m:
+            return x.replace_features(feats)
+        # the cache travels on, so that an inverse layer downstream finds this rulebook by its key
+        return SparseTensor(feats, rb.out_indices.contiguous(), rb.out_space, x.batch_size, x.rulebooks)
 
     def forward(self, x):
         rb = self._rulebook(x)
@@ -151,14 +172,12 @@ class _ConvBase(torch.nn.Module):
         if ci != self.in_channels or co != self.out_channels:
             feats = torch.nn.functional.pad(feats, (0, ci - self.in_channels))
             weight = torch.nn.functional.pad(weight, (0, co - self.out_channels, 0, ci - self.in_channels))
-        feats = _IndiceConv.apply(feats, weight, rb)
+        feats = _IndiceConv.apply(feats, weight, rb, self.inverse)
         if co != self.out_channels:
             feats = feats[:, :self.out_channels]
         if self.bias is not None:
             feats = feats + self.bias.to(feats.dtype)
-        if self.sub_m:
-            return x.replace_features(feats)
-        return SparseTensor(feats, rb.out_indices.contiguous(), rb.out_space, x.batch_size)
+        return self._result(x, rb, feats)
 
 
 class SubMConv3d(_ConvBase):
@@ -178,6 +197,27 @@ class SparseConv3d(_ConvBase):
                  indice_key=None):
         super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, False, bias,
                          indice_key)
+
+
+class SparseInverseConv3d(_ConvBase):
+    """Inverse of the `SparseConv3d` that cached its rulebook under `indice_key`: takes a tensor on that
+    layer's output cells back to its input cells (spconv / mmcv SparseInverseConv3d).  The rulebook
+    is read backwards; the filter is this layer's own [kd, kh, kw, Ci, Co]."""
+
+    inverse = True
+
+    def __init__(self, in_channels, out_channels, kernel_size, indice_key, bias=False):
+        super().__init__(in_channels, out_channels, kernel_size, 1, 0, 1, False, bias, indice_key)
+
+    def _rulebook(self, x):
+        rb = x.rulebooks.get(self.indice_key)
+        assert rb is not None, "no layer has cached a rulebook under indice_key %r" % (self.indice_key,)
+        assert rb.filter_space == tuple(self.kernel_size) and not rb.sub_m
+        assert rb.num_act_out == x.features.shape[0], "the input does not live on the partner layer's output"
+        return rb
+
+    def _result(self, x, rb, feats):
+        return SparseTensor(feats, rb.in_indices, rb.in_space, x.batch_size, x.rulebooks)
 
 
 class Voxelization(torch.nn.Module):

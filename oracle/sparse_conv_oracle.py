@@ -81,14 +81,25 @@ def filters_to_kcico(filters, layout, K, ci, co):
     return out
 
 
+def _swapped(indice_pairs):
+    """The rulebook with its two pair columns exchanged."""
+    return np.ascontiguousarray(_i32(indice_pairs)[:, ::-1, :])
+
+
 def _num64(indice_num):
     return np.ascontiguousarray(indice_num, dtype=np.int64)
 
 
-def forward(features, filters_kcico, indice_pairs, indice_num, num_act_out):
+def forward(features, filters_kcico, indice_pairs, indice_num, num_act_out, inverse=False):
+    """inverse=True is the sparse inverse convolution, which the reference does not
+    implement (indice_convolution_forward.cpp:74-78 rejects it): the operator of the PyTorch
+    sparse-convolution stacks the reference serves (spconv 1.x indice_conv / mmcv
+    SparseInverseConv3d, neither vendored here) runs the partner layer's rulebook backwards,
+    out[pairs[k,0,p]] += features[pairs[k,1,p]] . W[k]; that is this function on the rulebook
+    with its columns exchanged.  Pinned in tests against dense conv_transpose3d."""
     features = _f32(features)
     w = _f32(filters_kcico)
-    pairs = _i32(indice_pairs)
+    pairs = _swapped(indice_pairs) if inverse else _i32(indice_pairs)
     num = _num64(indice_num)
     K, _, L = pairs.shape
     ci, co = w.shape[1], w.shape[2]
@@ -100,7 +111,12 @@ def forward(features, filters_kcico, indice_pairs, indice_num, num_act_out):
     return out
 
 
-def backward_data(output_grad, filters_kcico, indice_pairs, indice_num):
+def backward_data(output_grad, filters_kcico, indice_pairs, indice_num, inverse=False, rows=None):
+    """inverse=True: dX[pairs[k,1,p]] += dY[pairs[k,0,p]] . W[k]^T over `rows` input rows, which
+    is the forward loop over the unchanged rulebook with dY as features and W[k]^T as filter."""
+    if inverse:
+        wt = np.ascontiguousarray(np.transpose(_f32(filters_kcico), (0, 2, 1)))
+        return forward(output_grad, wt, indice_pairs, indice_num, int(rows))
     dy = _f32(output_grad)
     w = _f32(filters_kcico)
     pairs = _i32(indice_pairs)
@@ -114,10 +130,12 @@ def backward_data(output_grad, filters_kcico, indice_pairs, indice_num):
     return dx
 
 
-def backward_filter(features, output_grad, indice_pairs, indice_num, fast=False):
+def backward_filter(features, output_grad, indice_pairs, indice_num, fast=False, inverse=False):
+    """inverse=True: dW[k] = sum_p features[pairs[k,1,p]]^T . dY[pairs[k,0,p]], the same loop on
+    the rulebook with its columns exchanged."""
     x = _f32(features)
     dy = _f32(output_grad)
-    pairs = _i32(indice_pairs)
+    pairs = _swapped(indice_pairs) if inverse else _i32(indice_pairs)
     num = _num64(indice_num)
     K, _, L = pairs.shape
     ci, co = x.shape[1], dy.shape[1]

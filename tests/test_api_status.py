@@ -514,3 +514,131 @@ def test_library_exports_every_declared_symbol():
     for sym in sorted(declared):
         assert hasattr(lib, sym), sym
     assert declared == set(m.SIGNATURES), declared ^ set(m.SIGNATURES)
+
+
+# --- extended modes (mluOpExtSetSparseConvExtendedModes): inverse = 1, tagged filters_grad ------
+
+def _d(dims, dtype="MLUOP_DTYPE_FLOAT", layout="MLUOP_LAYOUT_ARRAY"):
+    return make_desc({"layout": layout, "dtype": dtype, "dim_nb": len(dims), "dims": list(dims)})
+
+
+def _forward_status(handle, feat, filt, pairs, out, num, n_out, inverse):
+    lib = m.lib()
+    descs = [_d(feat), _d(filt), _d(pairs, "MLUOP_DTYPE_INT32"), _d(out)]
+    try:
+        size = ctypes.c_size_t(64)
+        st = lib.mluOpGetIndiceConvolutionForwardWorkspaceSize(handle.ptr, descs[0], descs[1], descs[2], descs[3],
+                                                               i64(num), n_out, inverse, 0, ctypes.byref(size))
+        if st != 0:
+            return st
+        return lib.mluOpIndiceConvolutionForward(handle.ptr, descs[0], FAKE, descs[1], FAKE, descs[2], FAKE,
+                                                 i64(num), n_out, inverse, 0, FAKE, size.value, descs[3], FAKE)
+    finally:
+        free_descs(*descs)
+
+
+def _backward_data_status(handle, dy, filt, pairs, dx, num, inverse):
+    lib = m.lib()
+    descs = [_d(dy), _d(filt), _d(pairs, "MLUOP_DTYPE_INT32"), _d(dx)]
+    try:
+        size = ctypes.c_size_t(64)
+        st = lib.mluOpGetIndiceConvolutionBackwardDataWorkspaceSize(handle.ptr, descs[0], descs[1], descs[2],
+                                                                    descs[3], i64(num), inverse, ctypes.byref(size))
+        if st != 0:
+            return st
+        return lib.mluOpIndiceConvolutionBackwardData(handle.ptr, descs[0], FAKE, descs[1], FAKE, descs[2], FAKE,
+                                                      i64(num), inverse, 0, FAKE, size.value, descs[3], FAKE)
+    finally:
+        free_descs(*descs)
+
+
+def _backward_filter_status(handle, feat, dy, pairs, dw, num, inverse, dw_layout="MLUOP_LAYOUT_ARRAY"):
+    lib = m.lib()
+    descs = [_d(feat), _d(dy), _d(pairs, "MLUOP_DTYPE_INT32"), _d(dw, layout=dw_layout)]
+    try:
+        size = ctypes.c_size_t(64)
+        st = lib.mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize(handle.ptr, descs[0], descs[1], descs[2],
+                                                                      descs[3], i64(num), inverse, 0,
+                                                                      ctypes.byref(size))
+        if st != 0:
+            return st
+        return lib.mluOpIndiceConvolutionBackwardFilter(handle.ptr, descs[0], FAKE, descs[1], FAKE, descs[2], FAKE,
+                                                        i64(num), inverse, 0, FAKE, size.value, descs[3], FAKE)
+    finally:
+        free_descs(*descs)
+
+
+@pytest.fixture()
+def extended(handle):
+    handle.set_extended_modes(True)
+    yield handle
+    handle.set_extended_modes(False)
+
+
+def test_inverse_keeps_the_reference_status_until_switched_on(handle):
+    K, L, n_in, ci, co = 8, 10, 6, 4, 5     # partner: 10 input rows, 6 output rows, 2x2x2 kernel
+    num = [3] * K
+    fwd = ([n_in, ci], [2, 2, 2, ci, co], [K, 2, L], [L, co], num, L, 1)
+    bwd = ([L, co], [2, 2, 2, ci, co], [K, 2, L], [n_in, ci], num, 1)
+    flt = ([n_in, ci], [L, co], [K, 2, L], [2, 2, 2, ci, co], num, 1)
+    assert _forward_status(handle, *fwd) == STATUS["MLUOP_STATUS_NOT_SUPPORTED"]
+    assert _backward_data_status(handle, *bwd) == STATUS["MLUOP_STATUS_NOT_SUPPORTED"]
+    assert _backward_filter_status(handle, *flt) == STATUS["MLUOP_STATUS_BAD_PARAM"]
+    handle.set_extended_modes(True)
+    try:
+        launched = STATUS["MLUOP_STATUS_EXECUTION_FAILED"]   # every check passed; a host-only handle stops here
+        assert _forward_status(handle, *fwd) == launched
+        assert _backward_data_status(handle, *bwd) == launched
+        assert _backward_filter_status(handle, *flt) == launched
+    finally:
+        handle.set_extended_modes(False)
+    assert _forward_status(handle, *fwd) == STATUS["MLUOP_STATUS_NOT_SUPPORTED"]
+    assert m.lib().mluOpExtSetSparseConvExtendedModes(None, 1) == STATUS["MLUOP_STATUS_BAD_PARAM"]
+
+
+def test_inverse_shape_checks(extended):
+    K, L, n_in, ci, co = 8, 10, 6, 4, 5
+    num = [3] * K
+    bad = STATUS["MLUOP_STATUS_BAD_PARAM"]
+    filt = [2, 2, 2, ci, co]
+    # indice_pairs.dim[2] is the row count of the output side under inverse = 1
+    assert _forward_status(extended, [n_in, ci], filt, [K, 2, L], [L + 1, co], num, L + 1, 1) == bad
+    assert _forward_status(extended, [n_in, ci], filt, [K, 2, L], [L, co], num, L - 1, 1) == bad
+    assert _forward_status(extended, [n_in, ci + 1], filt, [K, 2, L], [L, co], num, L, 1) == bad
+    assert _forward_status(extended, [n_in, ci], filt, [K, 2, L], [L, co], [n_in + 1] * K, L, 1) == bad
+    assert _forward_status(extended, [n_in, ci], filt, [K, 2, L], [L, co], num, L, 2) == bad
+    assert _backward_data_status(extended, [L + 1, co], filt, [K, 2, L], [n_in, ci], num, 1) == bad
+    assert _backward_data_status(extended, [L, co], filt, [K, 2, L], [2, ci], num, 1) == bad   # fewer rows than pairs
+    assert _backward_data_status(extended, [L, co], filt, [K, 2, L], [n_in, ci + 1], num, 1) == bad
+    assert _backward_filter_status(extended, [n_in, ci], [L + 1, co], [K, 2, L], filt, num, 1) == bad
+    assert _backward_filter_status(extended, [n_in, ci], [L, co], [K, 2, L], filt, num, 2) == bad
+    # the regular direction keeps its own rule with the switch on
+    assert _forward_status(extended, [L, ci], filt, [K, 2, L], [n_in, co], num, n_in, 0) == \
+        STATUS["MLUOP_STATUS_EXECUTION_FAILED"]
+    assert _forward_status(extended, [L + 1, ci], filt, [K, 2, L], [n_in, co], num, n_in, 0) == bad
+
+
+def test_tagged_filters_grad_layouts(handle):
+    K, L, n_out, ci, co = 8, 10, 6, 4, 5
+    num = [3] * K
+    ndhwc, ncdhw = [co, 2, 2, 2, ci], [co, ci, 2, 2, 2]
+    args = ([L, ci], [n_out, co], [K, 2, L])
+    # positional reading, as in the reference: the tagged shapes do not fit
+    assert _backward_filter_status(handle, *args, ndhwc, num, 0, "MLUOP_LAYOUT_NDHWC") == STATUS["MLUOP_STATUS_BAD_PARAM"]
+    assert _backward_filter_status(handle, *args, ncdhw, num, 0, "MLUOP_LAYOUT_NCDHW") == STATUS["MLUOP_STATUS_BAD_PARAM"]
+    assert _backward_filter_status(handle, *args, [2, 2, 2, ci, co], num, 0, "MLUOP_LAYOUT_NDHWC") == \
+        STATUS["MLUOP_STATUS_EXECUTION_FAILED"]
+    handle.set_extended_modes(True)
+    try:
+        launched = STATUS["MLUOP_STATUS_EXECUTION_FAILED"]
+        assert _backward_filter_status(handle, *args, ndhwc, num, 0, "MLUOP_LAYOUT_NDHWC") == launched
+        assert _backward_filter_status(handle, *args, ncdhw, num, 0, "MLUOP_LAYOUT_NCDHW") == launched
+        assert _backward_filter_status(handle, *args, [co, 2, 2, ci], [3] * 4, 0, "MLUOP_LAYOUT_NHWC") == \
+            STATUS["MLUOP_STATUS_BAD_PARAM"]          # K = 4 against 8 offsets in indice_pairs
+        assert _backward_filter_status(handle, ([L, ci]), [n_out, co], [4, 2, L], [co, 2, 2, ci], [3] * 4, 0,
+                                       "MLUOP_LAYOUT_NHWC") == launched
+        assert _backward_filter_status(handle, *args, [2, 2, 2, ci, co], num, 0, "MLUOP_LAYOUT_NDHWC") == \
+            STATUS["MLUOP_STATUS_BAD_PARAM"]          # now read as [Co, kd, kh, kw, Ci]
+        assert _backward_filter_status(handle, *args, [2, 2, 2, ci, co], num, 0, "MLUOP_LAYOUT_ARRAY") == launched
+    finally:
+        handle.set_extended_modes(False)

@@ -168,3 +168,46 @@ def test_small_channel_counts_are_padded_for_the_matrix_cores(gpu_handle):
                             (layer.weight.grad.cpu().numpy().reshape(27, 5, 12), dw, "grad w")):
         d1 = np.abs(got - want).sum() / np.abs(want).sum()
         assert d1 <= 1e-5, (what, d1)
+
+
+def test_inverse_layer_returns_to_the_partner_layers_cells(gpu_handle):
+    """SparseConv3d (stride 2) followed by the SparseInverseConv3d that shares its rulebook, against
+    dense conv3d -> conv_transpose3d in float64 read at the first layer's input cells, with the
+    gradients of features and both filters."""
+    import torch
+    import torch.nn.functional as F
+    from mluop_hip import nn as spnn
+    rng = np.random.default_rng(23)
+    batch, space, L, ci, cm, co = 2, (8, 10, 12), 300, 16, 32, 16
+    idx = random_voxels(rng, batch, space, L)
+    feats = rng.standard_normal((L, ci)).astype(np.float32)
+    torch.manual_seed(5)
+    down = spnn.SparseConv3d(ci, cm, 3, stride=2, padding=1, indice_key="down").cuda()
+    up = spnn.SparseInverseConv3d(cm, co, 3, indice_key="down").cuda()
+    x = torch.from_numpy(feats).cuda().requires_grad_(True)
+    st = spnn.SparseTensor(x, torch.from_numpy(idx).cuda(), space, batch)
+    mid = down(st)
+    y = up(mid)
+    assert y.spatial_shape == tuple(space) and torch.equal(y.indices, st.indices)
+    assert tuple(y.features.shape) == (L, co)
+    g = rng.standard_normal((L, co)).astype(np.float32)
+    (y.features * torch.from_numpy(g).cuda()).sum().backward()
+    torch.cuda.synchronize()
+
+    D, H, W = space
+    rx = torch.tensor(feats, dtype=torch.float64, requires_grad=True)
+    w1 = torch.tensor(down.weight.detach().cpu().numpy(), dtype=torch.float64, requires_grad=True)
+    w2 = torch.tensor(up.weight.detach().cpu().numpy(), dtype=torch.float64, requires_grad=True)
+    ii = torch.from_numpy(idx.astype(np.int64))
+    dense = torch.zeros((batch, D, H, W, ci), dtype=torch.float64).index_put(
+        (ii[:, 0], ii[:, 1], ii[:, 2], ii[:, 3]), rx).permute(0, 4, 1, 2, 3)
+    t = F.conv3d(dense, w1.permute(4, 3, 0, 1, 2), stride=2, padding=1)
+    opad = [s - ((o - 1) * 2 - 2 + 2 + 1) for s, o in zip(space, t.shape[2:])]
+    t = F.conv_transpose3d(t, w2.permute(3, 4, 0, 1, 2), stride=2, padding=1, output_padding=opad)
+    assert tuple(t.shape[2:]) == tuple(space)
+    rows = t[ii[:, 0], :, ii[:, 1], ii[:, 2], ii[:, 3]]
+    (rows * torch.from_numpy(g.astype(np.float64))).sum().backward()
+    np.testing.assert_allclose(y.features.detach().cpu().numpy(), rows.detach().numpy(), rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(x.grad.cpu().numpy(), rx.grad.numpy(), rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(down.weight.grad.cpu().numpy(), w1.grad.numpy(), rtol=1e-4, atol=2e-4)
+    np.testing.assert_allclose(up.weight.grad.cpu().numpy(), w2.grad.numpy(), rtol=1e-4, atol=2e-4)

@@ -82,6 +82,60 @@ def test_oracle_ops_match_dense_conv3d_and_autograd(case):
     assert abs(a - b) / scale < 1e-4 and abs(a - c) / scale < 1e-4
 
 
+INVERSE_CASES = [
+    # (batch, space, L, ks, pad, stride, dil, ci of the inverse layer, co of the inverse layer)
+    (2, (7, 8, 9), 150, (3, 3, 3), (1, 1, 1), (2, 2, 2), (1, 1, 1), 5, 4),
+    (1, (8, 8, 8), 100, (3, 3, 3), (2, 2, 2), (1, 1, 1), (2, 2, 2), 2, 3),
+    (1, (6, 7, 8), 90, (2, 2, 2), (0, 0, 0), (2, 2, 2), (1, 1, 1), 6, 2),
+    (1, (5, 9, 6), 80, (1, 3, 2), (0, 1, 0), (1, 2, 1), (1, 1, 1), 3, 3),
+]
+
+
+@pytest.mark.parametrize("case", INVERSE_CASES)
+def test_inverse_ops_match_dense_conv_transpose3d_and_autograd(case):
+    """The inverse convolution runs its partner's rulebook backwards: dense conv_transpose3d of the
+    partner's output grid, read back at the partner's input cells, is the same numbers, and its
+    autograd gives the two gradients."""
+    batch, space, L, ks, pad, stride, dil, ci, co = case
+    rng = np.random.default_rng(7)
+    idx = random_voxels(rng, batch, space, L)
+    ospace = out_space(space, ks, pad, stride, dil)
+    pairs, out_idx, num, n_out = oracle.get_indice_pairs(idx, batch, list(pad), list(stride), list(dil), list(ks),
+                                                         ospace, False, exact_count=True)
+    K = int(np.prod(ks))
+    feats = rng.standard_normal((n_out, ci)).astype(np.float32)   # live on the partner's output cells
+    w = rng.standard_normal(tuple(ks) + (ci, co)).astype(np.float32)
+    dy = rng.standard_normal((L, co)).astype(np.float32)          # gradient at the partner's input cells
+    wk = w.reshape(K, ci, co)
+
+    x = torch.zeros((batch, ci) + tuple(ospace), dtype=torch.float64)
+    oo = torch.from_numpy(out_idx[:n_out].astype(np.int64))
+    ii = torch.from_numpy(idx.astype(np.int64))
+    x[oo[:, 0], :, oo[:, 1], oo[:, 2], oo[:, 3]] = torch.from_numpy(feats.astype(np.float64))
+    x.requires_grad_(True)
+    wt = torch.from_numpy(w.astype(np.float64)).permute(3, 4, 0, 1, 2).contiguous().requires_grad_(True)
+    opad = [sp - ((o - 1) * s - 2 * p + d * (k - 1) + 1) for sp, o, s, p, d, k in zip(space, ospace, stride, pad, dil, ks)]
+    y = F.conv_transpose3d(x, wt, stride=tuple(stride), padding=tuple(pad), output_padding=tuple(opad),
+                           dilation=tuple(dil))
+    assert list(y.shape[2:]) == list(space)
+    ref_out = y[ii[:, 0], :, ii[:, 1], ii[:, 2], ii[:, 3]].detach().numpy()
+    g = torch.zeros_like(y)
+    g[ii[:, 0], :, ii[:, 1], ii[:, 2], ii[:, 3]] = torch.from_numpy(dy.astype(np.float64))
+    y.backward(g)
+    ref_dx = x.grad[oo[:, 0], :, oo[:, 1], oo[:, 2], oo[:, 3]].numpy()
+    ref_dw = wt.grad.permute(2, 3, 4, 0, 1).contiguous().numpy()
+
+    out = oracle.forward(feats, wk, pairs, num, L, inverse=True)
+    dx = oracle.backward_data(dy, wk, pairs, num, inverse=True, rows=n_out)
+    dw = oracle.backward_filter(feats, dy, pairs, num, inverse=True)
+    np.testing.assert_allclose(out, ref_out, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(dx, ref_dx, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(dw.reshape(w.shape), ref_dw, rtol=2e-5, atol=2e-4)
+    # the inverse forward is the partner's backward data with the filter's channel roles exchanged
+    same = oracle.backward_data(feats, np.ascontiguousarray(np.transpose(wk, (0, 2, 1))), pairs, num)
+    np.testing.assert_allclose(out, same, rtol=2e-5, atol=2e-5)  # fp32 sums in different orders
+
+
 def test_forward_skips_negative_pairs_and_respects_indice_num():
     rng = np.random.default_rng(2)
     L, K, ci, co = 6, 2, 3, 2
