@@ -642,3 +642,11 @@ def test_tagged_filters_grad_layouts(handle):
         assert _backward_filter_status(handle, *args, [2, 2, 2, ci, co], num, 0, "MLUOP_LAYOUT_ARRAY") == launched
     finally:
         handle.set_extended_modes(False)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    """No fallback path: without the built library the binding raises instead of computing elsewhere."""
+    monkeypatch.setattr(m, "_lib", None)
+    monkeypatch.setattr(m, "LIB_PATH", os.path.join(ROOT, "mlu-ops_amd", "lib", "no_such_library.so"))
+    with pytest.raises(RuntimeError, match="there is no fallback path"):
+        m.lib()
