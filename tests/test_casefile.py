@@ -181,3 +181,50 @@ def test_replay_refuses_other_operators(gpu_handle):
         text = f.read()
     with pytest.raises(ValueError):
         cf.replay(text, gpu_handle)
+
+
+REFERENCE_BWD_DATA_CASE = os.path.join(GOLDEN, "indice_convolution_backward_data", "case_0.prototxt")
+
+
+def reference_backward_data_case():
+    """The one sparse-convolution case the reference keeps in its tree
+    (zoo/indice_convolution_backward_data/test_case/case_0.prototxt, a verbatim data file): explicit
+    pairs, seeded random out_grad and filter (filled by this module's own generator: the reference
+    generator's bit stream is not reproduced), no stored baseline."""
+    cf = casefile()
+    node, base = cf.load(REFERENCE_BWD_DATA_CASE)
+    ins = [cf.CaseTensor(t, base) for t in node.all("input")]
+    out = cf.CaseTensor(node.all("output")[0], base)
+    return node, ins, out
+
+
+def test_reference_backward_data_case_reads():
+    cf = casefile()
+    node, (dy, w, pairs), out = reference_backward_data_case()
+    assert node.get("op_name") == "indice_convolution_backward_data"
+    assert dy.values.shape == (10, 100) and w.values.shape == (3, 3, 210, 100) and w.layout == 2  # HWCN
+    assert pairs.values.shape == (9, 2, 10) and pairs.values.dtype == np.int32
+    assert all(pairs.values[k, c].tolist() == list(range(10)) for k in range(9) for c in range(2))
+    assert list(out.shape) == [10, 210] and out.values is None
+    p = node.get("indice_convolution_backward_data_param")
+    assert p.all("indice_num") == [10] * 9 and p.get("inverse") == 0 and p.get("sub_m") == 0
+    assert cf.criteria(node) == (["DIFF1", "DIFF2"], [1e-5, 1e-5])
+    assert np.abs(dy.values).max() <= 1.0 and np.abs(w.values).max() <= 1.0   # U(-1, 1) as the file asks
+    # identity pairs at every offset: the operator reduces to one dense product with the summed filter
+    ref = oracle.backward_data(dy.values, w.values.reshape(9, 210, 100), pairs.values, [10] * 9)
+    dense = dy.values.astype(np.float64) @ w.values.astype(np.float64).sum(axis=(0, 1)).T
+    np.testing.assert_allclose(ref, dense, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.gpu
+def test_reference_backward_data_case_replays(gpu_handle):
+    """Replayed through the C API from the file itself and graded at the file's own thresholds
+    against the oracle on the same generated inputs."""
+    cf = casefile()
+    node, (dy, w, pairs), out = reference_backward_data_case()
+    res = cf.replay(REFERENCE_BWD_DATA_CASE, gpu_handle)
+    got = res.outputs["in_grad"]
+    assert got.shape == (10, 210)
+    ref = oracle.backward_data(dy.values, w.values.reshape(9, 210, 100), pairs.values, [10] * 9)
+    funcs, thresholds = cf.criteria(node)
+    assert cf.diff1(got, ref) <= thresholds[0] and cf.diff2(got, ref) <= thresholds[1]
