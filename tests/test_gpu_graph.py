@@ -57,3 +57,48 @@ def test_captured_step_replays_bit_exactly():
                 assert torch.equal(got, want)
     torch.cuda.current_stream().wait_stream(side)
     handle.close()
+
+
+def test_two_handles_on_two_streams_do_not_interfere():
+    """Each handle owns its queue and its pinned read-back slot: two different problems enqueued
+    alternately on two streams (default priority) give the results each gives alone."""
+    import torch
+    import mluop_hip as m
+    rng = np.random.default_rng(32)
+    ks = (3, 3, 3)
+
+    def problem(batch, space, L, ci, co, sub_m):
+        idx = torch.from_numpy(random_voxels(rng, batch, space, L)).cuda()
+        feats = torch.from_numpy(rng.standard_normal((L, ci)).astype(np.float32)).cuda().half()
+        w = torch.from_numpy((rng.standard_normal(ks + (ci, co)) * 0.1).astype(np.float32)).cuda().half()
+        ospace = list(space) if sub_m else m.regular_output_space(space, ks, [1, 1, 1], [2, 2, 2], [1, 1, 1])
+        stride = [1, 1, 1] if sub_m else [2, 2, 2]
+        return dict(idx=idx, feats=feats, w=w, batch=batch, space=space, ospace=ospace, stride=stride, sub_m=sub_m)
+
+    def run(handle, p):
+        pairs, out_idx, num, n_out = m.get_indice_pairs(handle, p["idx"], p["batch"], p["space"], ks, p["ospace"],
+                                                        [1, 1, 1], p["stride"], [1, 1, 1], p["sub_m"])
+        num_host = num.cpu().tolist()        # waits for this handle's queue only
+        out = m.indice_conv_forward(handle, p["feats"], p["w"], m.LAYOUT_ARRAY, pairs, num_host, n_out, p["sub_m"])
+        return pairs, num, out_idx[:n_out].clone(), out
+
+    problems = [problem(2, (12, 24, 24), 6000, 64, 64, True), problem(1, (16, 20, 28), 4000, 32, 64, False)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    handles, alone = [], []
+    for s, p in zip(streams, problems):
+        with torch.cuda.stream(s):
+            handles.append(m.make_handle_on_current_stream())
+            alone.append(run(handles[-1], p))
+            s.synchronize()
+    for rep in range(3):
+        together = []
+        for s, h, p in zip(streams, handles, problems):
+            with torch.cuda.stream(s):
+                together.append(run(h, p))
+        torch.cuda.synchronize()
+        for got, want in zip(together, alone):
+            for g, w_ in zip(got, want):
+                assert torch.equal(g, w_), "repetition %d" % rep
+    for h in handles:
+        h.close()
