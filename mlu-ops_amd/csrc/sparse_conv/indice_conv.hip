@@ -118,6 +118,13 @@ __global__ __launch_bounds__(256) void fillInt32(int32_t *dst, size_t n, int32_t
 // map[k][row] = partner row, for the first indice_num[k] pairs of every offset.
 // row_col / src_col select which pair column owns the result row (1 for
 // forward, 0 for backward data).  Indices outside their tensor are ignored.
+// A map slot holds one partner.  Rulebooks built from distinct coordinates name a
+// result row once per offset at most; when coordinates repeat (or the pairs are
+// made up, as in test case files) several pairs of one offset can name the same
+// row, and the reference adds them all.  Plain stores keep whichever of them was
+// written last; every workgroup of a gather kernel records how many slots of its
+// tile it found filled, and repairLostPairs adds what the other pairs would have
+// contributed when those counts fall short of the number of pairs.
 __global__ __launch_bounds__(256) void scatterRowMap(const int32_t *pairs, int L,
                                                      OffsetCounts inl, const int32_t *dev_counts,
                                                      int row_col, int src_col, int n_rows,
@@ -142,8 +149,10 @@ __global__ __launch_bounds__(256) void gatherConvSimt(const typename E::storage 
                                                       int64_t sQ, int64_t sC, const int32_t *map,
                                                       int R, int K, OffsetCounts inl,
                                                       const int32_t *dev_counts, int C,
+                                                      int32_t *filled,
                                                       typename E::storage *result) {
   constexpr int TR = 32, TC = 64, QC = 32;
+  int slots = 0;  // filled map slots of this tile (first wave, uniform)
   __shared__ float As[TR][QC + 1];
   __shared__ float Bs[QC][TC];
   __shared__ int s_src[TR];
@@ -156,6 +165,7 @@ __global__ __launch_bounds__(256) void gatherConvSimt(const typename E::storage 
     int v = -1;
     if (tid < TR && r0 + tid < R) v = map[(size_t)k * R + r0 + tid];
     if (tid < TR) s_src[tid] = v;
+    if (tid < 64) slots += __popcll(__ballot(v >= 0));
     if (!__syncthreads_or(v >= 0)) continue;
     for (int q0 = 0; q0 < Q; q0 += QC) {
 #pragma unroll
@@ -197,6 +207,7 @@ __global__ __launch_bounds__(256) void gatherConvSimt(const typename E::storage 
       if (c < C) E::store(result + (size_t)r * C + c, acc[i][j]);
     }
   }
+  if (tid == 0 && blockIdx.y == 0) filled[blockIdx.x] = slots;
 }
 
 // ---- MFMA gather convolution ---------------------------------------------------
@@ -305,7 +316,8 @@ template <typename E, int Q, int C>
 __global__ __launch_bounds__(mfmaThreads(C)) __attribute__((amdgpu_waves_per_eu(mfmaWavesPerSimd((int)sizeof(typename E::storage), Q, C),
                                    mfmaWavesPerSimd((int)sizeof(typename E::storage), Q, C))))
 void gatherConvMfma(const typename E::storage *A, const typename E::storage *packedW,
-                    const int32_t *map, int R, int K, int ldc, typename E::storage *result) {
+                    const int32_t *map, int R, int K, int ldc, int32_t *filled,
+                    typename E::storage *result) {
   typedef typename E::vec8 vec8;
   typedef typename E::storage S;
   constexpr int NB = mfmaColBlocksPerWave(C);
@@ -349,7 +361,11 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   const int tiles_per_xcd = gridDim.x >> 3;
   const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
   const int r0 = tile * TR;
-  if (r0 >= R) return;
+  if (r0 >= R) {
+    if (tid == 0 && blockIdx.y == 0) filled[blockIdx.x] = 0;
+    return;
+  }
+  int slots = 0;  // filled map slots of this tile
   const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
   for (int i = tid; i < (TR + 1) * ACC_STRIDE; i += NT) s_acc[i] = 0.f;
@@ -408,6 +424,7 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
     const int blk_incl = waveInclusiveScan(nb_mine);
     const int total = __builtin_amdgcn_readlane(ent_incl, 63);
     const int nblk = __builtin_amdgcn_readlane(blk_incl, 63);
+    slots += total;
     const int nbatch = (nblk + G - 1) / G;
     const int ent_first = ent_incl - cnt;
 #pragma unroll
@@ -570,6 +587,7 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
     *reinterpret_cast<uint4 *>(result + (size_t)(r0 + rr) * ldc + col_group * C + c0) =
         *reinterpret_cast<const uint4 *>(tmp);
   }
+  if (tid == 0 && blockIdx.y == 0) filled[blockIdx.x] = slots;
 }
 
 // ---- MFMA gather convolution for dense rulebooks -------------------------------
@@ -599,7 +617,7 @@ constexpr int denseThreads(int C) { return 64 * (C / 32) * kDenseRowSplit; }
 template <typename E, int Q, int C>
 __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
     const typename E::storage *A, const typename E::storage *packedW, const int32_t *map, int R,
-    int K, int ldc, typename E::storage *result) {
+    int K, int ldc, int32_t *filled, typename E::storage *result) {
   typedef typename E::vec8 vec8;
   typedef typename E::storage S;
   constexpr int NB = 2;                      // 16-column blocks per wave
@@ -633,7 +651,10 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
   const int tiles_per_xcd = gridDim.x >> 3;  // neighbouring tiles on one XCD, as above
   const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
   const int r0 = tile * TR;
-  if (r0 >= R) return;
+  if (r0 >= R) {
+    if (tid == 0 && blockIdx.y == 0) filled[blockIdx.x] = 0;
+    return;
+  }
   const int col_group = blockIdx.y;
   const int pair = lane & 15;
   const int quad = lane >> 4;
@@ -649,6 +670,7 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
   for (int g = 0; g < GPW; ++g)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[g][nb] = float4v{0.f, 0.f, 0.f, 0.f};
+  int slots = 0;  // filled map slots this wave staged
 
   for (int kc = 0; kc < K; kc += KC) {
     const int kn = (K - kc) < KC ? (K - kc) : KC;
@@ -659,6 +681,7 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
       s_map[kk][lane] = v;
       const unsigned long long any = __ballot(v >= 0);
       if (lane == 0) s_has[kk] = any != 0ull;
+      slots += __popcll(any);
     }
     __syncthreads();
     if (wave == 0) {
@@ -765,6 +788,155 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
         *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(tmp);
     }
   }
+  // s_has is free again: the waves' slot counts meet there
+  __syncthreads();
+  if (lane == 0) s_has[wave] = slots;
+  __syncthreads();
+  if (tid == 0 && blockIdx.y == 0) {
+    int all = 0;
+    for (int w = 0; w < WAVES; ++w) all += s_has[w];
+    filled[blockIdx.x] = all;
+  }
+}
+
+// ---- pairs that lost their map slot -----------------------------------------------
+// Runs behind every gather kernel as one workgroup and returns at once when the
+// kernels found as many filled map slots as there are pairs (always, for a rulebook
+// built from distinct coordinates).  Otherwise some pairs of one offset share a
+// result row, or lie outside their tensors: every pair is looked up again, the
+// first one that finds its partner in the slot claims it (the kernels have
+// multiplied that one), and each of the others is added to its result row here.
+// A touched row is rebuilt in an fp32 pool (kRepairPoolRows rows, indexed through
+// `shadow`): first the partners its map slots hold, as the kernel summed them, then
+// the lost pairs as the scan meets them, and it is rounded into the result once,
+// when the scan ends: the same single rounding as any other row.  (A row that has
+// to leave a full pool early and is touched again continues from its rounded value.)
+// Which of the colliding pairs owned the slot depends on the order their stores
+// landed in, so the last bits of such rows can differ from run to run; rows without
+// collisions are not touched.
+constexpr int kRepairPoolRows = 2048;
+
+struct RepairScratch {
+  int32_t *shadow;    // [R] pool row of a result row; -1 never pooled, -2 rounded back already
+  int32_t *pool_row;  // [kRepairPoolRows] result row of a pool row
+  float *pool;        // [kRepairPoolRows, C]
+};
+
+template <typename E>
+__global__ __launch_bounds__(256) void repairLostPairs(
+    const typename E::storage *A, int Q, const typename E::storage *W, int64_t sK, int64_t sQ,
+    int64_t sC, const int32_t *pairs, int L, int row_col, int src_col, int R, int n_src, int K,
+    OffsetCounts inl, const int32_t *dev_counts, int32_t *map, const int32_t *filled,
+    int n_filled, int expected, int C, RepairScratch scratch, typename E::storage *result) {
+  __shared__ int s_found;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  if (tid == 0) s_found = 0;
+  __syncthreads();
+  int mine = 0;
+  for (int i = tid; i < n_filled; i += 256) mine += filled[i];
+  mine = waveInclusiveScan(mine);
+  if (lane == 63) atomicAdd(&s_found, mine);
+  __syncthreads();
+  if (s_found == expected) return;
+
+  __shared__ int s_row[256];
+  __shared__ int s_src[256];
+  __shared__ int s_wave_lost[4];
+  __shared__ int s_pooled;  // pool rows in use
+  for (int i = tid; i < R; i += 256) scratch.shadow[i] = -1;
+  if (tid == 0) s_pooled = 0;
+  __syncthreads();
+  // rounds the pool back into the result and empties it
+  auto flush = [&]() {
+    const int n = s_pooled;
+    for (int i = 0; i < n; ++i) {
+      const int r = scratch.pool_row[i];
+      for (int c = tid; c < C; c += 256)
+        E::store(result + (size_t)r * C + c, scratch.pool[(size_t)i * C + c]);
+      if (tid == 0) scratch.shadow[r] = -2;
+    }
+    __syncthreads();
+    if (tid == 0) s_pooled = 0;
+    __syncthreads();
+  };
+  for (int k = 0; k < K; ++k) {
+    const int n = offsetCount(inl, dev_counts, k);
+    const int32_t *base = pairs + (size_t)k * 2 * L;
+    for (int p0 = 0; p0 < n; p0 += 256) {
+      const int p = p0 + tid;
+      int r = -1, src = -1;
+      bool lost = false;
+      if (p < n) {
+        r = base[(size_t)row_col * L + p];
+        src = base[(size_t)src_col * L + p];
+        if ((unsigned)r < (unsigned)R && (unsigned)src < (unsigned)n_src) {
+          int32_t *slot = map + (size_t)k * R + r;
+          // the claimed slot holds -2 - partner: no pair finds itself there twice
+          lost = !(*slot == src && atomicCAS(slot, src, -2 - src) == src);
+        }
+      }
+      // lost pairs of this step in pair order
+      const unsigned long long b = __ballot(lost);
+      if (lane == 0) s_wave_lost[wave] = __popcll(b);
+      __syncthreads();
+      int before = 0, total = 0;
+      for (int w = 0; w < 4; ++w) {
+        if (w < wave) before += s_wave_lost[w];
+        total += s_wave_lost[w];
+      }
+      if (lost) {
+        const int at = before + __popcll(b & ((1ull << lane) - 1ull));
+        s_row[at] = r;
+        s_src[at] = src;
+      }
+      __syncthreads();
+      for (int i = 0; i < total; ++i) {
+        const int row = s_row[i];
+        int at = scratch.shadow[row];
+        if (at < 0) {
+          const bool first_time = at == -1;
+          if (s_pooled == kRepairPoolRows) flush();
+          at = s_pooled;
+          __syncthreads();  // everybody has read the pool's fill state
+          if (tid == 0) {
+            scratch.shadow[row] = at;
+            scratch.pool_row[at] = row;
+            s_pooled = at + 1;
+          }
+          for (int c = tid; c < C; c += 256) {
+            float sum = 0.f;
+            if (first_time) {
+              // what the gather kernel summed: the partner every slot of the row holds
+              // (claimed slots hold -2 - partner)
+              for (int kk = 0; kk < K; ++kk) {
+                const int m = map[(size_t)kk * R + row];
+                if (m == -1) continue;
+                const typename E::storage *a = A + (size_t)(m >= 0 ? m : -2 - m) * Q;
+                const typename E::storage *w = W + (size_t)kk * sK + (size_t)c * sC;
+                float dot = 0.f;
+                for (int q = 0; q < Q; ++q) dot += E::load(a + q) * E::load(w + (size_t)q * sQ);
+                sum += dot;
+              }
+            } else {
+              sum = E::load(result + (size_t)row * C + c);
+            }
+            scratch.pool[(size_t)at * C + c] = sum;
+          }
+        }
+        const typename E::storage *a = A + (size_t)s_src[i] * Q;
+        for (int c = tid; c < C; c += 256) {
+          const typename E::storage *w = W + (size_t)k * sK + (size_t)c * sC;
+          float dot = 0.f;
+          for (int q = 0; q < Q; ++q) dot += E::load(a + q) * E::load(w + (size_t)q * sQ);
+          scratch.pool[(size_t)at * C + c] += dot;
+        }
+        __syncthreads();  // shadow and the pool row are in place for the next pair
+      }
+    }
+  }
+  flush();
 }
 
 // ---- backward filter -------------------------------------------------------------
@@ -1170,6 +1342,10 @@ GatherDims gatherDims(const ConvProblem &p, GatherDirection dir) {
 
 struct GatherWorkspace {
   int32_t *dev_counts = nullptr;
+  int32_t *filled = nullptr;  // map slots the gather kernel's workgroups found filled
+  int32_t *shadow = nullptr;  // repairLostPairs' scratch, touched only when pairs collide
+  int32_t *pool_row = nullptr;
+  float *pool = nullptr;
   int32_t *map = nullptr;
   void *packed = nullptr;
   size_t bytes = 0;
@@ -1185,6 +1361,10 @@ GatherWorkspace carveGather(const ConvProblem &p, const GatherDims &d, void *bas
     return r;
   };
   if (p.K > kMaxInlineK) ws.dev_counts = reinterpret_cast<int32_t *>(take((size_t)p.K * 4));
+  ws.filled = reinterpret_cast<int32_t *>(take(((size_t)d.R / 32 + 16) * 4));
+  ws.shadow = reinterpret_cast<int32_t *>(take((size_t)d.R * 4));
+  ws.pool_row = reinterpret_cast<int32_t *>(take((size_t)kRepairPoolRows * 4));
+  ws.pool = reinterpret_cast<float *>(take((size_t)kRepairPoolRows * d.C * 4));
   ws.map = reinterpret_cast<int32_t *>(take((size_t)p.K * d.R * 4));
   if (mfmaShapeOk(p.dtype, d.Q, d.C)) {
     // reduction channels are padded to whole 16-byte fragments (32 for the 2-byte types)
@@ -1239,16 +1419,31 @@ int mfmaTileCols(const ConvProblem &p, const GatherDims &d) {
   return per_tile_offset < 8.0 ? 64 : 128;
 }
 
+// The row map and, per workgroup of a gather kernel (blockIdx.x), the number of slots it
+// found filled in its tile.
+struct RowMap {
+  const int32_t *entries;
+  int32_t *filled;
+};
+
+// Workgroups along x: tiles rounded up to a multiple of the XCD count.
+int mfmaGridX(int R, int tile_cols) {
+  const int tr = mfmaTileRows(tile_cols);
+  return ((R + tr - 1) / tr + 7) / 8 * 8;
+}
+int denseGridX(int R) { return ((R + kDenseTileRows - 1) / kDenseTileRows + 7) / 8 * 8; }
+
 template <typename E, int Q, int C>
 void launchMfmaInstance(const LaunchCtx &lc, const void *A, const void *packed,
-                        const int32_t *map, int R, int K, int ldc, void *result) {
+                        RowMap map, int R, int K, int ldc, void *result) {
   constexpr int NT = mfmaThreads(C);
   constexpr int TR = mfmaTileRows(C);
-  const dim3 grid(((R + TR - 1) / TR + 7) / 8 * 8, ldc / C);  // a multiple of the XCD count
+  static_assert(TR == mfmaTileRows(C), "grid helper and kernel agree");
+  const dim3 grid(mfmaGridX(R, C), ldc / C);
   lc.begin("gatherConvMfma");
   gatherConvMfma<E, Q, C><<<grid, NT, 0, lc.stream>>>(
       static_cast<const typename E::storage *>(A),
-      static_cast<const typename E::storage *>(packed), map, R, K, ldc,
+      static_cast<const typename E::storage *>(packed), map.entries, R, K, ldc, map.filled,
       static_cast<typename E::storage *>(result));
   lc.end();
 }
@@ -1257,7 +1452,7 @@ void launchMfmaInstance(const LaunchCtx &lc, const void *A, const void *packed,
 // rows, so sparse rulebooks fill their 16-pair blocks better.
 template <typename E, int Q>
 void launchMfmaByC(const LaunchCtx &lc, int C, int tile_cols, const void *A, const void *packed,
-                   const int32_t *map, int R, int K, void *result) {
+                   RowMap map, int R, int K, void *result) {
   switch (tile_cols) {
     case 16: launchMfmaInstance<E, Q, 16>(lc, A, packed, map, R, K, C, result); break;
     case 32: launchMfmaInstance<E, Q, 32>(lc, A, packed, map, R, K, C, result); break;
@@ -1269,7 +1464,7 @@ void launchMfmaByC(const LaunchCtx &lc, int C, int tile_cols, const void *A, con
 
 template <typename E>
 void launchMfma(const LaunchCtx &lc, int Q, int C, int tile_cols, const void *A, const void *packed,
-                const int32_t *map, int R, int K, void *result) {
+                RowMap map, int R, int K, void *result) {
   switch (Q) {
     case 16: launchMfmaByC<E, 16>(lc, C, tile_cols, A, packed, map, R, K, result); break;
     case 32: launchMfmaByC<E, 32>(lc, C, tile_cols, A, packed, map, R, K, result); break;
@@ -1302,19 +1497,19 @@ bool useDenseKernel(const ConvProblem &p, const GatherDims &d) {
 }
 
 template <typename E, int Q, int C>
-void launchDenseInstance(const LaunchCtx &lc, const void *A, const void *packed, const int32_t *map,
+void launchDenseInstance(const LaunchCtx &lc, const void *A, const void *packed, RowMap map,
                          int R, int K, void *result) {
-  const dim3 grid(((R + kDenseTileRows - 1) / kDenseTileRows + 7) / 8 * 8, 1);
+  const dim3 grid(denseGridX(R), 1);
   lc.begin("gatherConvDense");
   gatherConvDense<E, Q, C><<<grid, denseThreads(C), 0, lc.stream>>>(
       static_cast<const typename E::storage *>(A), static_cast<const typename E::storage *>(packed),
-      map, R, K, C, static_cast<typename E::storage *>(result));
+      map.entries, R, K, C, map.filled, static_cast<typename E::storage *>(result));
   lc.end();
 }
 
 template <typename E>
 void launchDense(const LaunchCtx &lc, int Q, int C, const void *A, const void *packed,
-                 const int32_t *map, int R, int K, void *result) {
+                 RowMap map, int R, int K, void *result) {
   constexpr bool is_float = std::is_same<E, FloatElem>::value;
 #define DENSE_CASE(q)                                                                      \
   case q:                                                                                  \
@@ -1360,6 +1555,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
   const int64_t sQ = d.filter_forward ? f.stride_ci : f.stride_co;
   const int64_t sC = d.filter_forward ? f.stride_co : f.stride_ci;
   const size_t map_elems = (size_t)p.K * d.R;
+  int n_filled = 0;  // workgroups along x of the gather kernel = slot counts it leaves
   if (use_mfma) {
     const size_t frags = (size_t)p.K * (d.C / 16) * ((d.Q + E::kChunk - 1) / E::kChunk) * 64;
     const int fill_blocks = gridFor(map_elems / 4 + 1, 2048);
@@ -1370,22 +1566,41 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
         d.Q, d.C, static_cast<S *>(ws.packed));
     lc.end();
     launchScatterRowMap(lc, p, d, ws, inl, max_count);
-    if (useDenseKernel(p, d))
-      launchDense<E>(lc, d.Q, d.C, gathered, ws.packed, ws.map, d.R, p.K, result);
-    else
-      launchMfma<E>(lc, d.Q, d.C, mfmaTileCols(p, d), gathered, ws.packed, ws.map, d.R, p.K, result);
-    return;
+    const RowMap map = {ws.map, ws.filled};
+    if (useDenseKernel(p, d)) {
+      n_filled = denseGridX(d.R);
+      launchDense<E>(lc, d.Q, d.C, gathered, ws.packed, map, d.R, p.K, result);
+    } else {
+      const int tile_cols = mfmaTileCols(p, d);
+      n_filled = mfmaGridX(d.R, tile_cols);
+      launchMfma<E>(lc, d.Q, d.C, tile_cols, gathered, ws.packed, map, d.R, p.K, result);
+    }
+  } else {
+    lc.begin("fillInt32");
+    fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems, -1);
+    lc.end();
+    launchScatterRowMap(lc, p, d, ws, inl, max_count);
+    dim3 grid((d.R + 31) / 32, (d.C + 63) / 64);
+    n_filled = (int)grid.x;
+    lc.begin("gatherConvSimt");
+    gatherConvSimt<E><<<grid, 256, 0, lc.stream>>>(static_cast<const S *>(gathered), d.Q,
+                                                static_cast<const S *>(f.base), f.stride_k, sQ, sC,
+                                                ws.map, d.R, p.K, inl, ws.dev_counts, d.C,
+                                                ws.filled, static_cast<S *>(result));
+    lc.end();
   }
-  lc.begin("fillInt32");
-  fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems, -1);
-  lc.end();
-  launchScatterRowMap(lc, p, d, ws, inl, max_count);
-  dim3 grid((d.R + 31) / 32, (d.C + 63) / 64);
-  lc.begin("gatherConvSimt");
-  gatherConvSimt<E><<<grid, 256, 0, lc.stream>>>(static_cast<const S *>(gathered), d.Q,
-                                              static_cast<const S *>(f.base), f.stride_k, sQ, sC,
-                                              ws.map, d.R, p.K, inl, ws.dev_counts, d.C,
-                                              static_cast<S *>(result));
+  // one workgroup that returns at once unless pairs of one offset share a result row
+  long long expected = 0;
+  for (int k = 0; k < p.K; ++k) {
+    const int64_t n = p.indice_num[k];
+    expected += n < 0 ? 0 : (n > p.L ? p.L : n);
+  }
+  lc.begin("repairLostPairs");
+  repairLostPairs<E><<<1, 256, 0, lc.stream>>>(
+      static_cast<const S *>(gathered), d.Q, static_cast<const S *>(f.base), f.stride_k, sQ, sC,
+      p.indice_pairs, p.L, d.row_col, d.src_col, d.R, d.n_src, p.K, inl, ws.dev_counts, ws.map,
+      ws.filled, n_filled, (int)expected, d.C, RepairScratch{ws.shadow, ws.pool_row, ws.pool},
+      static_cast<S *>(result));
   lc.end();
 }
 

@@ -125,9 +125,7 @@ mluOpStatus_t foolCheckNoPtr(mluOpHandle_t handle, const mluOpTensorDescriptor_t
   // The tensor pair column 0 indexes has indice_pairs.dim[2] rows: input_grad,
   // or output_grad of an inverse convolution.
   const mluOpTensorDescriptor_t col0_desc = inverse == 1 ? output_grad_desc : input_grad_desc;
-  const mluOpTensorDescriptor_t col1_desc = inverse == 1 ? input_grad_desc : output_grad_desc;
   const char *col0_name = inverse == 1 ? "output_grad" : "input_grad";
-  const char *col1_name = inverse == 1 ? "input_grad" : "output_grad";
 
   if (K != indice_pairs_desc->getDimIndex(0)) {
     MLUOP_LOG(ERROR) << api << " The dims[0] of indice_pairs should be equal to kd*kh*kw.";
@@ -164,9 +162,11 @@ mluOpStatus_t foolCheckNoPtr(mluOpHandle_t handle, const mluOpTensorDescriptor_t
       return MLUOP_STATUS_BAD_PARAM;
     }
   }
-  if (col1_desc->getDimIndex(0) < max_indice_num) {
-    MLUOP_LOG(ERROR) << api << " The dims[0] of " << col1_name
-                     << " should be larger than or equal to the maximum number of indice_num.";
+  // (the reference's rule for output_grad; an inverse convolution's input_grad may have fewer
+  // rows than an offset has pairs when the partner layer's coordinates repeat)
+  if (inverse == 0 && output_grad_desc->getDimIndex(0) < max_indice_num) {
+    MLUOP_LOG(ERROR) << api << " The dims[0] of output_grad should be larger than or equal to "
+                     << "the maximum number of indice_num.";
     return MLUOP_STATUS_BAD_PARAM;
   }
   if (sub_m == 1 && K % 2 == 0) {

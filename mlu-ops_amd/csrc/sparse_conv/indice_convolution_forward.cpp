@@ -131,9 +131,9 @@ mluOpStatus_t foolProof(const std::string &api, mluOpHandle_t handle,
 
   for (int64_t i = 0; i < fd.num_filter; ++i) {
     std::string where = "i: " + std::to_string(i) + ".";
-    PARAM_CHECK_V2(api,
-                   indice_num[i] >= 0 && indice_num[i] <= indice_pairs_desc->getDimIndex(2) &&
-                       indice_num[i] <= features_desc->getDimIndex(0),
+    // (no more pairs than the pair lists are long: features_desc->getDimIndex(0) in the
+    // reference, which is the same number unless the convolution is an inverse one)
+    PARAM_CHECK_V2(api, indice_num[i] >= 0 && indice_num[i] <= indice_pairs_desc->getDimIndex(2),
                    where);
   }
   return MLUOP_STATUS_SUCCESS;

@@ -605,10 +605,14 @@ def test_inverse_shape_checks(extended):
     assert _forward_status(extended, [n_in, ci], filt, [K, 2, L], [L + 1, co], num, L + 1, 1) == bad
     assert _forward_status(extended, [n_in, ci], filt, [K, 2, L], [L, co], num, L - 1, 1) == bad
     assert _forward_status(extended, [n_in, ci + 1], filt, [K, 2, L], [L, co], num, L, 1) == bad
-    assert _forward_status(extended, [n_in, ci], filt, [K, 2, L], [L, co], [n_in + 1] * K, L, 1) == bad
+    assert _forward_status(extended, [n_in, ci], filt, [K, 2, L], [L, co], [L + 1] * K, L, 1) == bad
+    # more pairs than input rows is what repeated coordinates in the partner layer give
+    assert _forward_status(extended, [n_in, ci], filt, [K, 2, L], [L, co], [n_in + 1] * K, L, 1) == \
+        STATUS["MLUOP_STATUS_EXECUTION_FAILED"]
     assert _forward_status(extended, [n_in, ci], filt, [K, 2, L], [L, co], num, L, 2) == bad
     assert _backward_data_status(extended, [L + 1, co], filt, [K, 2, L], [n_in, ci], num, 1) == bad
-    assert _backward_data_status(extended, [L, co], filt, [K, 2, L], [2, ci], num, 1) == bad   # fewer rows than pairs
+    assert _backward_data_status(extended, [L, co], filt, [K, 2, L], [2, ci], num, 1) == \
+        STATUS["MLUOP_STATUS_EXECUTION_FAILED"]   # fewer input rows than pairs: repeated coordinates
     assert _backward_data_status(extended, [L, co], filt, [K, 2, L], [n_in, ci + 1], num, 1) == bad
     assert _backward_filter_status(extended, [n_in, ci], [L + 1, co], [K, 2, L], filt, num, 1) == bad
     assert _backward_filter_status(extended, [n_in, ci], [L, co], [K, 2, L], filt, num, 2) == bad

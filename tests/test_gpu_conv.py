@@ -243,3 +243,63 @@ def test_config4_all_ops_full_size(gpu_handle):
              ci=64, co=64, sub_m=True)
     print("config4 ops", flush=True)
     run_all_ops(gpu_handle, c, "float16")
+
+
+# --- pairs of one offset that share a result row -------------------------------------------------
+# Repeated input coordinates make mluOpGetIndicePairs list several inputs for one (offset, output
+# row); made-up pair tensors (test case files) can repeat anything.  The reference adds every pair.
+
+COLLISION_SHAPES = [
+    # (space, L, duplicated rows, ks, ci, co, sub_m, stride, force dense kernel)
+    ((8, 9, 10), 400, 60, (3, 3, 3), 64, 64, True, (1, 1, 1), False),       # pair-list MFMA kernel
+    ((8, 8, 8), 300, 80, (3, 3, 3), 128, 128, True, (1, 1, 1), True),       # register-accumulating kernel
+    ((8, 10, 10), 500, 100, (3, 3, 3), 32, 16, False, (2, 2, 2), False),    # regular, strided
+    ((6, 6, 6), 100, 40, (3, 3, 3), 21, 10, True, (1, 1, 1), False),        # generic FMA kernel
+    ((10, 10, 10), 300, 50, (5, 5, 7), 32, 32, True, (1, 1, 1), False),     # K = 175
+]
+
+
+@pytest.mark.parametrize("shape", COLLISION_SHAPES)
+@pytest.mark.parametrize("dtype_name", ["float32", "float16", "bfloat16"])
+def test_repeated_coordinates_are_all_added(gpu_handle, shape, dtype_name):
+    space, L, dup, ks, ci, co, sub_m, stride, dense = shape
+    print("collision case", shape, dtype_name, flush=True)
+    rng = np.random.default_rng(41)
+    idx = random_voxels(rng, 2, space, L, duplicates=dup)
+    pad = [k // 2 for k in ks]
+    pairs, num, n_out = build_rulebook(idx, 2, space, ks, pad, list(stride), [1, 1, 1], sub_m)
+    K = int(np.prod(ks))
+    # at least one offset lists one output row twice: the case this test is about
+    assert any(len(np.unique(pairs[k, 1, :num[k]])) < num[k] for k in range(K))
+    b = 1.0 / np.sqrt(K * ci)
+    c = dict(idx=idx, pairs=pairs, num=num, n_out=n_out, K=K, ks=ks, ci=ci, co=co, sub_m=sub_m,
+             feats=rng.standard_normal((idx.shape[0], ci)).astype(np.float32),
+             w=rng.uniform(-b, b, size=tuple(ks) + (ci, co)).astype(np.float32),
+             dy=(rng.standard_normal((n_out, co)) * 1e-1).astype(np.float32))
+    if dense:
+        os.environ["MLUOP_SPCONV_DENSE"] = "1"
+    try:
+        run_all_ops(gpu_handle, c, dtype_name)
+    finally:
+        os.environ.pop("MLUOP_SPCONV_DENSE", None)
+
+
+@pytest.mark.parametrize("ci,co", [(64, 64), (13, 70)])
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_made_up_pairs_with_repeats_everywhere(gpu_handle, ci, co, dtype_name):
+    """Uniformly random pair tensors, as a case file's random_data gives them: the same output row
+    many times per offset, the same input row many times per offset, identical pairs twice, and
+    more touched rows than the repair pool holds at once."""
+    rng = np.random.default_rng(42)
+    K, L, n_out = 9, 6000, 6200          # output_grad needs at least as many rows as an offset has pairs
+    pairs = np.full((K, 2, L), -1, dtype=np.int32)
+    num = rng.integers(L // 2, L + 1, size=K)
+    for k in range(K):
+        pairs[k, 0, :num[k]] = rng.integers(0, L, size=num[k])
+        pairs[k, 1, :num[k]] = rng.integers(0, n_out, size=num[k])
+    pairs[0, :, 1] = pairs[0, :, 0]                       # an identical pair, twice
+    c = dict(pairs=pairs, num=num, n_out=n_out, K=K, ks=(1, 3, 3), ci=ci, co=co, sub_m=False,
+             feats=rng.standard_normal((L, ci)).astype(np.float32),
+             w=(rng.standard_normal((1, 3, 3, ci, co)) / np.sqrt(K * ci)).astype(np.float32),
+             dy=(rng.standard_normal((n_out, co)) * 1e-1).astype(np.float32))
+    run_all_ops(gpu_handle, c, dtype_name)
