@@ -492,6 +492,12 @@ def main():
     result["backward_filter_tflops"] = step.conv_flops() / (result["backward_filter_ms"] * 1e-3) / 1e12
 
     result["graph_replay"] = graph_replay_step(torch, m, handle, step, step_ops, args.steps)
+    # Not part of the metric: the forward operator for a caller that promises distinct pairs, which
+    # spares the kernel that checks for pairs of one offset sharing a result row.
+    handle.promise_distinct_pairs(True)
+    _, per_p = time_ops(torch, [("forward", step.forward)], max(args.steps // 2, 5))
+    handle.promise_distinct_pairs(False)
+    result["forward_ms_distinct_pairs_promised"] = median(per_p["forward"])
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(step)
     print(json.dumps(result))

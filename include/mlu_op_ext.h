@@ -45,6 +45,15 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtGetKernelTiming(mluOpHandle_t handle, int in
  *     (kd,) kh, kw, Ci, Co whatever the tag says). */
 mluOpStatus_t MLUOP_WIN_API mluOpExtSetSparseConvExtendedModes(mluOpHandle_t handle, int enable);
 
+/* mluOpIndiceConvolutionForward and mluOpIndiceConvolutionBackwardData add every pair of
+ * indice_pairs, as the reference does, also when several pairs of one offset name the same
+ * result row (which mluOpGetIndicePairs produces for repeated input coordinates, and made-up
+ * pair tensors can hold anywhere).  Finding out costs one small kernel behind every call.  A
+ * caller whose coordinates are distinct (voxelized point clouds are) can promise so: with
+ * `promised` non-zero that kernel is not launched, and a rulebook that breaks the promise loses
+ * all but one of such pairs.  Off by default. */
+mluOpStatus_t MLUOP_WIN_API mluOpExtSetDistinctPairsPromise(mluOpHandle_t handle, int promised);
+
 #if defined(__cplusplus)
 }
 #endif

@@ -143,6 +143,12 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtSetSparseConvExtendedModes(mluOpHandle_t han
   return MLUOP_STATUS_SUCCESS;
 }
 
+mluOpStatus_t MLUOP_WIN_API mluOpExtSetDistinctPairsPromise(mluOpHandle_t handle, int promised) {
+  PARAM_CHECK("[mluOpExtSetDistinctPairsPromise]", handle != NULL);
+  handle->distinct_pairs_promised = promised != 0;
+  return MLUOP_STATUS_SUCCESS;
+}
+
 mluOpStatus_t MLUOP_WIN_API mluOpExtGetKernelTimingCount(mluOpHandle_t handle, int *count) {
   PARAM_CHECK("[mluOpExtGetKernelTimingCount]", handle != NULL);
   PARAM_CHECK("[mluOpExtGetKernelTimingCount]", count != NULL);

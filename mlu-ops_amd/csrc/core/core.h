@@ -37,6 +37,10 @@ struct mluOpContext {
   // Modes the reference rejects (inverse convolution, filters_grad written in its
   // tagged layout): off unless mluOpExtSetSparseConvExtendedModes switched them on.
   bool sparse_conv_extended = false;
+  // The caller's promise that no offset of a rulebook names a result row twice
+  // (mluOpExtSetDistinctPairsPromise): forward and backward data then skip the
+  // check that finds and adds such pairs.
+  bool distinct_pairs_promised = false;
 
   // What the kernel launchers need: the stream, and the timer while it is on.
   mluop::LaunchCtx launchCtx() { return mluop::LaunchCtx(queue, timer.enabled ? &timer : nullptr); }

@@ -40,6 +40,8 @@ struct ConvProblem {
   // Pair column 0 then names rows of the output-side tensors (L of them) and
   // column 1 rows of the input-side tensors (num_out of them).
   bool inverse = false;
+  // The caller promised that no offset names a result row twice: no check for lost pairs.
+  bool distinct_pairs = false;
   // Backward filter only: element strides of dW(k, ci, co) in filters_grad;
   // all zero = the positional [K, Ci, Co].
   int64_t grad_stride_k = 0, grad_stride_ci = 0, grad_stride_co = 0;

@@ -1589,6 +1589,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
                                                 ws.filled, static_cast<S *>(result));
     lc.end();
   }
+  if (p.distinct_pairs) return;
   // one workgroup that returns at once unless pairs of one offset share a result row
   long long expected = 0;
   for (int k = 0; k < p.K; ++k) {

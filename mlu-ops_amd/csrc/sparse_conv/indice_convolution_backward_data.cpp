@@ -292,9 +292,9 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardData(
     PARAM_CHECK(api, workspace != NULL);
   }
 
-  const ConvProblem p =
-      makeProblem(output_grad_desc, filters_desc, indice_pairs_desc, input_grad_desc, indice_num,
-                  inverse, indice_pairs);
+  ConvProblem p = makeProblem(output_grad_desc, filters_desc, indice_pairs_desc, input_grad_desc,
+                              indice_num, inverse, indice_pairs);
+  p.distinct_pairs = handle->distinct_pairs_promised;
   const size_t need =
       mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kBackwardData);
   if (workspace_size < need || workspace == NULL) {

@@ -235,8 +235,9 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionForward(
     PARAM_CHECK(api, workspace != nullptr);
   }
 
-  const ConvProblem p = makeProblem(features_desc, filters_desc, indice_pairs_desc, indice_num,
-                                    num_act_out, inverse, indice_pairs);
+  ConvProblem p = makeProblem(features_desc, filters_desc, indice_pairs_desc, indice_num,
+                              num_act_out, inverse, indice_pairs);
+  p.distinct_pairs = handle->distinct_pairs_promised;
   const size_t need = mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kForward);
   if (workspace_size < need || workspace == nullptr) {
     MLUOP_LOG(ERROR) << api << " workspace of " << workspace_size

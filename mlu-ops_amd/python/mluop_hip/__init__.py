@@ -121,6 +121,7 @@ SIGNATURES = {
     # mlu_op_ext.h
     "mluOpExtSetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int]),
     "mluOpExtSetSparseConvExtendedModes": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "mluOpExtSetDistinctPairsPromise": (ctypes.c_int, [_vp, ctypes.c_int]),
     "mluOpExtGetKernelTimingCount": (ctypes.c_int, [_vp, _ip]),
     "mluOpExtGetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int, ctypes.POINTER(ctypes.c_char_p),
                                                ctypes.POINTER(ctypes.c_float)]),
@@ -181,6 +182,10 @@ class Handle:
     def set_extended_modes(self, enable):
         """Accept inverse = 1 and tagged filters_grad layouts, which the reference rejects."""
         check(lib().mluOpExtSetSparseConvExtendedModes(self.ptr, 1 if enable else 0))
+
+    def promise_distinct_pairs(self, promised):
+        """No offset of the rulebooks names a result row twice: skip the check for lost pairs."""
+        check(lib().mluOpExtSetDistinctPairsPromise(self.ptr, 1 if promised else 0))
 
     def kernel_timings(self):
         """[(kernel name, milliseconds)] per launch since timing was enabled (waits for the queue)."""

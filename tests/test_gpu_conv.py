@@ -303,3 +303,33 @@ def test_made_up_pairs_with_repeats_everywhere(gpu_handle, ci, co, dtype_name):
              w=(rng.standard_normal((1, 3, 3, ci, co)) / np.sqrt(K * ci)).astype(np.float32),
              dy=(rng.standard_normal((n_out, co)) * 1e-1).astype(np.float32))
     run_all_ops(gpu_handle, c, dtype_name)
+
+
+def test_distinct_pairs_promise_skips_the_check(gpu_handle):
+    """With the promise the check kernel is not launched (one kernel fewer per call) and a rulebook
+    with distinct pairs gives the same bits; the default handle launches it."""
+    import torch
+    import mluop_hip
+    c = conv_case(43, 2, (8, 9, 10), 400, (3, 3, 3), 64, 64, True)
+    feats_t = to_torch(round_to(c["feats"], "float16"), "float16", "cuda")
+    w_t = to_torch(round_to(c["w"], "float16"), "float16", "cuda")
+    pairs_t = torch.from_numpy(c["pairs"]).cuda()
+    num_host = [int(v) for v in c["num"]]
+
+    def forward_and_kernels():
+        gpu_handle.set_kernel_timing(True)
+        out = mluop_hip.indice_conv_forward(gpu_handle, feats_t, w_t, mluop_hip.LAYOUT_ARRAY, pairs_t, num_host,
+                                            c["n_out"], True)
+        names = [name for name, _ in gpu_handle.kernel_timings()]
+        gpu_handle.set_kernel_timing(False)
+        return out, names
+
+    checked, names = forward_and_kernels()
+    assert names[-1] == "repairLostPairs"
+    gpu_handle.promise_distinct_pairs(True)
+    try:
+        promised, names_promised = forward_and_kernels()
+    finally:
+        gpu_handle.promise_distinct_pairs(False)
+    assert "repairLostPairs" not in names_promised and len(names_promised) == len(names) - 1
+    assert torch.equal(checked, promised)
