@@ -809,15 +809,16 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
 // A touched row is rebuilt in an fp32 pool (kRepairPoolRows rows, indexed through
 // `shadow`): first the partners its map slots hold, as the kernel summed them, then
 // the lost pairs as the scan meets them, and it is rounded into the result once,
-// when the scan ends: the same single rounding as any other row.  (A row that has
-// to leave a full pool early and is touched again continues from its rounded value.)
-// Which of the colliding pairs owned the slot depends on the order their stores
-// landed in, so the last bits of such rows can differ from run to run; rows without
+// the same single rounding as any other row.  When more pairs are lost than the
+// pool has rows, the scan is repeated per block of kRepairPoolRows result rows and
+// looks only at the pairs of that block, so a row is never rebuilt twice.  Which
+// of the colliding pairs owned the slot depends on the order their stores landed
+// in, so the last bits of such rows can differ from run to run; rows without
 // collisions are not touched.
 constexpr int kRepairPoolRows = 2048;
 
 struct RepairScratch {
-  int32_t *shadow;    // [R] pool row of a result row; -1 never pooled, -2 rounded back already
+  int32_t *shadow;    // [R] pool row of a result row, or -1
   int32_t *pool_row;  // [kRepairPoolRows] result row of a pool row
   float *pool;        // [kRepairPoolRows, C]
 };
@@ -848,68 +849,59 @@ __global__ __launch_bounds__(256) void repairLostPairs(
   for (int i = tid; i < R; i += 256) scratch.shadow[i] = -1;
   if (tid == 0) s_pooled = 0;
   __syncthreads();
-  // rounds the pool back into the result and empties it
-  auto flush = [&]() {
-    const int n = s_pooled;
-    for (int i = 0; i < n; ++i) {
-      const int r = scratch.pool_row[i];
-      for (int c = tid; c < C; c += 256)
-        E::store(result + (size_t)r * C + c, scratch.pool[(size_t)i * C + c]);
-      if (tid == 0) scratch.shadow[r] = -2;
-    }
-    __syncthreads();
-    if (tid == 0) s_pooled = 0;
-    __syncthreads();
-  };
-  for (int k = 0; k < K; ++k) {
-    const int n = offsetCount(inl, dev_counts, k);
-    const int32_t *base = pairs + (size_t)k * 2 * L;
-    for (int p0 = 0; p0 < n; p0 += 256) {
-      const int p = p0 + tid;
-      int r = -1, src = -1;
-      bool lost = false;
-      if (p < n) {
-        r = base[(size_t)row_col * L + p];
-        src = base[(size_t)src_col * L + p];
-        if ((unsigned)r < (unsigned)R && (unsigned)src < (unsigned)n_src) {
-          int32_t *slot = map + (size_t)k * R + r;
-          // the claimed slot holds -2 - partner: no pair finds itself there twice
-          lost = !(*slot == src && atomicCAS(slot, src, -2 - src) == src);
-        }
-      }
-      // lost pairs of this step in pair order
-      const unsigned long long b = __ballot(lost);
-      if (lane == 0) s_wave_lost[wave] = __popcll(b);
-      __syncthreads();
-      int before = 0, total = 0;
-      for (int w = 0; w < 4; ++w) {
-        if (w < wave) before += s_wave_lost[w];
-        total += s_wave_lost[w];
-      }
-      if (lost) {
-        const int at = before + __popcll(b & ((1ull << lane) - 1ull));
-        s_row[at] = r;
-        s_src[at] = src;
-      }
-      __syncthreads();
-      for (int i = 0; i < total; ++i) {
-        const int row = s_row[i];
-        int at = scratch.shadow[row];
-        if (at < 0) {
-          const bool first_time = at == -1;
-          if (s_pooled == kRepairPoolRows) flush();
-          at = s_pooled;
-          __syncthreads();  // everybody has read the pool's fill state
-          if (tid == 0) {
-            scratch.shadow[row] = at;
-            scratch.pool_row[at] = row;
-            s_pooled = at + 1;
+  // no more rows can be touched than pairs are lost (or lie outside their tensors)
+  const int n_pass = expected - s_found <= kRepairPoolRows
+                         ? 1
+                         : (R + kRepairPoolRows - 1) / kRepairPoolRows;
+  for (int pass = 0; pass < n_pass; ++pass) {
+    const int r_lo = n_pass == 1 ? 0 : pass * kRepairPoolRows;
+    const int r_hi = n_pass == 1 ? R : (r_lo + kRepairPoolRows < R ? r_lo + kRepairPoolRows : R);
+    for (int k = 0; k < K; ++k) {
+      const int n = offsetCount(inl, dev_counts, k);
+      const int32_t *base = pairs + (size_t)k * 2 * L;
+      for (int p0 = 0; p0 < n; p0 += 256) {
+        const int p = p0 + tid;
+        int r = -1, src = -1;
+        bool lost = false;
+        if (p < n) {
+          r = base[(size_t)row_col * L + p];
+          src = base[(size_t)src_col * L + p];
+          if (r >= r_lo && r < r_hi && (unsigned)src < (unsigned)n_src) {
+            int32_t *slot = map + (size_t)k * R + r;
+            // the claimed slot holds -2 - partner: no pair finds itself there twice
+            lost = !(*slot == src && atomicCAS(slot, src, -2 - src) == src);
           }
-          for (int c = tid; c < C; c += 256) {
-            float sum = 0.f;
-            if (first_time) {
-              // what the gather kernel summed: the partner every slot of the row holds
-              // (claimed slots hold -2 - partner)
+        }
+        // lost pairs of this step in pair order
+        const unsigned long long b = __ballot(lost);
+        if (lane == 0) s_wave_lost[wave] = __popcll(b);
+        __syncthreads();
+        int before = 0, total = 0;
+        for (int w = 0; w < 4; ++w) {
+          if (w < wave) before += s_wave_lost[w];
+          total += s_wave_lost[w];
+        }
+        if (lost) {
+          const int at = before + __popcll(b & ((1ull << lane) - 1ull));
+          s_row[at] = r;
+          s_src[at] = src;
+        }
+        __syncthreads();
+        for (int i = 0; i < total; ++i) {
+          const int row = s_row[i];
+          int at = scratch.shadow[row];
+          if (at < 0) {
+            at = s_pooled;
+            __syncthreads();  // everybody has read the pool's fill state
+            if (tid == 0) {
+              scratch.shadow[row] = at;
+              scratch.pool_row[at] = row;
+              s_pooled = at + 1;
+            }
+            // what the gather kernel summed: the partner every slot of the row holds
+            // (claimed slots hold -2 - partner)
+            for (int c = tid; c < C; c += 256) {
+              float sum = 0.f;
               for (int kk = 0; kk < K; ++kk) {
                 const int m = map[(size_t)kk * R + row];
                 if (m == -1) continue;
@@ -919,24 +911,31 @@ __global__ __launch_bounds__(256) void repairLostPairs(
                 for (int q = 0; q < Q; ++q) dot += E::load(a + q) * E::load(w + (size_t)q * sQ);
                 sum += dot;
               }
-            } else {
-              sum = E::load(result + (size_t)row * C + c);
+              scratch.pool[(size_t)at * C + c] = sum;
             }
-            scratch.pool[(size_t)at * C + c] = sum;
           }
+          const typename E::storage *a = A + (size_t)s_src[i] * Q;
+          for (int c = tid; c < C; c += 256) {
+            const typename E::storage *w = W + (size_t)k * sK + (size_t)c * sC;
+            float dot = 0.f;
+            for (int q = 0; q < Q; ++q) dot += E::load(a + q) * E::load(w + (size_t)q * sQ);
+            scratch.pool[(size_t)at * C + c] += dot;
+          }
+          __syncthreads();  // shadow and the pool row are in place for the next pair
         }
-        const typename E::storage *a = A + (size_t)s_src[i] * Q;
-        for (int c = tid; c < C; c += 256) {
-          const typename E::storage *w = W + (size_t)k * sK + (size_t)c * sC;
-          float dot = 0.f;
-          for (int q = 0; q < Q; ++q) dot += E::load(a + q) * E::load(w + (size_t)q * sQ);
-          scratch.pool[(size_t)at * C + c] += dot;
-        }
-        __syncthreads();  // shadow and the pool row are in place for the next pair
       }
     }
+    // round the rebuilt rows into the result; their pool rows are free again
+    const int pooled = s_pooled;
+    for (int i = 0; i < pooled; ++i) {
+      const int r = scratch.pool_row[i];
+      for (int c = tid; c < C; c += 256)
+        E::store(result + (size_t)r * C + c, scratch.pool[(size_t)i * C + c]);
+    }
+    __syncthreads();
+    if (tid == 0) s_pooled = 0;
+    __syncthreads();
   }
-  flush();
 }
 
 // ---- backward filter -------------------------------------------------------------

@@ -256,6 +256,7 @@ COLLISION_SHAPES = [
     ((8, 10, 10), 500, 100, (3, 3, 3), 32, 16, False, (2, 2, 2), False),    # regular, strided
     ((6, 6, 6), 100, 40, (3, 3, 3), 21, 10, True, (1, 1, 1), False),        # generic FMA kernel
     ((10, 10, 10), 300, 50, (5, 5, 7), 32, 32, True, (1, 1, 1), False),     # K = 175
+    ((32, 8, 35), 5000, 3000, (3, 3, 5), 128, 32, True, (1, 1, 1), False),  # more lost pairs than the repair pool has rows
 ]
 
 
