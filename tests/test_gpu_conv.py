@@ -334,3 +334,38 @@ def test_distinct_pairs_promise_skips_the_check(gpu_handle):
         gpu_handle.promise_distinct_pairs(False)
     assert "repairLostPairs" not in names_promised and len(names_promised) == len(names) - 1
     assert torch.equal(checked, promised)
+
+
+def _offset_view(torch, t, elements=1):
+    """The same values at an address `elements` past a fresh allocation: not 16-byte aligned."""
+    flat = torch.empty(t.numel() + 8, dtype=t.dtype, device=t.device)
+    view = flat[elements:elements + t.numel()].view(t.shape)
+    view.copy_(t)
+    assert view.data_ptr() % 16 != 0
+    return view
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "float16"])
+def test_tensors_that_are_not_16_byte_aligned(gpu_handle, dtype_name):
+    """Feature, gradient, filter and pair tensors at odd addresses: the kernels that move rows with
+    16-byte accesses step aside for the generic ones, and the numbers stay the same."""
+    import torch
+    import mluop_hip
+    c = conv_case(44, 2, (8, 9, 10), 400, (3, 3, 3), 64, 64, True)
+    feats_r, w_r, dy_r = (round_to(c[k], dtype_name) for k in ("feats", "w", "dy"))
+    w_k = w_r.reshape(c["K"], c["ci"], c["co"])
+    feats_t = _offset_view(torch, to_torch(feats_r, dtype_name, "cuda"))
+    w_t = _offset_view(torch, to_torch(w_r, dtype_name, "cuda"))
+    dy_t = _offset_view(torch, to_torch(dy_r, dtype_name, "cuda"))
+    pairs_t = _offset_view(torch, torch.from_numpy(c["pairs"]).cuda())
+    num_host = [int(v) for v in c["num"]]
+    out = mluop_hip.indice_conv_forward(gpu_handle, feats_t, w_t, mluop_hip.LAYOUT_ARRAY, pairs_t, num_host,
+                                        c["n_out"], True)
+    dx = mluop_hip.indice_conv_backward_data(gpu_handle, dy_t, w_t, mluop_hip.LAYOUT_ARRAY, pairs_t, num_host, True,
+                                             c["ci"])
+    dw = mluop_hip.indice_conv_backward_filter(gpu_handle, feats_t, dy_t, pairs_t, num_host, c["ks"], True)
+    torch.cuda.synchronize()
+    check_close(from_torch(out), oracle.forward(feats_r, w_k, c["pairs"], c["num"], c["n_out"]), dtype_name, "forward")
+    check_close(from_torch(dx), oracle.backward_data(dy_r, w_k, c["pairs"], c["num"]), dtype_name, "backward_data")
+    ref = oracle.backward_filter(feats_r, dy_r, c["pairs"], c["num"], fast=True)
+    check_close(from_torch(dw).reshape(ref.shape), ref, dtype_name, "backward_filter")

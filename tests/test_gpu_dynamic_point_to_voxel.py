@@ -159,3 +159,26 @@ def test_backward_mean_is_rejected_like_the_reference(gpu_handle):
     with pytest.raises(mluop_hip.MluOpError) as e:
         mluop_hip.dynamic_point_to_voxel_backward(gpu_handle, z, z, z, i4, i4, i4[:1], "mean")
     assert e.value.status == mluop_hip.STATUS_BAD_PARAM
+
+
+def test_inputs_at_odd_addresses(gpu_handle):
+    """feats and coors as views one element into their allocations (4-byte aligned only)."""
+    import torch
+    import mluop_hip
+    rng = np.random.default_rng(13)
+    n, c = 3000, 5
+    feats = rng.uniform(-100, 100, (n, c)).astype(np.float32)
+    coors = rng.integers(0, 9, (n, 3)).astype(np.int32)
+    ff = torch.empty(feats.size + 8, dtype=torch.float32, device="cuda")
+    fv = ff[1:1 + feats.size].view(feats.shape)
+    fv.copy_(torch.from_numpy(feats))
+    cc = torch.empty(coors.size + 8, dtype=torch.int32, device="cuda")
+    cv = cc[1:1 + coors.size].view(coors.shape)
+    cv.copy_(torch.from_numpy(coors))
+    assert fv.data_ptr() % 16 != 0 and cv.data_ptr() % 16 != 0
+    for mode in ("max", "mean"):
+        cv.copy_(torch.from_numpy(coors))
+        out = mluop_hip.dynamic_point_to_voxel_forward(gpu_handle, fv, cv, mode)
+        torch.cuda.synchronize()
+        got = [t.cpu().numpy() for t in out[:4]] + [int(out[4].item()), cv.cpu().numpy()]
+        assert_same(got, dpv.forward(mode, feats, coors))

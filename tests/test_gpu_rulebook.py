@@ -163,3 +163,27 @@ def test_largest_accepted_input_one_million_rows(gpu_handle):
     compare(gpu_handle, idx, 2, space, (3, 3, 3), [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
     print("regular 1M", flush=True)
     compare(gpu_handle, idx, 2, space, (2, 2, 2), [0, 0, 0], [2, 2, 2], [1, 1, 1], False)
+
+
+@pytest.mark.parametrize("sub_m", [True, False])
+def test_indices_that_are_not_16_byte_aligned(gpu_handle, sub_m):
+    """The (n, d, h, w) rows are read with one 16-byte load each when the tensor allows it; a tensor
+    at an odd address takes the element-wise path and gives the same rulebook."""
+    import torch
+    import mluop_hip
+    rng = np.random.default_rng(51)
+    batch, space, ks = 2, (8, 9, 10), (3, 3, 3)
+    idx = random_voxels(rng, batch, space, 500)
+    pad, stride, dil = [1, 1, 1], ([1, 1, 1] if sub_m else [2, 2, 2]), [1, 1, 1]
+    ospace = list(space) if sub_m else out_space(space, ks, pad, stride, dil)
+    flat = torch.empty(idx.size + 8, dtype=torch.int32, device="cuda")
+    t = flat[1:1 + idx.size].view(idx.shape)
+    t.copy_(torch.from_numpy(idx))
+    assert t.data_ptr() % 16 != 0
+    pairs, out_idx, num, n_out = mluop_hip.get_indice_pairs(gpu_handle, t, batch, space, ks, ospace, pad, stride, dil,
+                                                           sub_m)
+    torch.cuda.synchronize()
+    rp, ro, rn, rn_out = oracle.get_indice_pairs(idx, batch, pad, stride, dil, ks, ospace, sub_m,
+                                                 out_rows=out_idx.shape[0], exact_count=True)
+    assert n_out == rn_out and np.array_equal(num.cpu().numpy(), rn)
+    assert np.array_equal(pairs.cpu().numpy(), rp) and np.array_equal(out_idx.cpu().numpy(), ro)

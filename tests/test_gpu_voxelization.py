@@ -97,3 +97,21 @@ def test_statuses(gpu_handle):
     # zero caps: success, nothing written, no workspace asked for
     out = mluop_hip.voxelization(gpu_handle, pts, vs, cr, 0, 3)
     assert out[0].shape == (3, 0, 4)
+
+
+def test_points_at_an_odd_address(gpu_handle):
+    """A points tensor that is only 4-byte aligned (a view one element into its allocation)."""
+    import torch
+    import mluop_hip
+    rng = np.random.default_rng(12)
+    pts = lidar_like_points(rng, 3000, features=4, spread=(8.0, 4.0, 2.0))
+    vs, cr = [0.4, 0.4, 1.0], [0.0, -4.0, -2.0, 8.0, 4.0, 1.0]
+    flat = torch.empty(pts.size + 8, dtype=torch.float32, device="cuda")
+    view = flat[1:1 + pts.size].view(pts.shape)
+    view.copy_(torch.from_numpy(pts))
+    assert view.data_ptr() % 16 != 0
+    out = mluop_hip.voxelization(gpu_handle, view, torch.tensor(vs, dtype=torch.float32).cuda(),
+                                 torch.tensor(cr, dtype=torch.float32).cuda(), 5, 2000)
+    torch.cuda.synchronize()
+    got = (out[0].cpu().numpy(), out[1].cpu().numpy(), out[2].cpu().numpy(), int(out[3].item()))
+    assert_same(got, vox.voxelization(pts, vs, cr, 5, 2000))
