@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import sparse_conv_oracle as oracle
-from spconv_cases import THRESH, check_close, from_torch, out_space, round_to, to_torch
+from spconv_cases import THRESH, check_close, from_torch, out_space, random_voxels, round_to, to_torch
 
 pytestmark = [pytest.mark.gpu, pytest.mark.timeout(900)]
 
@@ -157,3 +157,51 @@ def test_config5b_regular_2x2x2_stride2_on_5a_outputs(gpu_handle, config5_voxels
     rows = np.sort(rng.choice(n_out, size=3000, replace=False))
     ref = sampled_rows_reference(feats, w.reshape(8, 128, 128), pairs.cpu().numpy(), num_host, rows)
     grade_sample(from_torch(out[torch.from_numpy(rows).cuda()]), ref, "float16", "config5b fp16")
+
+
+@pytest.mark.timeout(600)
+def test_convolutions_at_one_million_rows(gpu_handle):
+    """The most rows the API accepts (1 000 000), submanifold 3x3x3 at 64 channels fp16, checked
+    through properties that need no CPU pass over the whole tensor: a filter that is the identity at
+    the centre offset and zero elsewhere returns its input bit for bit (forward and backward data);
+    a random filter is compared with numpy on 2 000 sampled rows; the centre slice of the filter
+    gradient is the dense product X^T dY, computed by torch in fp32."""
+    import torch
+    import mluop_hip as m
+    rng = np.random.default_rng(91)
+    space, L, C, ks = (48, 512, 512), 1000000, 64, (3, 3, 3)
+    idx = random_voxels(rng, 2, space, L)
+    print("rulebook 1M", flush=True)
+    pairs, out_idx, num, n_out = m.get_indice_pairs(gpu_handle, torch.from_numpy(idx).cuda(), 2, space, ks, list(space),
+                                                    [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+    num_host = num.cpu().tolist()
+    assert n_out == L and num_host[13] == L
+    x = torch.randn(L, C, device="cuda").half()
+    dy = (torch.randn(L, C, device="cuda") * 0.1).half()
+    eye = torch.zeros(ks + (C, C), device="cuda", dtype=torch.float16)
+    eye[1, 1, 1] = torch.eye(C, device="cuda", dtype=torch.float16)
+    print("identity filter", flush=True)
+    out = m.indice_conv_forward(gpu_handle, x, eye, m.LAYOUT_ARRAY, pairs, num_host, L, True)
+    dx = m.indice_conv_backward_data(gpu_handle, dy, eye, m.LAYOUT_ARRAY, pairs, num_host, True, C)
+    torch.cuda.synchronize()
+    assert torch.equal(out, x) and torch.equal(dx, dy)
+
+    print("random filter, sampled rows", flush=True)
+    w = (torch.randn(ks + (C, C), device="cuda") / np.sqrt(27 * C)).half()
+    out = m.indice_conv_forward(gpu_handle, x, w, m.LAYOUT_ARRAY, pairs, num_host, L, True)
+    dw = m.indice_conv_backward_filter(gpu_handle, x, dy, pairs, num_host, ks, True)
+    torch.cuda.synchronize()
+    rows = rng.choice(L, size=2000, replace=False)
+    pn = pairs.cpu().numpy()
+    xf, wf = x.float().cpu().numpy(), w.float().cpu().numpy().reshape(27, C, C)
+    ref = np.zeros((2000, C), np.float64)
+    pos = {int(r): i for i, r in enumerate(rows)}
+    for k in range(27):
+        o = pn[k, 1, :num_host[k]]
+        sel = np.nonzero(np.isin(o, rows))[0]
+        for p in sel:
+            ref[pos[int(o[p])]] += xf[pn[k, 0, p]].astype(np.float64) @ wf[k]
+    got = out[torch.from_numpy(rows).cuda()].float().cpu().numpy()
+    check_close(got, ref.astype(np.float32), "float16", "forward, sampled rows")
+    centre = (x.float().t() @ dy.float()).cpu().numpy()
+    check_close(dw[1, 1, 1].float().cpu().numpy(), centre, "float16", "backward filter, centre offset")

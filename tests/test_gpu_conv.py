@@ -92,6 +92,7 @@ SHAPES = [
     (1, (20, 20, 20), 300, (3, 3, 3), 128, 128, True, (1, 1, 1)),  # sparse: two 64-column halves
     (1, (6, 6, 6), 100, (3, 3, 3), 21, 10, True, (1, 1, 1)),   # odd channel counts -> SIMT
     (1, (6, 6, 6), 100, (1, 3, 3), 13, 70, False, (1, 2, 1)),
+    (1, (6, 6, 6), 120, (3, 3, 3), 260, 300, True, (1, 1, 1)),   # wider than any matrix-core instance
     (1, (10, 10, 10), 400, (5, 5, 7), 32, 32, True, (1, 1, 1)),   # K = 175: counts in device memory, seven chunks of offsets
 ]
 
