@@ -288,7 +288,8 @@ def run_backbone(args, torch, m):
     net = torch.nn.ModuleList(layers).cuda().half()
 
     def step():
-        x = spnn.SparseTensor(feats.clone().requires_grad_(True), indices, grid[1:], grid[0])
+        # the voxels are distinct, as a voxelizer's output is: the layers skip the collision check
+        x = spnn.SparseTensor(feats.clone().requires_grad_(True), indices, grid[1:], grid[0], distinct=True)
         for layer in net:
             x = layer(x)
             x = x.replace_features(torch.relu(x.features))
@@ -304,7 +305,7 @@ def run_backbone(args, torch, m):
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
     rows = [int(idx.shape[0])]
-    x = spnn.SparseTensor(feats, indices, grid[1:], grid[0])
+    x = spnn.SparseTensor(feats, indices, grid[1:], grid[0], distinct=True)
     with torch.no_grad():
         for layer in net:
             x = layer(x)

@@ -35,7 +35,10 @@ class Rulebook:
     """indice_pairs [K,2,L] (device), indice_num as host ints, out_indices, num_act_out."""
 
     def __init__(self, pairs, out_indices, indice_num_host, num_act_out, filter_space, sub_m, out_space,
-                 in_indices=None, in_space=None):
+                 in_indices=None, in_space=None, distinct=False):
+        # the input coordinates were distinct: no offset names a result row twice, and the
+        # operators may skip their check for such pairs (mluOpExtSetDistinctPairsPromise)
+        self.distinct = distinct
         self.in_indices = in_indices  # what an inverse convolution over this rulebook gives back
         self.in_space = None if in_space is None else tuple(in_space)
         self.pairs = pairs
@@ -48,7 +51,11 @@ class Rulebook:
 
 
 class SparseTensor:
-    def __init__(self, features, indices, spatial_shape, batch_size, rulebooks=None):
+    """`distinct=True` is the caller's word that no coordinate occurs twice (the output of a
+    voxelizer, or of a strided layer, never repeats one); the convolution operators then skip
+    their check for pairs of one offset that share a result row."""
+
+    def __init__(self, features, indices, spatial_shape, batch_size, rulebooks=None, distinct=False):
         assert indices.dtype == torch.int32 and indices.dim() == 2 and indices.shape[1] == 4
         assert features.shape[0] == indices.shape[0]
         self.features = features
@@ -56,9 +63,11 @@ class SparseTensor:
         self.spatial_shape = tuple(int(s) for s in spatial_shape)
         self.batch_size = int(batch_size)
         self.rulebooks = {} if rulebooks is None else rulebooks
+        self.distinct = bool(distinct)
 
     def replace_features(self, features):
-        return SparseTensor(features, self.indices, self.spatial_shape, self.batch_size, self.rulebooks)
+        return SparseTensor(features, self.indices, self.spatial_shape, self.batch_size, self.rulebooks,
+                            self.distinct)
 
     def dense(self):
         """[N, C, D, H, W] dense tensor (for inspection and tests)."""
@@ -76,6 +85,7 @@ class _IndiceConv(torch.autograd.Function):
         handle = _handle()
         features = features.contiguous()
         weight = weight.contiguous()
+        handle.promise_distinct_pairs(rulebook.distinct)
         if inverse:
             # the partner layer's rulebook backwards: one output row per input row of the partner
             out = indice_conv_forward(handle, features, weight, LAYOUT_ARRAY, rulebook.pairs, rulebook.indice_num,
@@ -93,6 +103,7 @@ class _IndiceConv(torch.autograd.Function):
         features, weight = ctx.saved_tensors
         rb = ctx.rulebook
         handle = _handle()
+        handle.promise_distinct_pairs(rb.distinct)
         grad_out = grad_out.contiguous()
         grad_features = grad_weight = None
         inverse, sub_m = (1, False) if ctx.inverse else (0, rb.sub_m)
@@ -150,7 +161,7 @@ class _ConvBase(torch.nn.Module):
             self.stride, self.dilation, self.sub_m)
         # the operators take indice_num as host int64: one device-to-host copy per rulebook
         rb = Rulebook(pairs, out_indices[:n_out], num.cpu().tolist(), n_out, self.kernel_size, self.sub_m,
-                      out_space, in_indices=x.indices, in_space=x.spatial_shape)
+                      out_space, in_indices=x.indices, in_space=x.spatial_shape, distinct=x.distinct)
         if self.indice_key is not None:
             x.rulebooks[self.indice_key] = rb
         return rb
@@ -158,8 +169,10 @@ class _ConvBase(torch.nn.Module):
     def _result(self, x, rb, feats):
         if self.sub_m:
             return x.replace_features(feats)
-        # the cache travels on, so that an inverse layer downstream finds this rulebook by its key
-        return SparseTensor(feats, rb.out_indices.contiguous(), rb.out_space, x.batch_size, x.rulebooks)
+        # the cache travels on, so that an inverse layer downstream finds this rulebook by its key;
+        # the active output cells of a regular convolution are distinct by construction
+        return SparseTensor(feats, rb.out_indices.contiguous(), rb.out_space, x.batch_size, x.rulebooks,
+                            distinct=True)
 
     def forward(self, x):
         rb = self._rulebook(x)
@@ -217,7 +230,7 @@ class SparseInverseConv3d(_ConvBase):
         return rb
 
     def _result(self, x, rb, feats):
-        return SparseTensor(feats, rb.in_indices, rb.in_space, x.batch_size, x.rulebooks)
+        return SparseTensor(feats, rb.in_indices, rb.in_space, x.batch_size, x.rulebooks, distinct=rb.distinct)
 
 
 class Voxelization(torch.nn.Module):
@@ -253,4 +266,6 @@ def mean_voxel_features(voxels, num_points_per_voxel):
 def sparse_tensor_from_voxels(features, coors, spatial_shape, batch_index=0, batch_size=1):
     """SparseTensor of one cloud's voxels: indices (n, z, y, x) with n = batch_index."""
     n = torch.full((coors.shape[0], 1), int(batch_index), dtype=torch.int32, device=coors.device)
-    return SparseTensor(features, torch.cat([n, coors.to(torch.int32)], dim=1), spatial_shape, batch_size)
+    # a voxelizer emits every voxel once
+    return SparseTensor(features, torch.cat([n, coors.to(torch.int32)], dim=1), spatial_shape, batch_size,
+                        distinct=True)

@@ -211,3 +211,42 @@ def test_inverse_layer_returns_to_the_partner_layers_cells(gpu_handle):
     np.testing.assert_allclose(x.grad.cpu().numpy(), rx.grad.numpy(), rtol=1e-4, atol=1e-4)
     np.testing.assert_allclose(down.weight.grad.cpu().numpy(), w1.grad.numpy(), rtol=1e-4, atol=2e-4)
     np.testing.assert_allclose(up.weight.grad.cpu().numpy(), w2.grad.numpy(), rtol=1e-4, atol=2e-4)
+
+
+def test_repeated_coordinates_through_the_layers(gpu_handle):
+    """A tensor whose coordinates repeat (not marked distinct): the submanifold layer adds every
+    pair, as the dense reference does when the repeated rows' features are summed per cell... which
+    is not what a last-writer-wins rulebook means, so the reference here is the CPU oracle; and a
+    tensor marked distinct skips the operators' collision check."""
+    import torch
+    import mluop_hip
+    import sparse_conv_oracle as oracle
+    from mluop_hip import nn as spnn
+    rng = np.random.default_rng(25)
+    batch, space, L, ci, co = 1, (8, 9, 10), 300, 16, 32
+    idx = random_voxels(rng, batch, space, L, duplicates=60)
+    feats = rng.standard_normal((idx.shape[0], ci)).astype(np.float32)
+    layer = spnn.SubMConv3d(ci, co, 3).cuda()
+    st = spnn.SparseTensor(torch.from_numpy(feats).cuda(), torch.from_numpy(idx).cuda(), space, batch)
+    assert not st.distinct
+    out = layer(st).features
+    torch.cuda.synchronize()
+    pairs, out_idx, num, n_out = oracle.get_indice_pairs(idx, batch, [1, 1, 1], [1, 1, 1], [1, 1, 1], [3, 3, 3],
+                                                         list(space), True, exact_count=True)
+    w = layer.weight.detach().cpu().numpy().reshape(27, ci, co)
+    ref = oracle.forward(feats, w, pairs, num, n_out)
+    np.testing.assert_allclose(out.detach().cpu().numpy(), ref, rtol=1e-4, atol=1e-5)
+
+    h = spnn._handle()
+    clean = random_voxels(rng, batch, space, L)
+    x = torch.from_numpy(rng.standard_normal((L, ci)).astype(np.float32)).cuda()
+    for distinct, expect_check in ((False, True), (True, False)):
+        st = spnn.SparseTensor(x, torch.from_numpy(clean).cuda(), space, batch, distinct=distinct)
+        h.set_kernel_timing(True)
+        y = layer(st)
+        names = [n for n, _ in h.kernel_timings()]
+        h.set_kernel_timing(False)
+        assert ("repairLostPairs" in names) == expect_check
+        assert y.distinct == distinct
+    down = spnn.SparseConv3d(ci, co, 3, stride=2, padding=1).cuda()
+    assert down(spnn.SparseTensor(x, torch.from_numpy(clean).cuda(), space, batch)).distinct
