@@ -1,4 +1,5 @@
-"""Test-case files in the reference's prototxt form, for the four sparse-convolution operators.
+"""Test-case files in the reference's prototxt form, for the four sparse-convolution operators
+and the three operators upstream of them (voxelization, dynamic point-to-voxel forward/backward).
 
 The reference's gtest replays one operator call per case file: a protobuf `Node` in text format
 with `op_name`, `input {}` / `output {}` tensors (id, shape.dims, layout, dtype, and the values as
@@ -22,6 +23,21 @@ without a schema and takes the field names from the executors that consume them:
   indice_convolution_backward_param { indice_num[] sub_m inverse }
       (zoo/indice_convolution_backward_filter/indice_convolution_backward_filter.cpp:37-42)
       tensors: inputs features, output_grad, indice_pairs; output filters_grad
+  voxelization_param { max_points max_voxels ndim deterministic }   (zoo/voxelization/voxelization.cpp:47-54)
+      tensors: inputs points, voxel_size, coors_range; outputs voxels, coors,
+      num_points_per_voxel, voxel_num                                                 (:62-90)
+  dynamic_point_to_voxel_forward_param { reduce_type: REDUCE_MODE_MAX | REDUCE_MODE_MEAN }
+      (zoo/dynamic_point_to_voxel_forward/dynamic_point_to_voxel_forward.cpp:60-70)
+      tensors: inputs feats, coors; outputs voxel_feats, voxel_coors, point2voxel_map,
+      voxel_points_count, voxel_num                                                   (:71-85)
+  dynamic_point_to_voxel_backward_param { reduce_type }
+      (zoo/dynamic_point_to_voxel_backward/dynamic_point_to_voxel_backward.cpp:44-47)
+      tensors: inputs grad_voxel_feats, feats, voxel_feats, point2voxel_map, voxel_points_count,
+      voxel_num; output grad_feats
+
+A tensor may list fewer values than its shape has elements (the reference's own backward case
+does): the parser takes the element count from the value list and warns (parser.cpp:371-383), the
+rest of the buffer stays zero, and so it does here.
 
 `random_data` tensors are filled by numpy's generator from the recipe's seed and bounds: the
 distribution is the recipe's, the bit stream is not the reference generator's, so a case whose
@@ -229,7 +245,9 @@ class CaseTensor:
         for field in ("value_i", "value_l"):
             if msg.has(field):
                 vals = np.array(msg.all(field), dtype=np.int64)
-                assert vals.size == n, "%s: %d values for %d elements" % (self.id, vals.size, n)
+                assert vals.size <= n, "%s: %d values for %d elements" % (self.id, vals.size, n)
+                if vals.size < n:
+                    vals = np.concatenate([vals, np.zeros(n - vals.size, np.int64)])
                 if int_like:
                     return vals.astype(np.int32).reshape(self.shape)
                 # value_i of a floating tensor holds the elements' bit patterns (parser.cpp:568-578)
@@ -415,6 +433,76 @@ def indice_convolution_backward_filter_case(features, output_grad, indice_pairs,
         indice_num, sub_m, threshold)
 
 
+def _upstream_case(op_name, inputs, outputs, param_name, param, baseline, thresholds):
+    node = Message()
+    node.add("op_name", op_name)
+    for tid, arr, dtype_name in inputs:
+        node.add("input", tensor_message(tid, arr, dtype_name))
+    for tid, arr, dtype_name in outputs:
+        node.add("output", tensor_message(tid, arr, dtype_name, with_values=baseline))
+    node.add(param_name, param)
+    node.add("test_param", _test_param(thresholds))
+    return node
+
+
+def voxelization_case(points, voxel_size, coors_range, max_points, max_voxels, deterministic=True,
+                      baseline=None):
+    """`baseline` = (voxels, coors, num_points_per_voxel, voxel_num) to store as expected values."""
+    f = points.shape[1]
+    outs = baseline if baseline is not None else (
+        np.zeros((max_voxels, max_points, f), np.float32), np.zeros((max_voxels, 3), np.int32),
+        np.zeros((max_voxels,), np.int32), np.zeros((1,), np.int32))
+    p = Message()
+    p.add("max_points", int(max_points))
+    p.add("max_voxels", int(max_voxels))
+    p.add("ndim", 3)
+    p.add("deterministic", Enum("true" if deterministic else "false"))
+    return _upstream_case(
+        "voxelization",
+        [("points", points, "float32"), ("voxel_size", np.asarray(voxel_size, np.float32), "float32"),
+         ("coors_range", np.asarray(coors_range, np.float32), "float32")],
+        [("voxels", outs[0], "float32"), ("coors", outs[1], "int32"),
+         ("num_points_per_voxel", outs[2], "int32"),
+         ("voxel_num", np.asarray(outs[3], np.int32).reshape(1), "int32")],
+        "voxelization_param", p, baseline is not None, [("DIFF1", 0.0), ("DIFF2", 0.0)])
+
+
+def _reduce_param(reduce_type):
+    p = Message()
+    p.add("reduce_type", Enum({"max": "REDUCE_MODE_MAX", "mean": "REDUCE_MODE_MEAN"}[reduce_type]))
+    return p
+
+
+def dynamic_point_to_voxel_forward_case(feats, coors, reduce_type, baseline=None):
+    """`baseline` = (voxel_feats, voxel_coors, point2voxel_map, voxel_points_count, voxel_num)."""
+    n, c = feats.shape
+    outs = baseline if baseline is not None else (
+        np.zeros((n, c), np.float32), np.zeros((n, 3), np.int32), np.zeros((n,), np.int32),
+        np.zeros((n,), np.int32), np.zeros((1,), np.int32))
+    return _upstream_case(
+        "dynamic_point_to_voxel_forward", [("feats", feats, "float32"), ("coors", coors, "int32")],
+        [("voxel_feats", outs[0], "float32"), ("voxel_coors", outs[1], "int32"),
+         ("point2voxel_map", outs[2], "int32"), ("voxel_points_count", outs[3], "int32"),
+         ("voxel_num", np.asarray(outs[4], np.int32).reshape(1), "int32")],
+        "dynamic_point_to_voxel_forward_param", _reduce_param(reduce_type), baseline is not None,
+        [("DIFF1", 0.0), ("DIFF2", 0.0)])
+
+
+def dynamic_point_to_voxel_backward_case(grad_voxel_feats, feats, voxel_feats, point2voxel_map,
+                                         voxel_points_count, voxel_num, reduce_type="max", baseline=None):
+    """`baseline` = grad_feats to store as the expected values."""
+    out = baseline if baseline is not None else np.zeros(feats.shape, np.float32)
+    return _upstream_case(
+        "dynamic_point_to_voxel_backward",
+        [("grad_voxel_feats", grad_voxel_feats, "float32"), ("feats", feats, "float32"),
+         ("voxel_feats", voxel_feats, "float32"), ("point2voxel_map", point2voxel_map, "int32"),
+         ("voxel_points_count", voxel_points_count, "int32"),
+         ("voxel_num", np.asarray(voxel_num, np.int32).reshape(1), "int32")],
+        [("grad_feats", out, "float32")],
+        "dynamic_point_to_voxel_backward_param", _reduce_param(reduce_type), baseline is not None,
+        [("DIFF1", 0.0), ("DIFF2", 0.0)])
+
+
 # ---------------------------------------------------------------------------
 # replay
 # ---------------------------------------------------------------------------
@@ -435,7 +523,18 @@ def diff2(got, want):
     return float(np.sqrt(num / den)) if den > 0 else float(np.sqrt(num))
 
 
-_ERROR_FUNCS = {"DIFF1": diff1, "DIFF2": diff2}
+def diff3(got, want, dtype_name="float32"):
+    """Largest relative error; the absolute error where |want| is below 1e-4 (half) or 1e-6
+    (float) (evaluator.h: computeDiff3)."""
+    got, want = np.asarray(got, np.float64).reshape(-1), np.asarray(want, np.float64).reshape(-1)
+    if got.size == 0:
+        return 0.0
+    eps = {"float16": 1e-4, "float32": 1e-6}.get(dtype_name, 0.0)
+    num, den = np.abs(got - want), np.abs(want)
+    return float(np.where(den < eps, num, num / (den + 1e-9)).max())
+
+
+_ERROR_FUNCS = {"DIFF1": diff1, "DIFF2": diff2, "DIFF3": diff3}
 
 
 def criteria(node):
@@ -456,6 +555,11 @@ class Replay:
         self.outputs = {}
         self.errors = []
         self.passed = True
+
+
+def _reduce_name(param):
+    return {"REDUCE_MODE_MAX": "max", "REDUCE_MODE_MEAN": "mean", "REDUCE_MODE_SUM": "sum"}[
+        str(param.get("reduce_type", "REDUCE_MODE_MAX"))]
 
 
 def load(path_or_text):
@@ -524,22 +628,57 @@ def replay(path_or_text, handle):
                                                 sub_m, inverse, onchip_float=outs[0].onchip_dtype == DTYPE_FLOAT)
         torch.cuda.synchronize()
         res.outputs = {outs[0].id or "output": host(out)}
+    elif op == "voxelization":
+        p = node.get("voxelization_param")
+        assert p is not None, "voxelization_param missing"
+        assert len(ins) == 3 and len(outs) == 4, "voxelization: 3 inputs and 4 outputs"
+        assert int(p.get("ndim", 3)) == 3, "voxelization: ndim must be 3"
+        got = m.voxelization(handle, dev(ins[0]), dev(ins[1]).reshape(-1), dev(ins[2]).reshape(-1),
+                             int(p.get("max_points")), int(p.get("max_voxels")),
+                             _truthy(p.get("deterministic", 1)))
+        torch.cuda.synchronize()
+        res.outputs = {t.id or name: host(g) for t, name, g in
+                       zip(outs, ("voxels", "coors", "num_points_per_voxel", "voxel_num"), got)}
+    elif op == "dynamic_point_to_voxel_forward":
+        p = node.get("dynamic_point_to_voxel_forward_param")
+        assert p is not None, "dynamic_point_to_voxel_forward_param missing"
+        assert len(ins) == 2 and len(outs) == 5, "dynamic_point_to_voxel_forward: 2 inputs and 5 outputs"
+        got = m.dynamic_point_to_voxel_forward(handle, dev(ins[0]), dev(ins[1]), _reduce_name(p),
+                                               rows=outs[0].shape[0] if outs[0].shape else None)
+        torch.cuda.synchronize()
+        names = ("voxel_feats", "voxel_coors", "point2voxel_map", "voxel_points_count", "voxel_num")
+        arrays = [host(g) for g in got]
+        # rows past voxel_num of the per-voxel outputs are not defined by the operator
+        res.voxel_num = int(arrays[4][0])
+        for a in (arrays[0], arrays[1], arrays[3]):
+            a[res.voxel_num:] = 0
+        res.outputs = {t.id or name: a for t, name, a in zip(outs, names, arrays)}
+    elif op == "dynamic_point_to_voxel_backward":
+        p = node.get("dynamic_point_to_voxel_backward_param")
+        assert p is not None, "dynamic_point_to_voxel_backward_param missing"
+        assert len(ins) == 6 and len(outs) == 1, "dynamic_point_to_voxel_backward: 6 inputs and 1 output"
+        got = m.dynamic_point_to_voxel_backward(handle, *[dev(t) for t in ins], reduce_type=_reduce_name(p))
+        torch.cuda.synchronize()
+        res.outputs = {outs[0].id or "grad_feats": host(got)}
     else:
-        raise ValueError("case file names operator %r: only the sparse-convolution operators are built" % op)
+        raise ValueError("case file names operator %r, which is not built" % op)
 
     funcs, thresholds = criteria(node)
-    for t in outs:
+    for i, t in enumerate(outs):
         if t.values is None:
             continue
-        got = res.outputs[t.id] if t.id in res.outputs else list(res.outputs.values())[0]
+        got = res.outputs[t.id] if t.id in res.outputs else list(res.outputs.values())[i]
         want = t.values
         if op == "get_indice_pairs" and t is outs[0]:
             want = want.copy()
             want[res.num_act_out:] = 0
+        if op == "dynamic_point_to_voxel_forward" and i in (0, 1, 3):
+            want = want.copy()
+            want[res.voxel_num:] = 0
         for f, thr in zip(funcs, thresholds):
             if f not in _ERROR_FUNCS:
                 continue
-            e = _ERROR_FUNCS[f](got, want)
+            e = diff3(got, want, t.dtype_name) if f == "DIFF3" else _ERROR_FUNCS[f](got, want)
             res.errors.append((t.id, f, float(e), thr))
             if not e <= thr:
                 res.passed = False

@@ -70,7 +70,7 @@ def test_value_kinds_decode(tmp_path):
         "shape { dims: 1000 } dtype: DTYPE_FLOAT random_data { seed: 3 upper_bound: 2 lower_bound: -1 distribution: UNIFORM }"))
     assert np.array_equal(rnd.values, again.values)
     with pytest.raises(AssertionError):
-        cf.CaseTensor(cf.parse("shape { dims: 3 } dtype: DTYPE_INT32 value_i: 1"))
+        cf.CaseTensor(cf.parse("shape { dims: 1 } dtype: DTYPE_INT32 value_i: 1 value_i: 2"))
 
 
 def test_value_i_of_float_tensors_holds_bit_patterns():
@@ -228,3 +228,113 @@ def test_reference_backward_data_case_replays(gpu_handle):
     ref = oracle.backward_data(dy.values, w.values.reshape(9, 210, 100), pairs.values, [10] * 9)
     funcs, thresholds = cf.criteria(node)
     assert cf.diff1(got, ref) <= thresholds[0] and cf.diff2(got, ref) <= thresholds[1]
+
+
+# ---- the three operators upstream of the sparse convolutions ---------------------------------
+
+def test_fewer_values_than_elements_are_padded_with_zeros():
+    """The reference's backward case lists 150 values for a [34, 5] tensor (parser.cpp:371-383 takes
+    the count from the list and warns)."""
+    cf = casefile()
+    t = cf.CaseTensor(cf.parse("shape { dims: 2 dims: 3 } dtype: DTYPE_INT32 value_i: 4 value_i: 5 value_i: 6 value_i: 7"))
+    assert t.values.tolist() == [[4, 5, 6], [7, 0, 0]]
+    node, _ = cf.load(os.path.join(GOLDEN, "dynamic_point_to_voxel_backward", "case_1.prototxt"))
+    grad = cf.CaseTensor(node.all("input")[0])
+    assert grad.values.shape == (34, 5) and len(node.all("input")[0].all("value_i")) == 150
+    assert np.all(grad.values[30:] == 0) and np.any(grad.values[29] != 0)
+    with pytest.raises(AssertionError):
+        cf.CaseTensor(cf.parse("shape { dims: 1 } dtype: DTYPE_INT32 value_i: 4 value_i: 5"))
+
+
+def test_diff3_is_the_largest_relative_error():
+    cf = casefile()
+    want = np.array([1.0, -2.0, 0.0, 4.0], np.float32)
+    assert cf.diff3(want, want) == 0.0
+    got = want * np.float32(1.01)
+    assert abs(cf.diff3(got, want) - 0.01) < 1e-6
+    # where the baseline is (nearly) zero the absolute error counts
+    assert abs(cf.diff3(np.array([0.5], np.float32), np.array([0.0], np.float32)) - 0.5) < 1e-12
+    assert abs(cf.diff3(np.array([5e-5], np.float32), np.array([2e-5], np.float32), "float16") - 3e-5) < 1e-9
+    assert cf.diff3(np.array([5e-5], np.float32), np.array([2e-5], np.float32), "float32") > 1.4
+    import sparse_conv_oracle as oracle
+    rng = np.random.default_rng(0)
+    a, b = rng.standard_normal(1000).astype(np.float32), rng.standard_normal(1000).astype(np.float32)
+    assert abs(cf.diff3(a, b) - oracle.diff3(a, b)) <= 1e-9 * oracle.diff3(a, b)
+
+
+def test_written_upstream_cases_read_back_exactly():
+    import dynamic_point_to_voxel_oracle as dpv
+    import voxelization_oracle as vox
+    cf = casefile()
+    rng = np.random.default_rng(5)
+    pts = rng.uniform(-1, 5, (200, 4)).astype(np.float32)
+    vs, cr = [0.5, 0.5, 1.0], [0.0, 0.0, 0.0, 4.0, 4.0, 2.0]
+    want = vox.voxelization(pts, vs, cr, 5, 40)
+    node = cf.parse(cf.dump(cf.voxelization_case(pts, vs, cr, 5, 40, baseline=want)))
+    assert node.get("op_name") == "voxelization"
+    p = node.get("voxelization_param")
+    assert (p.get("max_points"), p.get("max_voxels"), p.get("ndim"), p.get("deterministic")) == (5, 40, 3, "true")
+    ins = [cf.CaseTensor(t).values for t in node.all("input")]
+    assert np.array_equal(ins[0], pts) and ins[1].tolist() == vs and ins[2].tolist() == cr
+    for t, w in zip(node.all("output"), want):
+        assert np.array_equal(cf.CaseTensor(t).values.reshape(-1), np.asarray(w).reshape(-1), equal_nan=True)
+
+    feats = rng.uniform(-100, 100, (50, 3)).astype(np.float32)
+    coors = rng.integers(-1, 4, (50, 3)).astype(np.int32)
+    fwd = dpv.forward("max", feats, coors)
+    node = cf.parse(cf.dump(cf.dynamic_point_to_voxel_forward_case(feats, coors, "max", baseline=fwd[:5])))
+    assert node.get("dynamic_point_to_voxel_forward_param").get("reduce_type") == "REDUCE_MODE_MAX"
+    assert len(node.all("input")) == 2 and len(node.all("output")) == 5
+    assert np.array_equal(cf.CaseTensor(node.all("output")[0]).values, fwd[0])
+    assert cf.CaseTensor(node.all("output")[4]).values.tolist() == [fwd[4]]
+
+    g = rng.standard_normal((50, 3)).astype(np.float32)
+    bwd = dpv.backward(g, feats, fwd[0], fwd[2], fwd[4])
+    node = cf.parse(cf.dump(cf.dynamic_point_to_voxel_backward_case(g, feats, fwd[0], fwd[2], fwd[3], fwd[4],
+                                                                    baseline=bwd)))
+    assert len(node.all("input")) == 6 and node.get("dynamic_point_to_voxel_backward_param") is not None
+    assert np.array_equal(cf.CaseTensor(node.all("output")[0]).values, bwd)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["dynamic_point_to_voxel_forward/case_0.prototxt",
+                                  "dynamic_point_to_voxel_forward/case_1.prototxt",
+                                  "dynamic_point_to_voxel_backward/case_1.prototxt"])
+def test_reference_upstream_cases_replay(gpu_handle, name):
+    """The reference's own case files with their stored baselines, through `replay` as they are.
+    Integer outputs and the backward gradient (copies of input values) must come out exact; the
+    forward features within the file's thresholds and, being sums in point order, within 1e-6."""
+    cf = casefile()
+    res = cf.replay(os.path.join(GOLDEN, name), gpu_handle)
+    assert res.passed, res.errors
+    assert len(res.errors) >= 1      # the backward case names one measure (DIFF3, threshold 0)
+    for tid, func, err, thr in res.errors:
+        assert err <= 1e-6, (tid, func, err)
+
+
+@pytest.mark.gpu
+def test_written_upstream_cases_replay(gpu_handle, tmp_path):
+    import dynamic_point_to_voxel_oracle as dpv
+    import voxelization_oracle as vox
+    cf = casefile()
+    rng = np.random.default_rng(6)
+    pts = rng.uniform(-1, 5, (3000, 4)).astype(np.float32)
+    vs, cr = [0.5, 0.5, 1.0], [0.0, 0.0, 0.0, 4.0, 4.0, 2.0]
+    path = tmp_path / "vox.prototxt"
+    path.write_text(cf.dump(cf.voxelization_case(pts, vs, cr, 5, 40, baseline=vox.voxelization(pts, vs, cr, 5, 40))))
+    res = cf.replay(str(path), gpu_handle)
+    assert res.passed and len(res.errors) == 8 and all(e[2] == 0.0 for e in res.errors), res.errors
+
+    feats = rng.uniform(-100, 100, (2000, 5)).astype(np.float32)
+    coors = rng.integers(-1, 9, (2000, 3)).astype(np.int32)
+    for mode in ("max", "mean"):
+        fwd = dpv.forward(mode, feats, coors.copy())
+        res = cf.replay(cf.dump(cf.dynamic_point_to_voxel_forward_case(feats, coors, mode, baseline=fwd[:5])),
+                        gpu_handle)
+        assert res.passed and len(res.errors) == 10 and all(e[2] == 0.0 for e in res.errors), res.errors
+    fwd = dpv.forward("max", feats, coors.copy())
+    g = rng.standard_normal((2000, 5)).astype(np.float32)
+    bwd = dpv.backward(g, feats, fwd[0], fwd[2], fwd[4])
+    res = cf.replay(cf.dump(cf.dynamic_point_to_voxel_backward_case(g, feats, fwd[0], fwd[2], fwd[3], fwd[4],
+                                                                    baseline=bwd)), gpu_handle)
+    assert res.passed and all(e[2] == 0.0 for e in res.errors), res.errors
