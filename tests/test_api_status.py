@@ -654,3 +654,30 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(m, "LIB_PATH", os.path.join(ROOT, "mlu-ops_amd", "lib", "no_such_library.so"))
     with pytest.raises(RuntimeError, match="there is no fallback path"):
         m.lib()
+
+
+def test_descriptors_from_many_threads():
+    """The descriptor pool is the one shared structure (locked, as core/tensor.cpp:205-241 locks
+    the reference's): eight threads create, set, read back and destroy descriptors at once."""
+    import threading
+    lib = m.lib()
+    errors = []
+
+    def worker(seed):
+        try:
+            for i in range(300):
+                dims = [seed + 1, (i % 7) + 1, 3]
+                d = m.TensorDescriptor(m.LAYOUT_ARRAY, m.DTYPE_FLOAT, dims)
+                n = lib.mluOpGetTensorElementNum(d.ptr)
+                if n != dims[0] * dims[1] * dims[2]:
+                    errors.append((seed, i, n))
+                d.close()
+        except Exception as e:
+            errors.append((seed, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(s,)) for s in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=60)
+    assert not errors, errors[:3]

@@ -102,3 +102,67 @@ def test_two_handles_on_two_streams_do_not_interfere():
                 assert torch.equal(g, w_), "repetition %d" % rep
     for h in handles:
         h.close()
+
+
+def test_four_host_threads_with_a_handle_each():
+    """The reference's convention: one handle per thread and queue, no shared mutable state on
+    the operator path except the descriptor pool (locked).  Four host threads, each with its own
+    stream and handle, run different problems at the same time (ctypes drops the interpreter lock
+    during every call into the library); each result equals the one computed alone."""
+    import threading
+    import torch
+    import mluop_hip as m
+    rng = np.random.default_rng(33)
+    ks = (3, 3, 3)
+    problems = []
+    for t, (L, ci, co, sub_m) in enumerate([(5000, 64, 64, True), (3000, 32, 64, False), (7000, 16, 32, True),
+                                            (2000, 128, 128, False)]):
+        space = (10 + t, 24, 20)
+        idx = torch.from_numpy(random_voxels(rng, 1, space, L)).cuda()
+        feats = torch.from_numpy(rng.standard_normal((idx.shape[0], ci)).astype(np.float32)).cuda().half()
+        w = torch.from_numpy((rng.standard_normal(ks + (ci, co)) * 0.1).astype(np.float32)).cuda().half()
+        stride = [1, 1, 1] if sub_m else [2, 2, 2]
+        ospace = list(space) if sub_m else m.regular_output_space(space, ks, [1, 1, 1], stride, [1, 1, 1])
+        problems.append(dict(idx=idx, feats=feats, w=w, space=space, ospace=ospace, stride=stride, sub_m=sub_m))
+    torch.cuda.synchronize()
+
+    def run(handle, p):
+        pairs, out_idx, num, n_out = m.get_indice_pairs(handle, p["idx"], 1, p["space"], ks, p["ospace"], [1, 1, 1],
+                                                        p["stride"], [1, 1, 1], p["sub_m"])
+        num_host = num.cpu().tolist()
+        out = m.indice_conv_forward(handle, p["feats"], p["w"], m.LAYOUT_ARRAY, pairs, num_host, n_out, p["sub_m"])
+        dx = m.indice_conv_backward_data(handle, out, p["w"], m.LAYOUT_ARRAY, pairs, num_host, p["sub_m"],
+                                         p["feats"].shape[1])
+        return [t.cpu() for t in (pairs, num, out_idx[:n_out], out, dx)]
+
+    main = m.make_handle_on_current_stream()
+    alone = [run(main, p) for p in problems]
+    main.close()
+
+    results, errors = [None] * len(problems), []
+    start = threading.Barrier(len(problems))
+
+    def worker(i):
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                handle = m.make_handle_on_current_stream()
+                start.wait(timeout=60)
+                for _ in range(5):
+                    results[i] = run(handle, problems[i])
+                stream.synchronize()
+                handle.close()
+        except Exception as e:          # reported by the main thread
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(problems))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    assert all(not t.is_alive() for t in threads)
+    for i, (got, want) in enumerate(zip(results, alone)):
+        for g, w_ in zip(got, want):
+            assert torch.equal(g, w_), "thread %d" % i
