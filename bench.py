@@ -499,6 +499,18 @@ def main():
     _, per_p = time_ops(torch, [("forward", step.forward)], max(args.steps // 2, 5))
     handle.promise_distinct_pairs(False)
     result["forward_ms_distinct_pairs_promised"] = median(per_p["forward"])
+    # Nor is this: the forward operator handed the row map of its rulebook, built once ahead
+    # (mluOpExtBuildRowMap), as layers that share a rulebook can; it then launches neither the
+    # map kernels nor that check.
+    row_map = m.RowMap(handle, step.pairs, list(step.counts), step.L, step.L, 1)
+
+    def forward_with_map():
+        row_map.announce()
+        step.forward()
+
+    _, per_m = time_ops(torch, [("forward", forward_with_map)], max(args.steps // 2, 5))
+    result["forward_ms_row_map_kept"] = median(per_m["forward"]) if row_map.usable else None
+    row_map.close()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(step)
     print(json.dumps(result))

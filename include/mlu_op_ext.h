@@ -54,6 +54,41 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtSetSparseConvExtendedModes(mluOpHandle_t han
  * all but one of such pairs.  Off by default. */
 mluOpStatus_t MLUOP_WIN_API mluOpExtSetDistinctPairsPromise(mluOpHandle_t handle, int promised);
 
+/* Row maps kept across calls.  mluOpIndiceConvolutionForward and ...BackwardData turn the pair
+ * lists into a [K, rows] map (partner row of every result row at every offset, or -1) on every
+ * call: the reference API (mlu_op.h:10321-10448, :9625-9773) hands them nothing else to keep.
+ * Layers that share a rulebook, and the forward and backward pass of each, can build the map
+ * once.  No counterpart in the reference.
+ *
+ *   mluOpExtGetRowMapSize  bytes of a map buffer for `rows` result rows.
+ *   mluOpExtBuildRowMap    fills `row_map` (device memory of that size, owned by the caller) on
+ *                          the handle's queue and waits for the queue once.  `row_column` is the
+ *                          pair column that names the result rows: 1 for a forward convolution
+ *                          (and an inverse layer's backward data), 0 for backward data (and an
+ *                          inverse layer's forward); `rows` / `source_rows` are the row counts
+ *                          of the result and of the gathered tensor, the one that column 0
+ *                          indexes being indice_pairs.dim[2].  `*lost_pairs` returns how many
+ *                          pairs found no slot of their own (several pairs of one offset naming
+ *                          one result row, or rows outside their tensors): such a map is not
+ *                          recorded and cannot be used; call the operators without it.
+ *   mluOpExtUseRowMap      announces a recorded map for the next mluOpIndiceConvolutionForward
+ *                          or ...BackwardData call on this handle, which must be given the same
+ *                          indice_pairs pointer, shapes and direction the map was built for
+ *                          (BAD_PARAM otherwise) and then launches neither the map kernels nor
+ *                          the check for colliding pairs.  The announcement ends with that call,
+ *                          whatever it returns.  The pair tensor must not have changed since the
+ *                          map was built.  NULL withdraws an announcement.
+ *   mluOpExtForgetRowMap   drops the record of a buffer about to be freed (NULL: all records). */
+mluOpStatus_t MLUOP_WIN_API mluOpExtGetRowMapSize(const mluOpTensorDescriptor_t indice_pairs_desc,
+                                                  int64_t rows, size_t *size);
+mluOpStatus_t MLUOP_WIN_API mluOpExtBuildRowMap(mluOpHandle_t handle,
+                                                const mluOpTensorDescriptor_t indice_pairs_desc,
+                                                const void *indice_pairs, const int64_t indice_num[],
+                                                int64_t rows, int64_t source_rows, int row_column,
+                                                void *row_map, size_t size, int64_t *lost_pairs);
+mluOpStatus_t MLUOP_WIN_API mluOpExtUseRowMap(mluOpHandle_t handle, const void *row_map);
+mluOpStatus_t MLUOP_WIN_API mluOpExtForgetRowMap(mluOpHandle_t handle, const void *row_map);
+
 #if defined(__cplusplus)
 }
 #endif

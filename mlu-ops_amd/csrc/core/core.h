@@ -41,6 +41,15 @@ struct mluOpContext {
   // (mluOpExtSetDistinctPairsPromise): forward and backward data then skip the
   // check that finds and adds such pairs.
   bool distinct_pairs_promised = false;
+  // Row maps built by mluOpExtBuildRowMap with no pair lost, and the one announced for the
+  // next forward / backward-data call (mluOpExtUseRowMap).
+  struct RowMapRecord {
+    const void *map;
+    const void *pairs;
+    int K, L, rows, source_rows, row_column;
+  };
+  std::vector<RowMapRecord> row_maps;
+  const void *pending_row_map = nullptr;
 
   // What the kernel launchers need: the stream, and the timer while it is on.
   mluop::LaunchCtx launchCtx() { return mluop::LaunchCtx(queue, timer.enabled ? &timer : nullptr); }

@@ -42,6 +42,10 @@ struct ConvProblem {
   bool inverse = false;
   // The caller promised that no offset names a result row twice: no check for lost pairs.
   bool distinct_pairs = false;
+  // Forward and backward data: the [K, rows] row map of exactly this rulebook and direction,
+  // built ahead by buildRowMap with no pair lost (so the pairs are distinct as well); the
+  // launch then neither clears nor fills a map of its own.
+  const int32_t *row_map = nullptr;
   // Backward filter only: element strides of dW(k, ci, co) in filters_grad;
   // all zero = the positional [K, Ci, Co].
   int64_t grad_stride_k = 0, grad_stride_ci = 0, grad_stride_co = 0;
@@ -56,6 +60,22 @@ size_t gatherConvWorkspaceBytes(const ConvProblem &p, GatherDirection dir);
 hipError_t launchGatherConv(const LaunchCtx &lc, const ConvProblem &p, GatherDirection dir,
                             const void *gathered, const FilterView &filters, void *workspace,
                             void *result);
+
+// A row map kept across calls: entry [k, r] is the partner row of result row r at offset k,
+// or -1.  `row_column` is the pair column that names the result rows (1: the rows are what
+// column 1 indexes, as in a forward convolution; 0: what column 0 indexes, as in backward
+// data), `rows` / `source_rows` the row counts of the result and of the gathered tensor.
+struct RowMapShape {
+  int K, L, rows, source_rows, row_column;
+};
+// The shape a launch of `dir` over `p` needs.
+RowMapShape rowMapShape(const ConvProblem &p, GatherDirection dir);
+// Bytes of a map buffer: the entries, one counter, the per-offset counts.
+size_t rowMapBytes(int K, int rows);
+// Clears and fills `row_map` on the stream and copies the number of filled slots to
+// `*filled_host` (pinned memory); the caller waits for the stream before reading it.
+hipError_t buildRowMap(const LaunchCtx &lc, const int32_t *indice_pairs, const int64_t *indice_num,
+                       const RowMapShape &shape, void *row_map, int32_t *filled_host);
 
 size_t backwardFilterWorkspaceBytes(const ConvProblem &p);
 hipError_t launchBackwardFilter(const LaunchCtx &lc, const ConvProblem &p, const void *features,

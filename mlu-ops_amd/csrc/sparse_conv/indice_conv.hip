@@ -938,6 +938,20 @@ __global__ __launch_bounds__(256) void repairLostPairs(
   }
 }
 
+// Number of map slots that hold a partner, added to *total (cleared beforehand).
+__global__ __launch_bounds__(256) void countFilledSlots(const int32_t *map, size_t n, int32_t *total) {
+  __shared__ int s_sum;
+  if (threadIdx.x == 0) s_sum = 0;
+  __syncthreads();
+  int mine = 0;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+    mine += map[i] >= 0 ? 1 : 0;
+  mine = waveInclusiveScan(mine);
+  if ((threadIdx.x & 63) == 63) atomicAdd(&s_sum, mine);
+  __syncthreads();
+  if (threadIdx.x == 0 && s_sum != 0) atomicAdd(total, s_sum);
+}
+
 // ---- backward filter -------------------------------------------------------------
 // Where dW(k, ci, co) goes in filters_grad (element strides).
 struct GradLayout {
@@ -1554,18 +1568,20 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
   const int64_t sQ = d.filter_forward ? f.stride_ci : f.stride_co;
   const int64_t sC = d.filter_forward ? f.stride_co : f.stride_ci;
   const size_t map_elems = (size_t)p.K * d.R;
+  const bool own_map = p.row_map == nullptr;  // else: built ahead, nothing to clear or fill
+  const int32_t *entries = own_map ? ws.map : p.row_map;
   int n_filled = 0;  // workgroups along x of the gather kernel = slot counts it leaves
   if (use_mfma) {
     const size_t frags = (size_t)p.K * (d.C / 16) * ((d.Q + E::kChunk - 1) / E::kChunk) * 64;
-    const int fill_blocks = gridFor(map_elems / 4 + 1, 2048);
+    const int fill_blocks = own_map ? gridFor(map_elems / 4 + 1, 2048) : 0;
     const int pack_blocks = gridFor(frags, 512);
     lc.begin("fillMapPackFilter");
     fillMapPackFilter<E><<<fill_blocks + pack_blocks, 256, 0, lc.stream>>>(
         ws.map, map_elems, fill_blocks, static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K,
         d.Q, d.C, static_cast<S *>(ws.packed));
     lc.end();
-    launchScatterRowMap(lc, p, d, ws, inl, max_count);
-    const RowMap map = {ws.map, ws.filled};
+    if (own_map) launchScatterRowMap(lc, p, d, ws, inl, max_count);
+    const RowMap map = {entries, ws.filled};
     if (useDenseKernel(p, d)) {
       n_filled = denseGridX(d.R);
       launchDense<E>(lc, d.Q, d.C, gathered, ws.packed, map, d.R, p.K, result);
@@ -1575,20 +1591,22 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
       launchMfma<E>(lc, d.Q, d.C, tile_cols, gathered, ws.packed, map, d.R, p.K, result);
     }
   } else {
-    lc.begin("fillInt32");
-    fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems, -1);
-    lc.end();
-    launchScatterRowMap(lc, p, d, ws, inl, max_count);
+    if (own_map) {
+      lc.begin("fillInt32");
+      fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems, -1);
+      lc.end();
+      launchScatterRowMap(lc, p, d, ws, inl, max_count);
+    }
     dim3 grid((d.R + 31) / 32, (d.C + 63) / 64);
     n_filled = (int)grid.x;
     lc.begin("gatherConvSimt");
     gatherConvSimt<E><<<grid, 256, 0, lc.stream>>>(static_cast<const S *>(gathered), d.Q,
                                                 static_cast<const S *>(f.base), f.stride_k, sQ, sC,
-                                                ws.map, d.R, p.K, inl, ws.dev_counts, d.C,
+                                                entries, d.R, p.K, inl, ws.dev_counts, d.C,
                                                 ws.filled, static_cast<S *>(result));
     lc.end();
   }
-  if (p.distinct_pairs) return;
+  if (p.distinct_pairs || !own_map) return;  // a map built ahead was checked when it was built
   // one workgroup that returns at once unless pairs of one offset share a result row
   long long expected = 0;
   for (int k = 0; k < p.K; ++k) {
@@ -1781,6 +1799,52 @@ hipError_t launchGatherConv(const LaunchCtx &lc, const ConvProblem &p, GatherDir
       break;
   }
   return hipGetLastError();
+}
+
+RowMapShape rowMapShape(const ConvProblem &p, GatherDirection dir) {
+  const GatherDims d = gatherDims(p, dir);
+  return RowMapShape{p.K, p.L, d.R, d.n_src, d.row_col};
+}
+
+// entries [K, rows] | filled-slot counter | per-offset counts [K] (for K beyond the inline limit)
+size_t rowMapBytes(int K, int rows) {
+  return alignUp((size_t)K * rows * 4) + alignUp(4) + alignUp((size_t)K * 4) + kBaseAlign;
+}
+
+hipError_t buildRowMap(const LaunchCtx &lc, const int32_t *indice_pairs, const int64_t *indice_num,
+                       const RowMapShape &shape, void *row_map, int32_t *filled_host) {
+  const size_t map_elems = (size_t)shape.K * shape.rows;
+  int32_t *map = static_cast<int32_t *>(row_map);
+  int32_t *counter = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(map) + alignUp(map_elems * 4));
+  int32_t *dev_counts = reinterpret_cast<int32_t *>(reinterpret_cast<char *>(counter) + alignUp(4));
+  ConvProblem p;
+  p.K = shape.K;
+  p.L = shape.L;
+  p.indice_pairs = indice_pairs;
+  p.indice_num = indice_num;
+  OffsetCounts inl;
+  int max_count = 0;
+  hipError_t err = prepareCounts(lc, p, &inl, shape.K > kMaxInlineK ? dev_counts : nullptr, &max_count);
+  if (err != hipSuccess) return err;
+  lc.begin("fillInt32");
+  fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(map, map_elems, -1);
+  lc.end();
+  fillInt32<<<1, 256, 0, lc.stream>>>(counter, 1, 0);
+  if (max_count > 0) {
+    dim3 grid((max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256, shape.K);
+    lc.begin("scatterRowMap");
+    scatterRowMap<<<grid, 256, 0, lc.stream>>>(indice_pairs, shape.L, inl,
+                                            shape.K > kMaxInlineK ? dev_counts : nullptr,
+                                            shape.row_column, 1 - shape.row_column, shape.rows,
+                                            shape.source_rows, map);
+    lc.end();
+  }
+  lc.begin("countFilledSlots");
+  countFilledSlots<<<gridFor(map_elems, 1024), 256, 0, lc.stream>>>(map, map_elems, counter);
+  lc.end();
+  err = hipGetLastError();
+  if (err != hipSuccess) return err;
+  return hipMemcpyAsync(filled_host, counter, 4, hipMemcpyDeviceToHost, lc.stream);
 }
 
 size_t backwardFilterWorkspaceBytes(const ConvProblem &p) {

@@ -7,6 +7,7 @@
 
 #include "core/core.h"
 #include "sparse_conv/indice_conv.h"
+#include "sparse_conv/row_map.h"
 
 namespace {
 
@@ -278,6 +279,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardData(
     const size_t workspace_size, const mluOpTensorDescriptor_t input_grad_desc,
     void *input_grad) {
   const std::string api = "[mluOpIndiceConvolutionBackwardData]";
+  const void *announced_map = mluop::sparse_conv::announcedRowMap(handle);
   bool is_zero = false;
   mluOpStatus_t st = foolCheckNoPtr(handle, output_grad_desc, filters_desc, indice_pairs_desc,
                                     indice_num, inverse, sub_m, input_grad_desc, &is_zero);
@@ -295,6 +297,8 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardData(
   ConvProblem p = makeProblem(output_grad_desc, filters_desc, indice_pairs_desc, input_grad_desc,
                               indice_num, inverse, indice_pairs);
   p.distinct_pairs = handle->distinct_pairs_promised;
+  st = mluop::sparse_conv::takeRowMap(api, handle, announced_map, GatherDirection::kBackwardData, &p);
+  if (st != MLUOP_STATUS_SUCCESS) return st;
   const size_t need =
       mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kBackwardData);
   if (workspace_size < need || workspace == NULL) {

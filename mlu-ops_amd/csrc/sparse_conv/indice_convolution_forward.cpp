@@ -6,6 +6,7 @@
 
 #include "core/core.h"
 #include "sparse_conv/indice_conv.h"
+#include "sparse_conv/row_map.h"
 
 namespace {
 
@@ -221,6 +222,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionForward(
     const int64_t sub_m, void *workspace, size_t workspace_size,
     const mluOpTensorDescriptor_t features_out_desc, void *features_out) {
   const std::string api = "[mluOpIndiceConvolutionForward]";
+  const void *announced_map = mluop::sparse_conv::announcedRowMap(handle);
   mluOpStatus_t st = foolProof(api, handle, features_desc, filters_desc, indice_pairs_desc,
                                indice_num, num_act_out, inverse, sub_m, features_out_desc);
   if (st != MLUOP_STATUS_SUCCESS) return st;
@@ -238,6 +240,8 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionForward(
   ConvProblem p = makeProblem(features_desc, filters_desc, indice_pairs_desc, indice_num,
                               num_act_out, inverse, indice_pairs);
   p.distinct_pairs = handle->distinct_pairs_promised;
+  st = mluop::sparse_conv::takeRowMap(api, handle, announced_map, GatherDirection::kForward, &p);
+  if (st != MLUOP_STATUS_SUCCESS) return st;
   const size_t need = mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kForward);
   if (workspace_size < need || workspace == nullptr) {
     MLUOP_LOG(ERROR) << api << " workspace of " << workspace_size

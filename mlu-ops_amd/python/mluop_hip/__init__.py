@@ -122,6 +122,12 @@ SIGNATURES = {
     "mluOpExtSetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int]),
     "mluOpExtSetSparseConvExtendedModes": (ctypes.c_int, [_vp, ctypes.c_int]),
     "mluOpExtSetDistinctPairsPromise": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "mluOpExtGetRowMapSize": (ctypes.c_int, [_vp, ctypes.c_int64, ctypes.POINTER(ctypes.c_size_t)]),
+    "mluOpExtBuildRowMap": (ctypes.c_int, [_vp, _vp, _vp, ctypes.POINTER(ctypes.c_int64), ctypes.c_int64,
+                                           ctypes.c_int64, ctypes.c_int, _vp, ctypes.c_size_t,
+                                           ctypes.POINTER(ctypes.c_int64)]),
+    "mluOpExtUseRowMap": (ctypes.c_int, [_vp, _vp]),
+    "mluOpExtForgetRowMap": (ctypes.c_int, [_vp, _vp]),
     "mluOpExtGetKernelTimingCount": (ctypes.c_int, [_vp, _ip]),
     "mluOpExtGetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int, ctypes.POINTER(ctypes.c_char_p),
                                                ctypes.POINTER(ctypes.c_float)]),
@@ -341,9 +347,48 @@ def _host_counts(indice_num):
     return (ctypes.c_int64 * max(len(vals), 1))(*vals)
 
 
+class RowMap:
+    """A [K, rows] row map built once for a rulebook and one direction (mluOpExtBuildRowMap):
+    `buffer` is the device memory, `lost_pairs` how many pairs found no slot of their own (a map
+    with lost pairs is not recorded by the library and `usable` is False)."""
+
+    def __init__(self, handle, indice_pairs, indice_num_host, rows, source_rows, row_column):
+        torch = _torch()
+        K, _, L = indice_pairs.shape
+        d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+        size = ctypes.c_size_t(0)
+        check(lib().mluOpExtGetRowMapSize(d_pairs.ptr, int(rows), ctypes.byref(size)), "mluOpExtGetRowMapSize")
+        self.handle = handle
+        self.pairs = indice_pairs          # the map is valid for this tensor only: keep it alive
+        self.buffer = torch.empty((size.value,), dtype=torch.uint8, device=indice_pairs.device)
+        lost = ctypes.c_int64(-1)
+        check(lib().mluOpExtBuildRowMap(handle.ptr, d_pairs.ptr, indice_pairs.data_ptr(),
+                                        _host_counts(indice_num_host), int(rows), int(source_rows),
+                                        int(row_column), self.buffer.data_ptr(), size.value, ctypes.byref(lost)),
+              "mluOpExtBuildRowMap")
+        self.lost_pairs = int(lost.value)
+        self.usable = self.lost_pairs == 0
+
+    def announce(self):
+        """The next forward / backward-data call on the handle uses this map."""
+        check(lib().mluOpExtUseRowMap(self.handle.ptr, self.buffer.data_ptr()), "mluOpExtUseRowMap")
+
+    def close(self):
+        if self.buffer is not None and self.handle.ptr:
+            lib().mluOpExtForgetRowMap(self.handle.ptr, self.buffer.data_ptr())
+        self.buffer = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def indice_conv_forward(handle, features, filters, filters_layout, indice_pairs, indice_num_host,
-                        num_act_out, sub_m, inverse=0):
-    """features [L,Ci], filters 5-D in `filters_layout`, indice_num_host: K python ints."""
+                        num_act_out, sub_m, inverse=0, row_map=None):
+    """features [L,Ci], filters 5-D in `filters_layout`, indice_num_host: K python ints.
+    `row_map`: a usable RowMap built for this pair tensor and direction."""
     torch = _torch()
     code = torch_dtype_code(features.dtype)
     K, _, L = indice_pairs.shape
@@ -362,6 +407,8 @@ def indice_conv_forward(handle, features, filters, filters_layout, indice_pairs,
         handle.ptr, d_feat.ptr, d_filt.ptr, d_pairs.ptr, d_out.ptr, counts, num_act_out, inverse,
         int(sub_m), ctypes.byref(size)), "mluOpGetIndiceConvolutionForwardWorkspaceSize")
     ws = _workspace(size.value, features.device)
+    if row_map is not None:
+        row_map.announce()
     check(lib().mluOpIndiceConvolutionForward(
         handle.ptr, d_feat.ptr, features.data_ptr(), d_filt.ptr, filters.data_ptr(), d_pairs.ptr,
         indice_pairs.data_ptr(), counts, num_act_out, inverse, int(sub_m), ws.data_ptr(),
@@ -370,7 +417,7 @@ def indice_conv_forward(handle, features, filters, filters_layout, indice_pairs,
 
 
 def indice_conv_backward_data(handle, output_grad, filters, filters_layout, indice_pairs,
-                              indice_num_host, sub_m, ci, inverse=0, rows=None):
+                              indice_num_host, sub_m, ci, inverse=0, rows=None, row_map=None):
     """input_grad [rows, ci]; rows = indice_pairs.shape[2] unless the convolution is an inverse one."""
     torch = _torch()
     code = torch_dtype_code(output_grad.dtype)
@@ -387,6 +434,8 @@ def indice_conv_backward_data(handle, output_grad, filters, filters_layout, indi
         handle.ptr, d_dy.ptr, d_filt.ptr, d_pairs.ptr, d_dx.ptr, counts, inverse,
         ctypes.byref(size)), "mluOpGetIndiceConvolutionBackwardDataWorkspaceSize")
     ws = _workspace(size.value, output_grad.device)
+    if row_map is not None:
+        row_map.announce()
     check(lib().mluOpIndiceConvolutionBackwardData(
         handle.ptr, d_dy.ptr, output_grad.data_ptr(), d_filt.ptr, filters.data_ptr(), d_pairs.ptr,
         indice_pairs.data_ptr(), counts, inverse, int(sub_m), ws.data_ptr(), size.value, d_dx.ptr,

@@ -681,3 +681,59 @@ def test_descriptors_from_many_threads():
     for t in threads:
         t.join(timeout=60)
     assert not errors, errors[:3]
+
+
+def test_row_map_entry_points(handle):
+    """Checks of mluOpExtGetRowMapSize / BuildRowMap / UseRowMap / ForgetRowMap; with every check
+    passed a handle without a device stops where the build would launch."""
+    lib = m.lib()
+    bad, failed = STATUS["MLUOP_STATUS_BAD_PARAM"], STATUS["MLUOP_STATUS_EXECUTION_FAILED"]
+    K, L, n_out = 27, 100, 40
+    def desc(dtype, dims):
+        return make_desc({"layout": "MLUOP_LAYOUT_ARRAY", "dtype": dtype, "dim_nb": len(dims), "dims": dims})
+
+    pairs = desc("MLUOP_DTYPE_INT32", [K, 2, L])
+    floats = desc("MLUOP_DTYPE_FLOAT", [K, 2, L])
+    flat = desc("MLUOP_DTYPE_INT32", [K, L])
+    try:
+        size = ctypes.c_size_t(0)
+        assert lib.mluOpExtGetRowMapSize(pairs, n_out, ctypes.byref(size)) == 0
+        assert size.value >= K * n_out * 4
+        assert lib.mluOpExtGetRowMapSize(None, n_out, ctypes.byref(size)) == bad
+        assert lib.mluOpExtGetRowMapSize(pairs, n_out, None) == bad
+        assert lib.mluOpExtGetRowMapSize(pairs, -1, ctypes.byref(size)) == bad
+        assert lib.mluOpExtGetRowMapSize(flat, n_out, ctypes.byref(size)) == bad
+        small = size.value
+        assert lib.mluOpExtGetRowMapSize(pairs, L, ctypes.byref(size)) == 0 and size.value > small
+        num, lost = i64([3] * K), ctypes.c_int64(0)
+
+        def build(desc=pairs, data=FAKE, counts=num, rows=n_out, source=L, column=1, out=FAKE, nbytes=None,
+                  lost_ref=ctypes.byref(lost), h=handle.ptr):
+            return lib.mluOpExtBuildRowMap(h, desc, data, counts, rows, source, column, out,
+                                           size.value if nbytes is None else nbytes, lost_ref)
+
+        assert build() == failed                       # all checks passed
+        assert build(rows=L, source=n_out, column=0) == failed
+        assert build(h=None) == bad
+        assert build(desc=None) == bad
+        assert build(desc=floats) == bad
+        assert build(data=None) == bad
+        assert build(counts=None) == bad
+        assert build(out=None) == bad
+        assert build(lost_ref=None) == bad
+        assert build(column=2) == bad
+        assert build(rows=0) == bad
+        assert build(source=L + 1) == bad              # column 0 indexes indice_pairs.dim[2] rows
+        assert build(rows=L + 1, source=n_out, column=0) == bad
+        assert build(nbytes=small - 1) == bad
+        assert build(counts=i64([L + 1] + [0] * (K - 1))) == bad
+        assert build(counts=i64([-1] + [0] * (K - 1))) == bad
+
+        assert lib.mluOpExtUseRowMap(None, FAKE) == bad
+        assert lib.mluOpExtUseRowMap(handle.ptr, FAKE) == bad      # nothing was built into it
+        assert lib.mluOpExtUseRowMap(handle.ptr, None) == 0        # withdraws an announcement
+        assert lib.mluOpExtForgetRowMap(handle.ptr, FAKE) == 0
+        assert lib.mluOpExtForgetRowMap(handle.ptr, None) == 0
+        assert lib.mluOpExtForgetRowMap(None, None) == bad
+    finally:
+        free_descs(pairs, floats, flat)
