@@ -286,6 +286,8 @@ def run_backbone(args, torch, m):
         layers += [spnn.SubMConv3d(co, co, 3, indice_key="s%d" % stage) for _ in range(2)]
         c = co
     net = torch.nn.ModuleList(layers).cuda().half()
+    # MLUOP_BENCH_SHARE_ROW_MAPS=1: layers of a stage share their rulebook's row maps
+    spnn.share_row_maps(os.environ.get("MLUOP_BENCH_SHARE_ROW_MAPS", "0") == "1")
 
     def step():
         # the voxels are distinct, as a voxelizer's output is: the layers skip the collision check

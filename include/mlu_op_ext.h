@@ -71,6 +71,9 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtSetDistinctPairsPromise(mluOpHandle_t handle
  *                          pairs found no slot of their own (several pairs of one offset naming
  *                          one result row, or rows outside their tensors): such a map is not
  *                          recorded and cannot be used; call the operators without it.
+ *                          With mluOpExtSetDistinctPairsPromise in force `lost_pairs` may be
+ *                          NULL: the build then neither counts nor waits, and the promise
+ *                          stands in for the verdict.
  *   mluOpExtUseRowMap      announces a recorded map for the next mluOpIndiceConvolutionForward
  *                          or ...BackwardData call on this handle, which must be given the same
  *                          indice_pairs pointer, shapes and direction the map was built for

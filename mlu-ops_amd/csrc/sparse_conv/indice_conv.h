@@ -72,8 +72,9 @@ struct RowMapShape {
 RowMapShape rowMapShape(const ConvProblem &p, GatherDirection dir);
 // Bytes of a map buffer: the entries, one counter, the per-offset counts.
 size_t rowMapBytes(int K, int rows);
-// Clears and fills `row_map` on the stream and copies the number of filled slots to
-// `*filled_host` (pinned memory); the caller waits for the stream before reading it.
+// Clears and fills `row_map` on the stream and, unless `filled_host` is null, counts the filled
+// slots and copies the count to `*filled_host` (pinned memory); the caller waits for the stream
+// before reading it.
 hipError_t buildRowMap(const LaunchCtx &lc, const int32_t *indice_pairs, const int64_t *indice_num,
                        const RowMapShape &shape, void *row_map, int32_t *filled_host);
 

@@ -1839,6 +1839,7 @@ hipError_t buildRowMap(const LaunchCtx &lc, const int32_t *indice_pairs, const i
                                             shape.source_rows, map);
     lc.end();
   }
+  if (filled_host == nullptr) return hipGetLastError();
   lc.begin("countFilledSlots");
   countFilledSlots<<<gridFor(map_elems, 1024), 256, 0, lc.stream>>>(map, map_elems, counter);
   lc.end();

@@ -61,7 +61,9 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtBuildRowMap(mluOpHandle_t handle,
   PARAM_CHECK(api, handle != NULL);
   PARAM_CHECK(api, indice_pairs_desc != NULL);
   PARAM_CHECK(api, indice_num != NULL);
-  PARAM_CHECK(api, lost_pairs != NULL);
+  // without a place for the verdict the build neither counts nor waits: the caller's promise
+  // of distinct pairs (mluOpExtSetDistinctPairsPromise) has to stand in for it
+  PARAM_CHECK(api, lost_pairs != NULL || handle->distinct_pairs_promised);
   PARAM_CHECK(api, indice_pairs_desc->dim == 3);
   PARAM_CHECK(api, indice_pairs_desc->dims[1] == 2);
   PARAM_CHECK(api, indice_pairs_desc->dtype == MLUOP_DTYPE_INT32);
@@ -92,13 +94,14 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtBuildRowMap(mluOpHandle_t handle,
     else ++i;
   }
   const RowMapShape shape{(int)K, (int)L, (int)rows, (int)source_rows, row_column};
-  HIP_CHECK_RETURN(api, mluop::sparse_conv::buildRowMap(handle->launchCtx(),
-                                                       static_cast<const int32_t *>(indice_pairs),
-                                                       indice_num, shape, row_map,
-                                                       handle->pinned_scalar));
-  HIP_CHECK_RETURN(api, hipStreamSynchronize(handle->queue));
-  *lost_pairs = expected - (int64_t)handle->pinned_scalar[0];
-  if (*lost_pairs == 0) {
+  HIP_CHECK_RETURN(api, mluop::sparse_conv::buildRowMap(
+                            handle->launchCtx(), static_cast<const int32_t *>(indice_pairs), indice_num,
+                            shape, row_map, lost_pairs != NULL ? handle->pinned_scalar : nullptr));
+  if (lost_pairs != NULL) {
+    HIP_CHECK_RETURN(api, hipStreamSynchronize(handle->queue));
+    *lost_pairs = expected - (int64_t)handle->pinned_scalar[0];
+  }
+  if (lost_pairs == NULL || *lost_pairs == 0) {
     if (maps.size() >= 256) maps.erase(maps.begin());
     maps.push_back({row_map, indice_pairs, (int)K, (int)L, (int)rows, (int)source_rows, row_column});
   }

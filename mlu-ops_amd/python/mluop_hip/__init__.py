@@ -352,7 +352,9 @@ class RowMap:
     `buffer` is the device memory, `lost_pairs` how many pairs found no slot of their own (a map
     with lost pairs is not recorded by the library and `usable` is False)."""
 
-    def __init__(self, handle, indice_pairs, indice_num_host, rows, source_rows, row_column):
+    def __init__(self, handle, indice_pairs, indice_num_host, rows, source_rows, row_column, verify=True):
+        """verify=False (needs the handle's distinct-pairs promise) skips the count of lost pairs and
+        the wait for the queue that reads it."""
         torch = _torch()
         K, _, L = indice_pairs.shape
         d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
@@ -361,13 +363,14 @@ class RowMap:
         self.handle = handle
         self.pairs = indice_pairs          # the map is valid for this tensor only: keep it alive
         self.buffer = torch.empty((size.value,), dtype=torch.uint8, device=indice_pairs.device)
-        lost = ctypes.c_int64(-1)
+        lost = ctypes.c_int64(0)
         check(lib().mluOpExtBuildRowMap(handle.ptr, d_pairs.ptr, indice_pairs.data_ptr(),
                                         _host_counts(indice_num_host), int(rows), int(source_rows),
-                                        int(row_column), self.buffer.data_ptr(), size.value, ctypes.byref(lost)),
+                                        int(row_column), self.buffer.data_ptr(), size.value,
+                                        ctypes.byref(lost) if verify else None),
               "mluOpExtBuildRowMap")
-        self.lost_pairs = int(lost.value)
-        self.usable = self.lost_pairs == 0
+        self.lost_pairs = int(lost.value) if verify else None
+        self.usable = not verify or self.lost_pairs == 0
 
     def announce(self):
         """The next forward / backward-data call on the handle uses this map."""

@@ -720,7 +720,12 @@ def test_row_map_entry_points(handle):
         assert build(data=None) == bad
         assert build(counts=None) == bad
         assert build(out=None) == bad
-        assert build(lost_ref=None) == bad
+        assert build(lost_ref=None) == bad             # no place for the verdict and no promise
+        handle.promise_distinct_pairs(True)
+        try:
+            assert build(lost_ref=None) == failed      # the promise stands in for it
+        finally:
+            handle.promise_distinct_pairs(False)
         assert build(column=2) == bad
         assert build(rows=0) == bad
         assert build(source=L + 1) == bad              # column 0 indexes indice_pairs.dim[2] rows

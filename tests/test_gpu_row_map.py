@@ -87,6 +87,30 @@ def test_map_kernels_and_collision_check_are_not_launched(gpu_handle):
     rm.close()
 
 
+def test_unverified_build_needs_the_promise(gpu_handle):
+    import torch
+    import mluop_hip as m
+    rng = np.random.default_rng(56)
+    idx = random_voxels(rng, 1, (10, 12, 12), 900)
+    pairs, num, n_out = rulebook(m, gpu_handle, idx, 1, (10, 12, 12), (3, 3, 3), (1, 1, 1), True)
+    feats = torch.randn(idx.shape[0], 64, device="cuda").half()
+    w = (torch.randn(3, 3, 3, 64, 64, device="cuda") * 0.1).half()
+    with pytest.raises(m.MluOpError) as e:
+        m.RowMap(gpu_handle, pairs, num, n_out, idx.shape[0], 1, verify=False)
+    assert e.value.status == m.STATUS_BAD_PARAM
+    plain = m.indice_conv_forward(gpu_handle, feats, w, m.LAYOUT_ARRAY, pairs, num, n_out, True)
+    gpu_handle.promise_distinct_pairs(True)
+    try:
+        rm = m.RowMap(gpu_handle, pairs, num, n_out, idx.shape[0], 1, verify=False)
+        assert rm.usable and rm.lost_pairs is None
+        out = m.indice_conv_forward(gpu_handle, feats, w, m.LAYOUT_ARRAY, pairs, num, n_out, True, row_map=rm)
+    finally:
+        gpu_handle.promise_distinct_pairs(False)
+    torch.cuda.synchronize()
+    assert torch.equal(out, plain)
+    rm.close()
+
+
 def test_inverse_layer_with_maps(gpu_handle):
     import torch
     import mluop_hip as m
