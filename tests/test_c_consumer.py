@@ -80,6 +80,10 @@ int main(void) {
 
   EXPECT(mluOpExtSetSparseConvExtendedModes(handle, 1), MLUOP_STATUS_SUCCESS);
   EXPECT(mluOpExtSetDistinctPairsPromise(handle, 1), MLUOP_STATUS_SUCCESS);
+  EXPECT(mluOpExtGetRowMapSize(pairs, L, &bytes), MLUOP_STATUS_SUCCESS);
+  if (bytes < (size_t)K * L * 4) return 9;
+  EXPECT(mluOpExtUseRowMap(handle, fake), MLUOP_STATUS_BAD_PARAM);
+  EXPECT(mluOpExtForgetRowMap(handle, NULL), MLUOP_STATUS_SUCCESS);
 
   EXPECT(mluOpDestroyTensorDescriptor(indices), MLUOP_STATUS_SUCCESS);
   EXPECT(mluOpDestroyTensorDescriptor(pairs), MLUOP_STATUS_SUCCESS);
