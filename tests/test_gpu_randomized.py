@@ -108,6 +108,32 @@ def test_rulebook_and_convolutions(gpu_handle, block):
             except m.MluOpError:
                 continue   # e.g. more pairs in an offset than output_grad has rows: refused as in the reference
             torch.cuda.synchronize()
+            # with the rulebook's row maps kept across calls the operators must give the same bits
+            # (a map that lost pairs, as repeated coordinates make it, is refused and not tried)
+            fwd_map = m.RowMap(gpu_handle, pairs, num_host, y_rows, x_rows, 0 if inverse else 1)
+            bwd_map = m.RowMap(gpu_handle, pairs, num_host, x_rows, y_rows, 1 if inverse else 0)
+            # (repeated coordinates collide in the map whose rows are the outputs, not in the other)
+            assert dup > 0 or (fwd_map.usable and bwd_map.usable), what
+            if fwd_map.usable:
+                if inverse:
+                    out2 = m.indice_conv_forward(gpu_handle, xt, wt, m.LAYOUT_ARRAY, pairs, num_host, rows, False,
+                                                 inverse=1, row_map=fwd_map)
+                else:
+                    out2 = m.indice_conv_forward(gpu_handle, xt, wt, lay, pairs, num_host, n_out, sub_m,
+                                                 row_map=fwd_map)
+                torch.cuda.synchronize()
+                assert torch.equal(out2, out), what + " forward with its row map"
+            if bwd_map.usable:
+                if inverse:
+                    dx2 = m.indice_conv_backward_data(gpu_handle, dyt, wt, m.LAYOUT_ARRAY, pairs, num_host, False, ci,
+                                                      inverse=1, rows=n_out, row_map=bwd_map)
+                else:
+                    dx2 = m.indice_conv_backward_data(gpu_handle, dyt, wt, lay, pairs, num_host, sub_m, ci,
+                                                      row_map=bwd_map)
+                torch.cuda.synchronize()
+                assert torch.equal(dx2, dx), what + " backward data with its row map"
+            fwd_map.close()
+            bwd_map.close()
             grade(from_torch(out), oracle.forward(x, wk, pairs_o, num_o, y_rows, inverse=inverse), "forward")
             grade(from_torch(dx), oracle.backward_data(dy, wk, pairs_o, num_o, inverse=inverse, rows=x_rows)
                   if inverse else oracle.backward_data(dy, wk, pairs_o, num_o), "backward data")
