@@ -388,6 +388,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only-step", action="store_true",
                     help="run just warmup + timed steps (for profiler runs)")
+    ap.add_argument("--with-backward", action="store_true",
+                    help="with --only-step: every step also runs backward data and backward filter "
+                         "(profiler runs of the backward kernels; the printed figures stay those of "
+                         "rulebook + forward)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="with --only-step: also run one 64 MiB device-to-device copy, the known-size "
                          "kernel that scales the profiler's FETCH_SIZE / WRITE_SIZE counters")
@@ -436,6 +440,11 @@ def main():
         "rulebook_ms": rb_ms, "rulebook_ms_min": min(per["get_indice_pairs"]),
     }
     if args.only_step:
+        if args.with_backward:
+            for _ in range(args.steps):
+                step.backward_data()
+                step.backward_filter()
+            torch.cuda.synchronize()
         if args.calibration_copy:
             src = torch.ones(16 * 1024 * 1024, dtype=torch.float32, device="cuda")
             dst = torch.empty_like(src)
