@@ -40,6 +40,10 @@ WORKLOADS = {
     "config1": dict(grid=(1, 40, 400, 352), per_batch=20000, gen="uniform", seed=1, ci=16, co=16,
                     dtype="float32", ks=(3, 3, 3),
                     text="BASELINE config 1: subm 3x3x3, 20000 uniform voxels in 1x40x400x352, Ci=Co=16 fp32"),
+    "config5a": dict(grid=(1, 64, 1024, 1024), per_batch=400000, gen="surface", seed=5, ci=128, co=128,
+                     dtype="float16", ks=(5, 5, 5),
+                     text="BASELINE config 5, first layer: subm 5x5x5, 400000 voxels on 50 planes and spheres "
+                          "(5 % uniform noise) in 1x64x1024x1024, Ci=Co=128 fp16"),
 }
 
 
@@ -54,6 +58,8 @@ class Step:
         grid = wl["grid"]
         if wl["gen"] == "clustered":
             idx = m.datagen.clustered_voxels(grid, wl["per_batch"], wl["seed"])
+        elif wl["gen"] == "surface":
+            idx = m.datagen.surface_voxels(grid, wl["per_batch"], wl["seed"])
         else:
             idx = m.datagen.uniform_voxels(grid, wl["per_batch"] * grid[0], wl["seed"])
         self.idx_np = idx

@@ -1295,6 +1295,87 @@ __global__ __launch_bounds__(64 * kSliceSumWaves) void sliceSum(const float *par
   }
 }
 
+// The same sum on a flat grid for filters with many offsets, where most offsets own
+// a handful of slices and a 1024-thread workgroup per 256 elements is mostly idle
+// waves (at 125 offsets x 128 x 128: 8000 workgroups, dispatch-bound).  An offset with
+// at most 16 slices is "thin": each wave sums one 256-element chunk on its own, so a
+// workgroup covers 16 chunks and needs no barrier.  The additions are those of
+// sliceSum in the same order (a wave's partial there is 0 + slice g when the offset
+// has at most 16 slices), so both kernels give the same bits.
+struct SumGrid {
+  int first[kMaxInlineK];  // workgroups in front of the offset's first one
+};
+constexpr int kThinSlices = kSliceSumWaves;
+
+template <typename E>
+__global__ __launch_bounds__(64 * kSliceSumWaves) void sliceSumFlat(const float *partial,
+                                                                    SliceTable tab, SumGrid grid,
+                                                                    int K, int slice_len,
+                                                                    int tile_elems, int Co,
+                                                                    GradLayout lay,
+                                                                    typename E::storage *dW) {
+  constexpr int W = kSliceSumWaves;
+  __shared__ float4v s_part[W][64];
+  // last offset whose first workgroup is not behind this one
+  int lo = 0, hi = K - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (grid.first[mid] <= (int)blockIdx.x) lo = mid; else hi = mid - 1;
+  }
+  const int k = lo;
+  const int chunk = blockIdx.x - grid.first[k];
+  const int lane = threadIdx.x & 63;
+  const int g = threadIdx.x >> 6;
+  const int slices = (tab.n[k] + slice_len - 1) / slice_len;
+  const float *tiles = partial + (size_t)tab.first[k] * tile_elems;
+  if (slices <= kThinSlices) {
+    const int e = ((chunk * W + g) * 64 + lane) * 4;
+    if (e >= tile_elems) return;
+    float4v t[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      t[i] = float4v{0.f, 0.f, 0.f, 0.f};
+      if (i < slices) t[i] += *reinterpret_cast<const float4v *>(tiles + (size_t)i * tile_elems + e);
+    }
+#pragma unroll
+    for (int span = 1; span < W; span *= 2)
+#pragma unroll
+      for (int i = 0; i < W; i += 2 * span) t[i] += t[i + span];
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      E::store(dW + gradOffset(lay, k, (e + v) / Co, (e + v) % Co), t[0][v]);
+    return;
+  }
+  const int e = (chunk * 64 + lane) * 4;
+  float4v acc[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) acc[u] = float4v{0.f, 0.f, 0.f, 0.f};
+  {
+    const float *src = tiles + e;
+    for (int i0 = g; i0 < slices; i0 += 8 * W) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + W * u;
+        if (i < slices) acc[u] += *reinterpret_cast<const float4v *>(src + (size_t)i * tile_elems);
+      }
+    }
+  }
+  s_part[g][lane] = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+  __syncthreads();
+  if (g == 0) {
+    float4v t[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) t[i] = s_part[i][lane];
+#pragma unroll
+    for (int span = 1; span < W; span *= 2)
+#pragma unroll
+      for (int i = 0; i < W; i += 2 * span) t[i] += t[i + span];
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      E::store(dW + gradOffset(lay, k, (e + v) / Co, (e + v) % Co), t[0][v]);
+  }
+}
+
 // ---- host side -----------------------------------------------------------------------
 
 inline size_t alignUp(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
@@ -1310,6 +1391,16 @@ inline char *alignPtr(void *p) {
 inline int gridFor(size_t n, int cap = 8192) {
   size_t b = (n + 255) / 256;
   return (int)(b < 1 ? 1 : (b > (size_t)cap ? (size_t)cap : b));
+}
+
+// Test switch: "1" sums the backward filter's partial tiles on the flat grid whatever
+// the shape, "0" never does (the two kernels must give the same bits); unset, the
+// grid's size decides.
+constexpr int kFlatSumFromBlocks = 2048;
+int sliceSumMode() {
+  const char *v = getenv("MLUOP_SPCONV_FLAT_SLICE_SUM");
+  if (v == nullptr || (v[0] != '0' && v[0] != '1')) return -1;
+  return v[0] - '0';
 }
 
 bool forceSimt() {
@@ -1686,9 +1777,25 @@ void launchFilterMfmaInstance(const LaunchCtx &lc, const ConvProblem &p, const S
         p.L, p.inverse ? 1 : 0, p.inverse ? p.num_out : p.L, p.inverse ? p.L : p.num_out, p.K,
         tab, slice_len, partial);
   lc.end();
+  // Many offsets of few slices each: the flat grid, on which such an offset takes a
+  // sixteenth of the workgroups (same bits).
+  constexpr int kChunks = CI * CO / 256;
+  SumGrid sg;
+  int blocks = 0;
+  for (int k = 0; k < p.K; ++k) {
+    const int sl = (tab.n[k] + slice_len - 1) / slice_len;
+    sg.first[k] = blocks;
+    blocks += sl <= kThinSlices ? (kChunks + kSliceSumWaves - 1) / kSliceSumWaves : kChunks;
+  }
+  const int flat_mode = sliceSumMode();
+  const bool flat = flat_mode == 1 || (flat_mode < 0 && kChunks * p.K > kFlatSumFromBlocks);
   lc.begin("sliceSum");
-  sliceSum<E><<<dim3(CI * CO / 256, p.K), 64 * kSliceSumWaves, 0, lc.stream>>>(
-      partial, tab, slice_len, CI * CO, CO, gradLayout(p), static_cast<S *>(filters_grad));
+  if (flat)
+    sliceSumFlat<E><<<blocks, 64 * kSliceSumWaves, 0, lc.stream>>>(
+        partial, tab, sg, p.K, slice_len, CI * CO, CO, gradLayout(p), static_cast<S *>(filters_grad));
+  else
+    sliceSum<E><<<dim3(kChunks, p.K), 64 * kSliceSumWaves, 0, lc.stream>>>(
+        partial, tab, slice_len, CI * CO, CO, gradLayout(p), static_cast<S *>(filters_grad));
   lc.end();
 }
 

@@ -370,3 +370,38 @@ def test_tensors_that_are_not_16_byte_aligned(gpu_handle, dtype_name):
     check_close(from_torch(dx), oracle.backward_data(dy_r, w_k, c["pairs"], c["num"]), dtype_name, "backward_data")
     ref = oracle.backward_filter(feats_r, dy_r, c["pairs"], c["num"], fast=True)
     check_close(from_torch(dw).reshape(ref.shape), ref, dtype_name, "backward_filter")
+
+
+@pytest.mark.parametrize("case", [
+    # (space, L, ks, ci, co)
+    ((41, 400, 352), 40000, (3, 3, 3), 64, 64),   # centre offset: hundreds of slices, the others a few
+    ((20, 40, 40), 20000, (3, 3, 3), 32, 16),     # offsets between 17 and 128 slices next to thin ones
+    ((12, 12, 12), 1500, (5, 5, 5), 128, 128),    # 125 offsets of one or two slices: the shape the flat grid is for
+    ((8, 8, 8), 300, (3, 3, 3), 16, 16),          # one 256-element chunk per offset
+])
+@pytest.mark.parametrize("dtype_name", ["float32", "float16", "bfloat16"])
+def test_flat_slice_sum_gives_the_bits_of_the_grid_one(gpu_handle, case, dtype_name):
+    """Backward filter adds an offset's partial tiles with one of two kernels, chosen by the size of
+    the grid; both add the slices in the same order and tree, so the filter gradient must not
+    depend on the choice.  Also graded against the oracle."""
+    import torch
+    import mluop_hip
+    space, L, ks, ci, co = case
+    print("slice sum case", case, dtype_name, flush=True)
+    c = conv_case(23, 1, space, L, ks, ci, co, True)
+    feats_t = to_torch(round_to(c["feats"], dtype_name), dtype_name, "cuda")
+    dy_t = to_torch(round_to(c["dy"], dtype_name), dtype_name, "cuda")
+    pairs_t = torch.from_numpy(c["pairs"]).cuda()
+    num_host = [int(v) for v in c["num"]]
+    got = {}
+    try:
+        for mode in ("1", "0"):
+            os.environ["MLUOP_SPCONV_FLAT_SLICE_SUM"] = mode
+            if mode == "1":
+                run_all_ops(gpu_handle, c, dtype_name, check=("bwd_filter",))
+            dw = mluop_hip.indice_conv_backward_filter(gpu_handle, feats_t, dy_t, pairs_t, num_host, c["ks"], True)
+            torch.cuda.synchronize()
+            got[mode] = dw.view(torch.int16 if dtype_name != "float32" else torch.int32).cpu()
+    finally:
+        os.environ.pop("MLUOP_SPCONV_FLAT_SLICE_SUM", None)
+    assert torch.equal(got["1"], got["0"])
