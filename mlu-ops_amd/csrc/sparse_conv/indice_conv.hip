@@ -140,6 +140,35 @@ __global__ __launch_bounds__(256) void scatterRowMap(const int32_t *pairs, int L
   }
 }
 
+// The same on a flat grid: an offset gets the workgroups its pairs need and no
+// more.  The (pairs, offset) grid above is sized by the fullest offset; at 125
+// offsets of which one holds a quarter of all pairs, nine in ten of its workgroups
+// exit at once and their dispatch is what the kernel costs.
+struct OffsetBlocks {
+  int first[kMaxInlineK];  // workgroups in front of the offset's first one
+};
+
+__global__ __launch_bounds__(256) void scatterRowMapFlat(const int32_t *pairs, int L,
+                                                         OffsetCounts inl, OffsetBlocks blocks,
+                                                         int K, int row_col, int src_col,
+                                                         int n_rows, int n_src, int32_t *map) {
+  // last offset whose first workgroup is not behind this one (an offset without
+  // pairs shares its prefix with the next one and is never chosen)
+  int lo = 0, hi = K - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (blocks.first[mid] <= (int)blockIdx.x) lo = mid; else hi = mid - 1;
+  }
+  const int k = lo;
+  const int p = ((int)blockIdx.x - blocks.first[k]) * 256 + threadIdx.x;
+  if (p >= inl.n[k]) return;
+  const int32_t *base = pairs + (size_t)k * 2 * L;
+  const int r = base[(size_t)row_col * L + p];
+  const int s = base[(size_t)src_col * L + p];
+  if ((unsigned)r < (unsigned)n_rows && (unsigned)s < (unsigned)n_src)
+    map[(size_t)k * n_rows + r] = s;
+}
+
 // ---- SIMT gather convolution -------------------------------------------------
 // result[r, c] = sum_k sum_q A[map[k][r], q] * B(k, q, c),
 // B(k, q, c) = W[k*sK + q*sQ + c*sC].  32 x 64 result tile per block.
@@ -1640,13 +1669,42 @@ void launchDense(const LaunchCtx &lc, int Q, int C, const void *A, const void *p
 #undef DENSE_CASE
 }
 
+// Test switch: "1" builds every row map on the flat grid.
+constexpr int kFlatScatterFromBlocks = 16384;
+bool forceFlatScatter() {
+  const char *v = getenv("MLUOP_SPCONV_FLAT_SCATTER");
+  return v != nullptr && v[0] == '1';
+}
+
+// Caller brackets this with its timing marks.  dev_counts != nullptr: more offsets
+// than the inline tables hold, counts in device memory, grid kernel only.
+void enqueueScatterRowMap(hipStream_t stream, const int32_t *pairs, int L, int K,
+                          const OffsetCounts &inl, const int32_t *dev_counts, int max_count,
+                          int row_col, int src_col, int n_rows, int n_src, int32_t *map) {
+  const int gx = (max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256;
+  if (dev_counts == nullptr && K <= kMaxInlineK &&
+      ((long long)gx * K > kFlatScatterFromBlocks || forceFlatScatter())) {
+    OffsetBlocks ob;
+    int blocks = 0;
+    for (int k = 0; k < K; ++k) {
+      ob.first[k] = blocks;
+      blocks += inl.n[k] > 0 ? (inl.n[k] + 255) / 256 : 0;
+    }
+    if (blocks > 0)
+      scatterRowMapFlat<<<blocks, 256, 0, stream>>>(pairs, L, inl, ob, K, row_col, src_col, n_rows,
+                                                   n_src, map);
+    return;
+  }
+  scatterRowMap<<<dim3(gx, K), 256, 0, stream>>>(pairs, L, inl, dev_counts, row_col, src_col,
+                                                 n_rows, n_src, map);
+}
+
 void launchScatterRowMap(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d,
                          const GatherWorkspace &ws, const OffsetCounts &inl, int max_count) {
   if (max_count <= 0) return;
-  dim3 grid((max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256, p.K);
   lc.begin("scatterRowMap");
-  scatterRowMap<<<grid, 256, 0, lc.stream>>>(p.indice_pairs, p.L, inl, ws.dev_counts, d.row_col,
-                                          d.src_col, d.R, d.n_src, ws.map);
+  enqueueScatterRowMap(lc.stream, p.indice_pairs, p.L, p.K, inl, ws.dev_counts, max_count, d.row_col,
+                       d.src_col, d.R, d.n_src, ws.map);
   lc.end();
 }
 
@@ -1938,12 +1996,10 @@ hipError_t buildRowMap(const LaunchCtx &lc, const int32_t *indice_pairs, const i
   lc.end();
   fillInt32<<<1, 256, 0, lc.stream>>>(counter, 1, 0);
   if (max_count > 0) {
-    dim3 grid((max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256, shape.K);
     lc.begin("scatterRowMap");
-    scatterRowMap<<<grid, 256, 0, lc.stream>>>(indice_pairs, shape.L, inl,
-                                            shape.K > kMaxInlineK ? dev_counts : nullptr,
-                                            shape.row_column, 1 - shape.row_column, shape.rows,
-                                            shape.source_rows, map);
+    enqueueScatterRowMap(lc.stream, indice_pairs, shape.L, shape.K, inl,
+                         shape.K > kMaxInlineK ? dev_counts : nullptr, max_count, shape.row_column,
+                         1 - shape.row_column, shape.rows, shape.source_rows, map);
     lc.end();
   }
   if (filled_host == nullptr) return hipGetLastError();

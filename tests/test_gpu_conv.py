@@ -405,3 +405,38 @@ def test_flat_slice_sum_gives_the_bits_of_the_grid_one(gpu_handle, case, dtype_n
     finally:
         os.environ.pop("MLUOP_SPCONV_FLAT_SLICE_SUM", None)
     assert torch.equal(got["1"], got["0"])
+
+
+@pytest.mark.parametrize("shape", [SHAPES[0], SHAPES[3], SHAPES[4], SHAPES[5],
+                                   (1, (30, 30, 30), 40, (3, 3, 3), 32, 32, True, (1, 1, 1))])  # offsets without pairs
+@pytest.mark.parametrize("dtype_name", ["float32", "float16"])
+def test_flat_row_map_scatter_gives_the_same_results(gpu_handle, shape, dtype_name):
+    """The row map of a gather convolution is written by one of two kernels, chosen by the size of
+    the grid; with distinct coordinates every map slot has one writer, so forward and backward
+    data must not depend on the choice.  Also graded against the oracle."""
+    import torch
+    import mluop_hip
+    batch, space, L, ks, ci, co, sub_m, stride = shape
+    print("flat scatter case", shape, dtype_name, flush=True)
+    c = conv_case(31, batch, space, L, ks, ci, co, sub_m, stride)
+    feats_t = to_torch(round_to(c["feats"], dtype_name), dtype_name, "cuda")
+    w_t = to_torch(round_to(c["w"], dtype_name), dtype_name, "cuda")
+    dy_t = to_torch(round_to(c["dy"], dtype_name), dtype_name, "cuda")
+    pairs_t = torch.from_numpy(c["pairs"]).cuda()
+    num_host = [int(v) for v in c["num"]]
+    got = {}
+    try:
+        for mode in ("1", "0"):
+            os.environ["MLUOP_SPCONV_FLAT_SCATTER"] = mode
+            if mode == "1":
+                run_all_ops(gpu_handle, c, dtype_name, check=("fwd", "bwd_data"))
+            out = mluop_hip.indice_conv_forward(gpu_handle, feats_t, w_t, mluop_hip.LAYOUT_ARRAY, pairs_t, num_host,
+                                                c["n_out"], c["sub_m"])
+            dx = mluop_hip.indice_conv_backward_data(gpu_handle, dy_t, w_t, mluop_hip.LAYOUT_ARRAY, pairs_t,
+                                                     num_host, c["sub_m"], c["ci"])
+            torch.cuda.synchronize()
+            as_int = torch.int16 if dtype_name != "float32" else torch.int32
+            got[mode] = (out.view(as_int).cpu(), dx.view(as_int).cpu())
+    finally:
+        os.environ.pop("MLUOP_SPCONV_FLAT_SCATTER", None)
+    assert torch.equal(got["1"][0], got["0"][0]) and torch.equal(got["1"][1], got["0"][1])
