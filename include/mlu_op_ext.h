@@ -92,6 +92,25 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtBuildRowMap(mluOpHandle_t handle,
 mluOpStatus_t MLUOP_WIN_API mluOpExtUseRowMap(mluOpHandle_t handle, const void *row_map);
 mluOpStatus_t MLUOP_WIN_API mluOpExtForgetRowMap(mluOpHandle_t handle, const void *row_map);
 
+/* mluOpIndiceConvolutionBackwardFilter for callers that cannot allocate device memory (code
+ * under HIP graph capture, serving loops, harnesses that forbid hipMalloc) and therefore have
+ * no workspace to hand over.  No counterpart in the reference.  Same arguments, checks and
+ * result bits as mluOpIndiceConvolutionBackwardFilter (mlu_op.h), without `workspace` and
+ * `workspace_size`: the partial sums live in an array of MLUOP_EXT_NO_ALLOC_SCRATCH_BYTES that
+ * the library holds on every GPU it runs on until the process ends.  The call allocates and
+ * frees nothing and does not wait for the queue.  MLUOP_STATUS_NOT_SUPPORTED when the shape
+ * needs more scratch memory than that (mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize
+ * reports the need) or more than 128 kernel offsets.  All calls on one GPU share the array:
+ * calls that can overlap there (different queues, different handles) race and must be ordered
+ * by the caller. */
+#define MLUOP_EXT_NO_ALLOC_SCRATCH_BYTES (16 * 1024 * 1024)
+mluOpStatus_t MLUOP_WIN_API mluOpExtIndiceConvolutionBackwardFilterNoAlloc(
+    mluOpHandle_t handle, const mluOpTensorDescriptor_t features_desc, const void *features,
+    const mluOpTensorDescriptor_t output_grad_desc, const void *output_grad,
+    const mluOpTensorDescriptor_t indice_pairs_desc, const void *indice_pairs,
+    const int64_t indice_num[], const int64_t inverse, const int64_t subm,
+    const mluOpTensorDescriptor_t filters_grad_desc, void *filters_grad);
+
 #if defined(__cplusplus)
 }
 #endif

@@ -8,6 +8,7 @@
 
 #include "core/core.h"
 #include "mlu_op_ext.h"
+#include "sparse_conv/no_alloc_scratch.h"
 
 namespace {
 
@@ -70,6 +71,15 @@ mluOpStatus_t MLUOP_WIN_API mluOpCreate(mluOpHandle_t *handle) {
     return MLUOP_STATUS_ALLOC_FAILED;
   }
   ctx->pinned_scalar = static_cast<int32_t *>(pinned);
+  // `dev` is the current device: the address of the library's scratch array on it is looked
+  // up here, once, so that the entry point that uses it has nothing to set up.
+  err = mluop::sparse_conv::lookUpNoAllocScratch(dev);
+  if (err != hipSuccess) {
+    (void)hipGetLastError();
+    MLUOP_LOG(WARNING) << "[mluOpCreate] hipGetSymbolAddress for the scratch array failed: "
+                       << hipGetErrorString(err)
+                       << "; mluOpExtIndiceConvolutionBackwardFilterNoAlloc will refuse to run.";
+  }
   *handle = ctx;
   return MLUOP_STATUS_SUCCESS;
 }

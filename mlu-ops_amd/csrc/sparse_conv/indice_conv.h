@@ -79,6 +79,9 @@ hipError_t buildRowMap(const LaunchCtx &lc, const int32_t *indice_pairs, const i
                        const RowMapShape &shape, void *row_map, int32_t *filled_host);
 
 size_t backwardFilterWorkspaceBytes(const ConvProblem &p);
+// True when launchBackwardFilter only enqueues kernels for this shape: no staging copy of the
+// per-offset counts, no wait for the stream.
+bool backwardFilterLaunchesOnly(const ConvProblem &p);
 hipError_t launchBackwardFilter(const LaunchCtx &lc, const ConvProblem &p, const void *features,
                                 const void *output_grad, void *workspace, void *filters_grad);
 

@@ -2015,6 +2015,8 @@ size_t backwardFilterWorkspaceBytes(const ConvProblem &p) {
   return carveFilterGrad(p, nullptr).bytes;
 }
 
+bool backwardFilterLaunchesOnly(const ConvProblem &p) { return p.K <= kMaxInlineK; }
+
 hipError_t launchBackwardFilter(const LaunchCtx &lc, const ConvProblem &p, const void *features,
                                 const void *output_grad, void *workspace, void *filters_grad) {
   const FilterGradWorkspace ws = carveFilterGrad(p, workspace);

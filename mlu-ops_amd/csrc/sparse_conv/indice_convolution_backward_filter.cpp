@@ -3,12 +3,27 @@
 // kernels/sparse_conv/indice_convolution_backward_filter/
 // indice_convolution_backward_filter.cpp:100-258 and :536-620; bfloat16 is
 // accepted in addition to half and float.
+#include <hip/hip_runtime.h>
+
+#include <mutex>
 #include <string>
 
 #include "core/core.h"
+#include "mlu_op_ext.h"
 #include "sparse_conv/indice_conv.h"
+#include "sparse_conv/no_alloc_scratch.h"
 
 namespace {
+
+// Device memory of mluOpExtIndiceConvolutionBackwardFilterNoAlloc: the fp32 partial tiles
+// that the ordinary entry point keeps in the caller's workspace.  One copy per GPU, held
+// until the process ends.  The name is a host-side stand-in: host code uses the address
+// hipGetSymbolAddress returned for the device in question, never the name.
+static __device__ __align__(256) unsigned char scratch[MLUOP_EXT_NO_ALLOC_SCRATCH_BYTES];
+
+constexpr int kMaxScratchDevices = 64;
+std::mutex g_scratch_lock;
+void *g_scratch_ptr[kMaxScratchDevices] = {nullptr};
 
 using mluop::sparse_conv::ConvProblem;
 using mluop::sparse_conv::ElemType;
@@ -190,6 +205,23 @@ ConvProblem makeProblem(mluOpHandle_t handle, const mluOpTensorDescriptor_t feat
 
 }  // namespace
 
+namespace mluop {
+namespace sparse_conv {
+
+hipError_t lookUpNoAllocScratch(int device) {
+  if (device < 0 || device >= kMaxScratchDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (g_scratch_ptr[device] != nullptr) return hipSuccess;
+  void *ptr = nullptr;
+  const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (err != hipSuccess) return err;
+  g_scratch_ptr[device] = ptr;
+  return hipSuccess;
+}
+
+}  // namespace sparse_conv
+}  // namespace mluop
+
 extern "C" {
 
 mluOpStatus_t MLUOP_WIN_API mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize(
@@ -249,6 +281,53 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardFilter(
   HIP_CHECK_RETURN(api, mluop::sparse_conv::launchBackwardFilter(handle->launchCtx(), p, features,
                                                                 output_grad, workspace,
                                                                 filters_grad));
+  return MLUOP_STATUS_SUCCESS;
+}
+
+mluOpStatus_t MLUOP_WIN_API mluOpExtIndiceConvolutionBackwardFilterNoAlloc(
+    mluOpHandle_t handle, const mluOpTensorDescriptor_t features_desc, const void *features,
+    const mluOpTensorDescriptor_t output_grad_desc, const void *output_grad,
+    const mluOpTensorDescriptor_t indice_pairs_desc, const void *indice_pairs,
+    const int64_t indice_num[], const int64_t inverse, const int64_t subm,
+    const mluOpTensorDescriptor_t filters_grad_desc, void *filters_grad) {
+  const std::string api = "[mluOpExtIndiceConvolutionBackwardFilterNoAlloc]";
+  (void)subm;
+  mluOpStatus_t st = baseParamCheck(api, handle, features_desc, output_grad_desc,
+                                    indice_pairs_desc, filters_grad_desc, indice_num, inverse);
+  if (st != MLUOP_STATUS_SUCCESS) return st;
+  if (anyZeroElement(features_desc, output_grad_desc, indice_pairs_desc, filters_grad_desc)) {
+    return MLUOP_STATUS_SUCCESS;
+  }
+  PARAM_CHECK(api, features != nullptr);
+  PARAM_CHECK(api, output_grad != nullptr);
+  PARAM_CHECK(api, indice_pairs != nullptr);
+  PARAM_CHECK(api, filters_grad != nullptr);
+  const ConvProblem p =
+      makeProblem(handle, features_desc, output_grad_desc, indice_pairs_desc, filters_grad_desc,
+                  indice_num, inverse, indice_pairs);
+  if (!mluop::sparse_conv::backwardFilterLaunchesOnly(p)) {
+    MLUOP_LOG(ERROR) << api << " a kernel volume of " << p.K << " offsets needs a staging copy "
+                     << "and a wait for the queue; use mluOpIndiceConvolutionBackwardFilter.";
+    return MLUOP_STATUS_NOT_SUPPORTED;
+  }
+  const size_t need = mluop::sparse_conv::backwardFilterWorkspaceBytes(p);
+  if (need > (size_t)MLUOP_EXT_NO_ALLOC_SCRATCH_BYTES) {
+    MLUOP_LOG(ERROR) << api << " this shape needs " << need << " bytes of scratch memory, the "
+                     << "library holds " << (size_t)MLUOP_EXT_NO_ALLOC_SCRATCH_BYTES
+                     << "; use mluOpIndiceConvolutionBackwardFilter with a workspace.";
+    return MLUOP_STATUS_NOT_SUPPORTED;
+  }
+  DEVICE_HANDLE_CHECK(api, handle);
+  void *ptr = handle->device < kMaxScratchDevices ? g_scratch_ptr[handle->device] : nullptr;
+  if (ptr == nullptr) {
+    MLUOP_LOG(ERROR) << api << " the scratch memory of device " << handle->device
+                     << " was not found when the handle was created.";
+    return MLUOP_STATUS_NOT_INITIALIZED;
+  }
+  // no event pairs here: the per-kernel timer creates events on demand
+  const mluop::LaunchCtx lc(handle->queue, nullptr);
+  HIP_CHECK_RETURN(api, mluop::sparse_conv::launchBackwardFilter(lc, p, features, output_grad,
+                                                                ptr, filters_grad));
   return MLUOP_STATUS_SUCCESS;
 }
 

@@ -128,6 +128,8 @@ SIGNATURES = {
                                            ctypes.POINTER(ctypes.c_int64)]),
     "mluOpExtUseRowMap": (ctypes.c_int, [_vp, _vp]),
     "mluOpExtForgetRowMap": (ctypes.c_int, [_vp, _vp]),
+    "mluOpExtIndiceConvolutionBackwardFilterNoAlloc": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64p, ctypes.c_int64, ctypes.c_int64, _vp, _vp]),
     "mluOpExtGetKernelTimingCount": (ctypes.c_int, [_vp, _ip]),
     "mluOpExtGetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int, ctypes.POINTER(ctypes.c_char_p),
                                                ctypes.POINTER(ctypes.c_float)]),
@@ -478,6 +480,28 @@ def indice_conv_backward_filter(handle, features, output_grad, indice_pairs, ind
         indice_pairs.data_ptr(), counts, inverse, int(sub_m), ws.data_ptr(), size.value, d_dw.ptr,
         dw.data_ptr()), "mluOpIndiceConvolutionBackwardFilter")
     return dw
+
+
+NO_ALLOC_SCRATCH_BYTES = 16 * 1024 * 1024  # MLUOP_EXT_NO_ALLOC_SCRATCH_BYTES
+
+
+def indice_conv_backward_filter_no_alloc(handle, features, output_grad, indice_pairs, indice_num_host,
+                                         filter_space, sub_m, filters_grad, inverse=0,
+                                         onchip_float=True):
+    """mluOpExtIndiceConvolutionBackwardFilterNoAlloc into the caller's `filters_grad`
+    ([kd, kh, kw, Ci, Co]): no workspace, the library's own scratch array instead."""
+    code = torch_dtype_code(features.dtype)
+    K, _, L = indice_pairs.shape
+    d_x = TensorDescriptor(LAYOUT_ARRAY, code, list(features.shape))
+    d_dy = TensorDescriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
+    d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+    d_dw = TensorDescriptor(LAYOUT_ARRAY, code, list(filters_grad.shape),
+                            onchip_dtype=DTYPE_FLOAT if onchip_float else None)
+    check(lib().mluOpExtIndiceConvolutionBackwardFilterNoAlloc(
+        handle.ptr, d_x.ptr, features.data_ptr(), d_dy.ptr, output_grad.data_ptr(), d_pairs.ptr,
+        indice_pairs.data_ptr(), _host_counts(indice_num_host), inverse, int(sub_m), d_dw.ptr,
+        filters_grad.data_ptr()), "mluOpExtIndiceConvolutionBackwardFilterNoAlloc")
+    return filters_grad
 
 
 def voxelization(handle, points, voxel_size, coors_range, max_points, max_voxels, deterministic=True):
