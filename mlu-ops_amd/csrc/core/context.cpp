@@ -2,6 +2,7 @@
 // small per-handle switches.  Behaviour follows reference
 // core/context.cpp:158-470; the MLU attribute reads become a read of the HIP
 // device properties and the queue is a hipStream_t.
+#include <chrono>
 #include <cstdlib>
 #include <cstring>
 #include <new>
@@ -64,13 +65,21 @@ mluOpStatus_t MLUOP_WIN_API mluOpCreate(mluOpHandle_t *handle) {
   ctx->cu_count = prop.multiProcessorCount;
   ctx->lds_bytes = (int)prop.sharedMemPerBlock;
   void *pinned = nullptr;
-  err = hipHostMalloc(&pinned, 64, hipHostMallocDefault);
+  const size_t pinned_bytes = 64 + sizeof(mluOpContext::RulebookReport) * mluOpContext::kRulebookNotes;
+  err = hipHostMalloc(&pinned, pinned_bytes, hipHostMallocDefault);
   if (err != hipSuccess) {
     MLUOP_LOG(ERROR) << "[mluOpCreate] hipHostMalloc failed: " << hipGetErrorString(err);
     delete ctx;
     return MLUOP_STATUS_ALLOC_FAILED;
   }
   ctx->pinned_scalar = static_cast<int32_t *>(pinned);
+  memset(pinned, 0, pinned_bytes);
+  ctx->rulebook_reports =
+      reinterpret_cast<mluOpContext::RulebookReport *>(static_cast<char *>(pinned) + 64);
+  // Stamps and tickets only have to differ from what earlier calls, of this handle or of
+  // another, left in memory: start somewhere no other handle starts.
+  ctx->next_stamp = ((unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count()
+                     << 20) ^ (unsigned long long)reinterpret_cast<uintptr_t>(ctx) ^ 0x9E3779B97F4A7C15ull;
   // `dev` is the current device: the address of the library's scratch array on it is looked
   // up here, once, so that the entry point that uses it has nothing to set up.
   err = mluop::sparse_conv::lookUpNoAllocScratch(dev);

@@ -50,6 +50,27 @@ struct mluOpContext {
   };
   std::vector<RowMapRecord> row_maps;
   const void *pending_row_map = nullptr;
+  // Rulebooks mluOpGetIndicePairs built on this handle, by the address of their pair tensor.
+  // The last kernel of a rulebook reports into a slot of pinned host memory whether the
+  // input rows were in cell order (then both pair columns ascend inside every offset); the
+  // convolution operators read the slot, without waiting for anything, to choose their way
+  // through the pair lists.  A note is a hint about speed only: what the kernels rely on is
+  // checked on the device in every call.
+  struct RulebookReport {       // pinned host memory, written by the device
+    unsigned long long stamp;   // the note's stamp, stored after the flag
+    unsigned int rows_in_order;
+    unsigned int unused;
+  };
+  struct RulebookNote {
+    const void *pairs = nullptr;
+    int K = 0, L = 0;
+    unsigned long long stamp = 0;
+  };
+  static constexpr int kRulebookNotes = 32;
+  RulebookNote rulebook_notes[kRulebookNotes];
+  RulebookReport *rulebook_reports = nullptr;  // kRulebookNotes slots behind pinned_scalar
+  int next_rulebook_note = 0;
+  unsigned long long next_stamp = 1;   // also the source of per-call tickets
 
   // What the kernel launchers need: the stream, and the timer while it is on.
   mluop::LaunchCtx launchCtx() { return mluop::LaunchCtx(queue, timer.enabled ? &timer : nullptr); }

@@ -8,6 +8,7 @@
 
 #include "core/core.h"
 #include "sparse_conv/rulebook.h"
+#include "sparse_conv/rulebook_notes.h"
 
 namespace {
 
@@ -205,16 +206,18 @@ mluOpStatus_t MLUOP_WIN_API mluOpGetIndicePairs(
   int32_t *pairs = static_cast<int32_t *>(indice_pairs);
   int32_t *out_rows = static_cast<int32_t *>(out_indices);
   int32_t *counts = static_cast<int32_t *>(indice_num);
+  const mluop::sparse_conv::RulebookReportTarget report =
+      mluop::sparse_conv::openRulebookNote(handle, indice_pairs, g.K, g.L);
   if (g.sub_m) {
     // Submanifold mode leaves num_act_out untouched, as the reference does
     // (normal_get_indice_pairs.cpp:848-975): the caller uses the input row count.
     HIP_CHECK_RETURN(api, mluop::sparse_conv::launchSubmRulebook(handle->launchCtx(), g, in_rows, workspace,
-                                                                 pairs, out_rows, counts));
+                                                                 pairs, out_rows, counts, report));
     return MLUOP_STATUS_SUCCESS;
   }
   HIP_CHECK_RETURN(api, mluop::sparse_conv::launchRegularRulebook(handle->launchCtx(), g, in_rows, workspace,
                                                                   pairs, out_rows, counts,
-                                                                  handle->pinned_scalar));
+                                                                  handle->pinned_scalar, report));
   // The output row count travels back through the host descriptor, which needs
   // one wait on the queue (the reference waits at normal_get_indice_pairs.cpp:531-533).
   HIP_CHECK_RETURN(api, hipStreamSynchronize(handle->queue));

@@ -46,6 +46,12 @@ struct ConvProblem {
   // built ahead by buildRowMap with no pair lost (so the pairs are distinct as well); the
   // launch then neither clears nor fills a map of its own.
   const int32_t *row_map = nullptr;
+  // Forward and backward data: the caller has reason to believe (it is checked on the
+  // device) that inside every offset the pair column naming the result rows ascends strictly
+  // and all indices are in range, so the kernels read the lists cut by tile instead of
+  // building a row map.  `ticket` is a value no earlier launch on this workspace used.
+  bool lists_in_order = false;
+  unsigned long long ticket = 0;
   // Backward filter only: element strides of dW(k, ci, co) in filters_grad;
   // all zero = the positional [K, Ci, Co].
   int64_t grad_stride_k = 0, grad_stride_ci = 0, grad_stride_co = 0;

@@ -286,6 +286,169 @@ __global__ __launch_bounds__(256) void fillMapPackFilter(int32_t *map, size_t ma
   }
 }
 
+// ---- where a gather kernel finds the pairs of its tile -------------------------------
+//
+// Either a dense row map (above), or the pair lists themselves, cut by tile.  The
+// second needs the column of the pairs that names the result rows to ascend strictly
+// inside every offset, which is how mluOpGetIndicePairs lists them: its input-row
+// column always does (backward data), its output-row column does when the input rows
+// are ordered by cell (forward).  The pairs of one offset that fall into a tile of
+// result rows are then one contiguous piece of the list, and a [K, tiles + 1] table
+// of cut positions replaces the [K, rows] map: nothing to clear, no slot a second pair
+// could lose, a few kilobytes instead of K * rows * 4 bytes.
+struct MapSource {
+  static constexpr bool kSegments = false;
+  const int32_t *map;
+  int32_t *filled;
+};
+
+struct SegmentSource {
+  static constexpr bool kSegments = true;
+  const int32_t *pairs;               // [K, 2, L]
+  const int32_t *cuts;                // [K, cut_stride]: first pair of every tile, then the count
+  const unsigned long long *verdict;  // holds `ticket` when some list is not in order
+  unsigned long long ticket;
+  int L, row_col, src_col, n_src, cut_stride;
+  const void *W;                      // the filter as the caller passed it, for lists out of order
+  int64_t sK, sQ, sC;
+  OffsetCounts counts;
+};
+
+// The pairs of one tile of result rows [r_begin, r_end) when the lists cannot be cut:
+// every workgroup reads all pairs of all offsets, and each pair that names one of its
+// rows is multiplied by one wave, a lane per result column, and added to the tile's
+// fp32 rows in LDS (`acc`, cleared by the caller).  Offsets are taken in order with a
+// barrier between them, so a row sees its offsets in the order the list kernels use;
+// only rows that several pairs of one offset name depend on timing in their last
+// bits.  It is slow and runs only when a pair tensor was changed
+// after the library had seen it in order.
+template <typename E, int NT>
+__device__ __forceinline__ void scanAllPairsForTile(const typename E::storage *A, int Q,
+                                                    const SegmentSource &src, int K, int r_begin,
+                                                    int r_end, int C, int col0, float *acc,
+                                                    int acc_stride) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const typename E::storage *W = static_cast<const typename E::storage *>(src.W);
+  for (int k = 0; k < K; ++k) {
+    const int n = src.counts.n[k];
+    const int32_t *row_list = src.pairs + ((size_t)k * 2 + src.row_col) * src.L;
+    const int32_t *src_list = src.pairs + ((size_t)k * 2 + src.src_col) * src.L;
+    for (int p0 = 0; p0 < n; p0 += NT) {
+      const int p = p0 + tid;
+      int r = -1, g = -1;
+      if (p < n) {
+        r = row_list[p];
+        g = src_list[p];
+      }
+      const bool hit = r >= r_begin && r < r_end && (unsigned)g < (unsigned)src.n_src;
+      unsigned long long m = __ballot(hit);
+      while (m) {
+        const int from = __ffsll((long long)m) - 1;
+        m &= m - 1;
+        const int rr = __shfl(r, from, kWave) - r_begin;
+        const typename E::storage *a = A + (size_t)__shfl(g, from, kWave) * Q;
+        for (int c = lane; c < C; c += kWave) {
+          const typename E::storage *w = W + (size_t)k * src.sK + (size_t)(col0 + c) * src.sC;
+          float dot = 0.f;
+          for (int q = 0; q < Q; ++q) dot += E::load(a + q) * E::load(w + (size_t)q * src.sQ);
+          atomicAdd(&acc[rr * acc_stride + c], dot);
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// One launch in front of a gather kernel that reads pair lists: the first
+// `pack_blocks` workgroups repack the filter into operand fragments (as
+// fillMapPackFilter does), the others walk the pair lists, one pair per lane, and
+//  * check what the gather kernel relies on: result rows in range and strictly
+//    ascending inside the offset, gathered rows in range.  A violation stores `ticket`
+//    in *verdict (a value no earlier call used, so the word needs no clearing);
+//  * write the cut table: pair p is the first pair of every tile after its
+//    predecessor's tile up to its own, and the last pair of an offset closes the
+//    remaining tiles with the pair count (an offset without pairs gets one workgroup
+//    that closes all its tiles with 0).  A lane with more than a few tiles to close
+//    hands them to the whole wave.
+template <typename E>
+__global__ __launch_bounds__(256) void packFilterCutPairLists(
+    const typename E::storage *W, int64_t sK, int64_t sQ, int64_t sC, int K, int Q, int C,
+    typename E::storage *packed, int pack_blocks, const int32_t *pairs, int L, OffsetCounts inl,
+    OffsetBlocks blocks, int row_col, int src_col, int R, int n_src, int tile_shift, int n_tiles,
+    int32_t *cuts, unsigned long long *verdict, unsigned long long ticket) {
+  if ((int)blockIdx.x < pack_blocks) {
+    constexpr int VEC = E::kVec, CHUNK = E::kChunk;
+    const int chunks = (Q + CHUNK - 1) / CHUNK;
+    const size_t total = (size_t)K * (C / 16) * chunks * 64;
+    for (size_t t = (size_t)blockIdx.x * 256 + threadIdx.x; t < total;
+         t += (size_t)pack_blocks * 256) {
+      const int lane = (int)(t & 63);
+      size_t rest = t >> 6;
+      const int kb = (int)(rest % chunks);
+      rest /= chunks;
+      const int nb = (int)(rest % (C / 16));
+      const int k = (int)(rest / (C / 16));
+      const int c = nb * 16 + (lane & 15);
+      const int qb = kb * CHUNK + VEC * (lane >> 4);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        packed[t * VEC + e] =
+            qb + e < Q ? W[(size_t)k * sK + (size_t)(qb + e) * sQ + (size_t)c * sC] : typename E::storage(0);
+    }
+    return;
+  }
+  const int b = (int)blockIdx.x - pack_blocks;
+  int lo = 0, hi = K - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (blocks.first[mid] <= b) lo = mid; else hi = mid - 1;
+  }
+  const int k = lo;
+  const int n = inl.n[k];
+  const int p = (b - blocks.first[k]) * 256 + (int)threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const bool live = p < n;
+  const int32_t *row_list = pairs + ((size_t)k * 2 + row_col) * L;
+  const int32_t *src_list = pairs + ((size_t)k * 2 + src_col) * L;
+  int r = 0, prev = -1, s = 0;
+  if (live) {
+    r = row_list[p];
+    s = src_list[p];
+    if (p > 0) prev = row_list[p - 1];
+  }
+  const bool ok = (unsigned)r < (unsigned)R && (unsigned)s < (unsigned)n_src && r > prev;
+  if (live && !ok) *verdict = ticket;
+  // tiles (t_lo .. t_mid] open at p, tiles (t_mid .. n_tiles] close with n; clamped so
+  // that a list out of order, whose table nobody reads, still writes inside the table
+  int t_mid = r >> tile_shift;
+  t_mid = t_mid < 0 ? 0 : (t_mid > n_tiles - 1 ? n_tiles - 1 : t_mid);
+  int t_lo = p == 0 ? -1 : (prev >> tile_shift);
+  t_lo = t_lo < -1 ? -1 : (t_lo > t_mid ? t_mid : t_lo);
+  int32_t *row_cuts = cuts + (size_t)k * (n_tiles + 1);
+  // job 0: value p over (t_lo, t_mid]; job 1 (last pair only): value n over (t_mid, n_tiles]
+#pragma unroll
+  for (int job = 0; job < 2; ++job) {
+    // (an offset without pairs has one workgroup, whose first lane closes all tiles with 0)
+    const bool empty_offset = n == 0 && threadIdx.x == 0;
+    const int first = empty_offset ? 0 : (job == 0 ? t_lo + 1 : t_mid + 1);
+    const int last = job == 0 ? t_mid : n_tiles;
+    const int value = job == 0 ? p : n;
+    const bool mine = ((live && (job == 0 || p == n - 1)) || (empty_offset && job == 1)) && first <= last;
+    const bool wide = mine && last - first >= 4;
+    if (mine && !wide)
+      for (int t = first; t <= last; ++t) row_cuts[t] = value;
+    unsigned long long m = __ballot(wide);
+    while (m) {
+      const int from = __ffsll((long long)m) - 1;
+      m &= m - 1;
+      const int f = __shfl(first, from, kWave), l = __shfl(last, from, kWave);
+      const int v = __shfl(value, from, kWave);
+      for (int t = f + lane; t <= l; t += kWave) row_cuts[t] = v;
+    }
+  }
+}
+
 constexpr int mfmaTileRows(int C) {
   // fp32 accumulator tile of about 34 KiB
   return C <= 64 ? 128 : 64;
@@ -341,12 +504,11 @@ constexpr int mfmaBatchBlocks(int elem_bytes, int Q, int C) {
 //       the accumulator row of that pair with one 16-byte read-modify-write.
 //       Lanes past the end of a short block repeat its first entry and
 //       accumulate into a spare row.
-template <typename E, int Q, int C>
+template <typename E, int Q, int C, typename SRC>
 __global__ __launch_bounds__(mfmaThreads(C)) __attribute__((amdgpu_waves_per_eu(mfmaWavesPerSimd((int)sizeof(typename E::storage), Q, C),
                                    mfmaWavesPerSimd((int)sizeof(typename E::storage), Q, C))))
 void gatherConvMfma(const typename E::storage *A, const typename E::storage *packedW,
-                    const int32_t *map, int R, int K, int ldc, int32_t *filled,
-                    typename E::storage *result) {
+                    SRC source, int R, int K, int ldc, typename E::storage *result) {
   typedef typename E::vec8 vec8;
   typedef typename E::storage S;
   constexpr int NB = mfmaColBlocksPerWave(C);
@@ -391,13 +553,27 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
   const int r0 = tile * TR;
   if (r0 >= R) {
-    if (tid == 0 && blockIdx.y == 0) filled[blockIdx.x] = 0;
+    if constexpr (!SRC::kSegments) {
+      if (tid == 0 && blockIdx.y == 0) source.filled[blockIdx.x] = 0;
+    }
     return;
   }
   int slots = 0;  // filled map slots of this tile
   const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
   for (int i = tid; i < (TR + 1) * ACC_STRIDE; i += NT) s_acc[i] = 0.f;
+
+  // Pair lists that turned out not to be in order (a caller who changed the tensor
+  // behind the library's back): the tile collects its pairs by reading all of them.
+  bool in_order = true;
+  if constexpr (SRC::kSegments) {
+    in_order = *source.verdict != source.ticket;
+    if (!in_order) {
+      __syncthreads();
+      scanAllPairsForTile<E, NT>(A, Q, source, K, r0, r0 + TR < R ? r0 + TR : R, C, blockIdx.y * C,
+                                 s_acc, ACC_STRIDE);
+    }
+  }
 
   // per-lane constants of the multiply phase
   const char *a_bytes = reinterpret_cast<const char *>(A);
@@ -411,39 +587,85 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   char *acc_lane = reinterpret_cast<char *>(s_acc) + (wave * 16 * NB + 4 * quad) * 4;
   const char *stage_lane = s_stage + quad * 16;
 
-  for (int kc = 0; kc < K; kc += KC) {
+  for (int kc = 0; kc < (in_order ? K : 0); kc += KC) {
     const int kn = (K - kc) < KC ? (K - kc) : KC;
-    // A: map entries of this wave's offsets; unconditional loads from clamped
-    // addresses keep all of them in flight (offsets without pairs hold -1).
-    int idx[KPW][NSEG];
-#pragma unroll
-    for (int j = 0; j < KPW; ++j) {
-      const int kk = wave + j * ALLW;
-      const int k_safe = kk < kn ? kc + kk : kc;
-#pragma unroll
-      for (int seg = 0; seg < NSEG; ++seg) {
-        const int r = r0 + seg * 64 + lane;
-        idx[j][seg] = map[(size_t)k_safe * R + (r < R ? r : R - 1)];
+    // A: the pairs of this wave's offsets; unconditional loads from clamped
+    // addresses keep all of them in flight.
+    int idx[KPW][NSEG];   // partner row, or -1
+    int own[KPW][NSEG];   // result row inside the tile (pair lists only)
+    if constexpr (SRC::kSegments) {
+      // lane 2j + e fetches cut e of this wave's j-th offset
+      int cut = 0;
+      {
+        const int kk = wave + (lane >> 1) * ALLW;
+        if ((lane >> 1) < KPW && kk < kn)
+          cut = source.cuts[(size_t)(kc + kk) * source.cut_stride + tile + (lane & 1)];
       }
-    }
-    // Pinning the loaded values here keeps the loads above unconditional and all
-    // in flight; selecting on them directly lets the compiler branch around
-    // every single load and wait for it.
+      int first[KPW], count[KPW];
 #pragma unroll
-    for (int j = 0; j < KPW; ++j)
+      for (int j = 0; j < KPW; ++j) {
+        const int kk = wave + j * ALLW;
+        first[j] = __shfl(cut, 2 * j, kWave);
+        const int end = __shfl(cut, 2 * j + 1, kWave);
+        int c = end - first[j];
+        c = c < 0 ? 0 : (c > TR ? TR : c);
+        count[j] = (kk < kn && source.counts.n[kk < kn ? kc + kk : kc] > 0) ? c : 0;
+        const int k_safe = kk < kn ? kc + kk : kc;
+        const int32_t *row_list = source.pairs + ((size_t)k_safe * 2 + source.row_col) * source.L;
+        const int32_t *src_list = source.pairs + ((size_t)k_safe * 2 + source.src_col) * source.L;
 #pragma unroll
-      for (int seg = 0; seg < NSEG; ++seg) asm volatile("" : "+v"(idx[j][seg]));
-#pragma unroll
-    for (int j = 0; j < KPW; ++j) {
-      const int kk = wave + j * ALLW;
-      int c = 0;
-#pragma unroll
-      for (int seg = 0; seg < NSEG; ++seg) {
-        const int r = r0 + seg * 64 + lane;
-        if (!(kk < kn && r < R)) idx[j][seg] = -1;
-        c += __popcll(__ballot(idx[j][seg] >= 0));
+        for (int seg = 0; seg < NSEG; ++seg) {
+          int p = first[j] + seg * 64 + lane;
+          p = p < 0 ? 0 : (p < source.L ? p : source.L - 1);
+          own[j][seg] = row_list[p];
+          idx[j][seg] = src_list[p];
+        }
       }
-      if (lane == 0 && kk < KC) s_cnt[kk] = c;
+#pragma unroll
+      for (int j = 0; j < KPW; ++j)
+#pragma unroll
+        for (int seg = 0; seg < NSEG; ++seg) asm volatile("" : "+v"(idx[j][seg]), "+v"(own[j][seg]));
+#pragma unroll
+      for (int j = 0; j < KPW; ++j) {
+        const int kk = wave + j * ALLW;
+#pragma unroll
+        for (int seg = 0; seg < NSEG; ++seg) {
+          if (seg * 64 + lane >= count[j]) idx[j][seg] = -1;
+          own[j][seg] = (own[j][seg] - r0) & (TR - 1);
+        }
+        if (lane == 0 && kk < KC) s_cnt[kk] = count[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < KPW; ++j) {
+        const int kk = wave + j * ALLW;
+        const int k_safe = kk < kn ? kc + kk : kc;
+#pragma unroll
+        for (int seg = 0; seg < NSEG; ++seg) {
+          const int r = r0 + seg * 64 + lane;
+          idx[j][seg] = source.map[(size_t)k_safe * R + (r < R ? r : R - 1)];
+          own[j][seg] = seg * 64 + lane;
+        }
+      }
+      // Pinning the loaded values here keeps the loads above unconditional and all
+      // in flight; selecting on them directly lets the compiler branch around
+      // every single load and wait for it.
+#pragma unroll
+      for (int j = 0; j < KPW; ++j)
+#pragma unroll
+        for (int seg = 0; seg < NSEG; ++seg) asm volatile("" : "+v"(idx[j][seg]));
+#pragma unroll
+      for (int j = 0; j < KPW; ++j) {
+        const int kk = wave + j * ALLW;
+        int c = 0;
+#pragma unroll
+        for (int seg = 0; seg < NSEG; ++seg) {
+          const int r = r0 + seg * 64 + lane;
+          if (!(kk < kn && r < R)) idx[j][seg] = -1;
+          c += __popcll(__ballot(idx[j][seg] >= 0));
+        }
+        if (lane == 0 && kk < KC) s_cnt[kk] = c;
+      }
     }
     __syncthreads();
     // every wave scans the counts: entries and blocks in front of each offset
@@ -464,8 +686,7 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
       for (int seg = 0; seg < NSEG; ++seg) {
         const unsigned long long b = __ballot(idx[j][seg] >= 0);
         if (idx[j][seg] >= 0)
-          s_ent[base + __popcll(b & lt_mask)] =
-              ((uint32_t)idx[j][seg] << 8) | (uint32_t)(seg * 64 + lane);
+          s_ent[base + __popcll(b & lt_mask)] = ((uint32_t)idx[j][seg] << 8) | (uint32_t)own[j][seg];
         base += __popcll(b);
       }
     }
@@ -616,7 +837,244 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
     *reinterpret_cast<uint4 *>(result + (size_t)(r0 + rr) * ldc + col_group * C + c0) =
         *reinterpret_cast<const uint4 *>(tmp);
   }
-  if (tid == 0 && blockIdx.y == 0) filled[blockIdx.x] = slots;
+  if constexpr (!SRC::kSegments) {
+    if (tid == 0 && blockIdx.y == 0) source.filled[blockIdx.x] = slots;
+  }
+}
+
+// ---- MFMA gather convolution, one free-running wavefront per tile ---------------------
+//
+// The kernel above spends a tile's life waiting: cut positions, then pairs, then
+// gathered rows round by round behind barriers, then a filter slice from L2 for every
+// thinly filled offset, with two tiles a CU to overlap it all.  For results of up to 32
+// columns a tile of 128 result rows fits a single wavefront that never meets a barrier:
+// its fp32 accumulator tile and one 16-row stage slot are all the LDS it needs, so
+// seven tiles share a CU, a layer of a few hundred thousand rows is resident at once,
+// and what the wave waits for is hidden by its own requests running ahead in register
+// rings:
+//   unit      = up to 16 pairs of one offset, walked in offset order;
+//   t + 10    the unit's pairs are requested (lane l: pair l % 16);
+//   t + 5     its gathered rows (row-contiguous 16-byte pieces) and the offset's filter
+//             fragments are requested;
+//   t         rows go through the LDS slot (written row-major, read as MFMA operand
+//             fragments), all column blocks are multiplied and the products added to the
+//             pairs' fp32 rows, read from and written back to LDS 16 bytes a lane.
+// Requests are unconditional (clamped addresses) so that the number of loads in flight
+// at every point of the loop is fixed.  It reads pair lists only (SegmentSource).
+// Measured against the kernel above on 120 000 rows with 2.2 pairs a row: 32 -> 32
+// channels 26 us against 32 us; at 64 result columns (two waves a tile, 32 columns
+// each) it loses, 43 us against 41 us, and is not used.
+constexpr int kWaveTileRows = 128;
+constexpr bool waveKernelShape(int elem_bytes, int Q, int C) {
+  const int chunk = elem_bytes == 4 ? 16 : 32;
+  return C <= 32 && Q * elem_bytes <= 256 && ((Q + chunk - 1) / chunk) * (C / 16) <= 8;
+}
+template <typename E, int Q, int C>
+__global__ __launch_bounds__(64) void gatherConvWave(
+    const typename E::storage *A, const typename E::storage *packedW, SegmentSource source, int R,
+    int K, typename E::storage *result) {
+  typedef typename E::vec8 vec8;
+  typedef typename E::storage S;
+  constexpr int NB = C / 16;                            // column blocks
+  constexpr int KB = (Q + E::kChunk - 1) / E::kChunk;
+  constexpr bool kPartialFragment = Q < E::kChunk;
+  constexpr int TR = kWaveTileRows;
+  constexpr int ACC_STRIDE = C + 4;
+  constexpr int ROW_BYTES = Q * (int)sizeof(S);
+  constexpr int STAGE_STRIDE = ROW_BYTES + 16;
+  constexpr int PPR = ROW_BYTES / 16;                   // 16-byte pieces per row
+  constexpr int RL = (16 * PPR + 63) / 64;              // wave-loads per unit of rows
+  constexpr int EPL = 64 / PPR >= 16 ? 16 : 64 / PPR;   // rows per wave-load
+  constexpr int NE = 12;   // pair ring (units) = units per trip of the unrolled loop
+  constexpr int NR = 6;    // row and filter ring (units)
+  constexpr int AHEAD_ROWS = 5;
+  constexpr int AHEAD_PAIRS = 10;
+  static_assert(PPR >= 2 && PPR <= 32 && AHEAD_ROWS < NR && AHEAD_PAIRS < NE && NE % NR == 0, "ring sizes");
+  constexpr int ACC_QUADS = (TR + 1) * ACC_STRIDE / 4;
+
+  __shared__ __attribute__((aligned(16))) float s_acc[(TR + 1) * ACC_STRIDE];
+  __shared__ __attribute__((aligned(16))) char s_stage[16 * STAGE_STRIDE];
+
+  const int lane = threadIdx.x;
+  const int tiles_per_xcd = gridDim.x >> 3;  // neighbouring tiles on one XCD
+  const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
+  const int r0 = tile * TR;
+  if (r0 >= R) return;
+
+  // this tile's piece of every offset's list (lane l: offsets l and l + 64)
+  const unsigned long long verdict = *source.verdict;
+  int piece_first[2] = {0, 0}, piece_count[2] = {0, 0};
+#pragma unroll
+  for (int o = 0; o < 2; ++o) {
+    const int k = lane + 64 * o;
+    if (k < K) {
+      const int32_t *c = source.cuts + (size_t)k * source.cut_stride + tile;
+      piece_first[o] = c[0];
+      piece_count[o] = c[1];
+    }
+  }
+#pragma unroll 8
+  for (int i = lane; i < ACC_QUADS; i += 64)
+    reinterpret_cast<float4v *>(s_acc)[i] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  constexpr int VALS = 16 / (int)sizeof(S);
+  auto write_out = [&]() {
+    for (int i = lane; i < TR * C / VALS; i += 64) {
+      const int rr = i / (C / VALS);
+      const int c0 = (i % (C / VALS)) * VALS;
+      if (r0 + rr >= R) break;
+      S tmp[VALS];
+#pragma unroll
+      for (int e = 0; e < VALS; ++e) E::store(&tmp[e], s_acc[rr * ACC_STRIDE + c0 + e]);
+      *reinterpret_cast<uint4 *>(result + (size_t)(r0 + rr) * C + c0) = *reinterpret_cast<const uint4 *>(tmp);
+    }
+  };
+  if (verdict == source.ticket) {
+    // lists out of order: every pair of every offset is looked at
+    scanAllPairsForTile<E, 64>(A, Q, source, K, r0, r0 + TR < R ? r0 + TR : R, C, 0, s_acc, ACC_STRIDE);
+    write_out();
+    return;
+  }
+  unsigned long long has[2];
+#pragma unroll
+  for (int o = 0; o < 2; ++o) {
+    int c = piece_count[o] - piece_first[o];
+    c = c < 0 ? 0 : (c > TR ? TR : c);
+    if (lane + 64 * o >= K) c = 0;
+    piece_count[o] = c;
+    has[o] = __ballot(c > 0);
+  }
+  // first offset above `after` that has pairs in this tile, or 128
+  auto next_offset = [&](int after) {
+    const int from = after + 1;
+    const unsigned long long lo = from < 64 ? (has[0] & (~0ull << from)) : 0ull;
+    if (lo) return (int)__builtin_ctzll(lo);
+    const unsigned long long hi = from <= 64 ? has[1] : (from < 128 ? (has[1] & (~0ull << (from - 64))) : 0ull);
+    if (hi) return 64 + (int)__builtin_ctzll(hi);
+    return 128;
+  };
+  auto of = [&](const int (&v)[2], int k) {
+    const int a = __builtin_amdgcn_readlane(v[0], k & 63), b = __builtin_amdgcn_readlane(v[1], k & 63);
+    return k < 64 ? a : b;
+  };
+  // the walk over units: offset, first pair and pair count of the unit a request is made for
+  int walk_k = next_offset(-1);
+  int walk_left = walk_k < 128 ? of(piece_count, walk_k) : 0;
+  int walk_at = walk_k < 128 ? of(piece_first, walk_k) : 0;
+  int unit_k[NE], unit_at[NE], unit_n[NE];
+  auto next_unit = [&](int &k, int &at, int &n) {
+    k = walk_k;
+    at = walk_at;
+    n = walk_left < 16 ? walk_left : 16;
+    if (walk_k < 128) {
+      walk_left -= n;
+      walk_at += n;
+      if (walk_left <= 0) {
+        walk_k = next_offset(walk_k);
+        walk_left = walk_k < 128 ? of(piece_count, walk_k) : 0;
+        walk_at = walk_k < 128 ? of(piece_first, walk_k) : 0;
+      }
+    }
+  };
+
+  const char *a_bytes = reinterpret_cast<const char *>(A);
+  const char *b_base = reinterpret_cast<const char *>(packedW) + (size_t)lane * 16;
+  const uint32_t kBytesPerOffset = (uint32_t)(C / 16) * KB * 64 * 16;
+  const int pair = lane & 15;
+  const int quad = lane >> 4;
+  char *acc_lane = reinterpret_cast<char *>(s_acc) + 4 * quad * 4;
+  char *stage = s_stage;
+
+  int pair_row[NE], pair_src[NE];
+  u32x4 rows[NR][RL];
+  vec8 w[NR][KB][NB];
+
+  auto request_pairs = [&](int slot) {
+    next_unit(unit_k[slot], unit_at[slot], unit_n[slot]);
+    const int k = unit_k[slot] < K ? unit_k[slot] : 0;
+    int p = unit_at[slot] + pair;
+    p = p < 0 ? 0 : (p < source.L ? p : source.L - 1);
+    const int32_t *list = source.pairs + (size_t)k * 2 * source.L;
+    pair_row[slot] = list[(size_t)source.row_col * source.L + p];
+    pair_src[slot] = list[(size_t)source.src_col * source.L + p];
+    // The requests must stay where they are written, far ahead of their use: nothing that
+    // may touch memory moves across this point, so the compiler cannot sink the loads
+    // towards the instructions that consume them (and no register is named, so nothing
+    // is waited for here).
+    asm volatile("" ::: "memory");
+  };
+  auto request_rows = [&](int pslot, int rslot) {
+    const int n = unit_n[pslot];
+    const int k = unit_k[pslot] < K ? unit_k[pslot] : 0;
+#pragma unroll
+    for (int h = 0; h < RL; ++h) {
+      const int e = lane / PPR + EPL * h;  // which pair's row this lane fetches a piece of
+      int g = __shfl(pair_src[pslot], e & 15, kWave);
+      if (e >= n || (unsigned)g >= (unsigned)source.n_src) g = 0;
+      rows[rslot][h] = *reinterpret_cast<const u32x4 *>(a_bytes + (size_t)g * ROW_BYTES + (lane % PPR) * 16);
+    }
+    const char *bk = b_base + (size_t)k * kBytesPerOffset;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        w[rslot][kb][nb] = *reinterpret_cast<const vec8 *>(bk + (nb * KB + kb) * 1024);
+    asm volatile("" ::: "memory");
+  };
+  auto multiply = [&](int pslot, int rslot) {
+    const int n = unit_n[pslot];
+    const int acc_row = pair < n ? ((pair_row[pslot] - r0) & (TR - 1)) : TR;
+    char *dst = acc_lane + acc_row * (ACC_STRIDE * 4);
+    // (products summed from zero, then added: the arithmetic of the kernel above, so the
+    // two give the same bits)
+    float4v acc[NB], prod[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      acc[nb] = *reinterpret_cast<float4v *>(dst + nb * 64);
+      prod[nb] = float4v{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int h = 0; h < RL; ++h) {
+      const int e = lane / PPR + EPL * h;
+      if (16 * PPR >= 64 || lane < 16 * PPR)
+        *reinterpret_cast<u32x4 *>(stage + e * STAGE_STRIDE + (lane % PPR) * 16) = rows[rslot][h];
+    }
+    vec8 afr[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+      afr[kb] = *reinterpret_cast<const vec8 *>(stage + pair * STAGE_STRIDE + kb * 64 + quad * 16);
+    if constexpr (kPartialFragment) {
+      if (quad * E::kVec >= Q) afr[0] = vec8{};
+    }
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) prod[nb] = E::mfma(w[rslot][kb][nb], afr[kb], prod[nb]);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      acc[nb] += prod[nb];
+      *reinterpret_cast<float4v *>(dst + nb * 64) = acc[nb];
+    }
+  };
+
+#pragma unroll
+  for (int u = 0; u < AHEAD_PAIRS; ++u) request_pairs(u);
+#pragma unroll
+  for (int u = 0; u < AHEAD_ROWS; ++u) request_rows(u, u);
+  bool more = unit_k[0] < 128;
+  while (more) {
+#pragma unroll
+    for (int u = 0; u < NE; ++u) {
+      // unit t = t0 + u: pair slot u, row slot u % NR
+      if (more) {
+        request_pairs((u + AHEAD_PAIRS) % NE);
+        request_rows((u + AHEAD_ROWS) % NE, (u + AHEAD_ROWS) % NR);
+        multiply(u, u % NR);
+        more = unit_k[(u + 1) % NE] < 128;
+      }
+    }
+  }
+  write_out();
 }
 
 // ---- MFMA gather convolution for dense rulebooks -------------------------------
@@ -643,10 +1101,10 @@ constexpr int kDenseDepth = 4;   // stage buffers: offsets i .. i+3 are resident
 constexpr int kDenseRowSplit = 2;  // waves along the rows of a tile
 constexpr int denseThreads(int C) { return 64 * (C / 32) * kDenseRowSplit; }
 
-template <typename E, int Q, int C>
+template <typename E, int Q, int C, typename SRC>
 __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
-    const typename E::storage *A, const typename E::storage *packedW, const int32_t *map, int R,
-    int K, int ldc, int32_t *filled, typename E::storage *result) {
+    const typename E::storage *A, const typename E::storage *packedW, SRC source, int R,
+    int K, int ldc, typename E::storage *result) {
   typedef typename E::vec8 vec8;
   typedef typename E::storage S;
   constexpr int NB = 2;                      // 16-column blocks per wave
@@ -681,10 +1139,33 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
   const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
   const int r0 = tile * TR;
   if (r0 >= R) {
-    if (tid == 0 && blockIdx.y == 0) filled[blockIdx.x] = 0;
+    if constexpr (!SRC::kSegments) {
+      if (tid == 0 && blockIdx.y == 0) source.filled[blockIdx.x] = 0;
+    }
     return;
   }
   const int col_group = blockIdx.y;
+  if constexpr (SRC::kSegments) {
+    if (*source.verdict == source.ticket) {
+      // pair lists out of order: fp32 rows in the stage memory, as many columns at a
+      // time as fit, every pair looked at by every workgroup
+      float *acc = reinterpret_cast<float *>(&s_stage[0][0]);
+      constexpr int CP = D * ROW_BYTES / 4 >= C ? C : 64;  // columns per pass
+      static_assert(D * ROW_BYTES / 4 >= 64, "a pass of 64 columns fits the stage");
+      const int r_end = r0 + TR < R ? r0 + TR : R;
+      for (int c0 = 0; c0 < C; c0 += CP) {
+        for (int i = tid; i < TR * CP; i += WAVES * 64) acc[i] = 0.f;
+        __syncthreads();
+        scanAllPairsForTile<E, WAVES * 64>(A, Q, source, K, r0, r_end, CP, col_group * C + c0, acc, CP);
+        for (int i = tid; i < TR * CP; i += WAVES * 64) {
+          const int rr = i / CP, c = i % CP;
+          if (r0 + rr < R) E::store(result + (size_t)(r0 + rr) * ldc + col_group * C + c0 + c, acc[i]);
+        }
+        __syncthreads();
+      }
+      return;
+    }
+  }
   const int pair = lane & 15;
   const int quad = lane >> 4;
   const char *a_bytes = reinterpret_cast<const char *>(A);
@@ -705,12 +1186,32 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
     const int kn = (K - kc) < KC ? (K - kc) : KC;
     __syncthreads();  // the chunk before is finished with s_map and the stage
     for (int kk = wave; kk < kn; kk += WAVES) {
-      const int r = r0 + lane;
-      const int v = r < R ? map[(size_t)(kc + kk) * R + r] : -1;
-      s_map[kk][lane] = v;
-      const unsigned long long any = __ballot(v >= 0);
-      if (lane == 0) s_has[kk] = any != 0ull;
-      slots += __popcll(any);
+      if constexpr (SRC::kSegments) {
+        // the offset's pairs of this tile are one piece of its list: lane l of the
+        // piece writes its partner at the result row's position (same wave, in order
+        // behind the clearing store)
+        s_map[kk][lane] = -1;
+        int cut = 0;
+        if (lane < 2) cut = source.cuts[(size_t)(kc + kk) * source.cut_stride + tile + lane];
+        const int first = __shfl(cut, 0, kWave);
+        int count = __shfl(cut, 1, kWave) - first;
+        count = count < 0 ? 0 : (count > TR ? TR : count);
+        if (lane < count) {
+          int p = first + lane;
+          p = p < 0 ? 0 : (p < source.L ? p : source.L - 1);
+          const int32_t *list = source.pairs + (size_t)(kc + kk) * 2 * source.L;
+          const int own = (list[(size_t)source.row_col * source.L + p] - r0) & (TR - 1);
+          s_map[kk][own] = list[(size_t)source.src_col * source.L + p];
+        }
+        if (lane == 0) s_has[kk] = count > 0;
+      } else {
+        const int r = r0 + lane;
+        const int v = r < R ? source.map[(size_t)(kc + kk) * R + r] : -1;
+        s_map[kk][lane] = v;
+        const unsigned long long any = __ballot(v >= 0);
+        if (lane == 0) s_has[kk] = any != 0ull;
+        slots += __popcll(any);
+      }
     }
     __syncthreads();
     if (wave == 0) {
@@ -817,14 +1318,16 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
         *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(tmp);
     }
   }
-  // s_has is free again: the waves' slot counts meet there
-  __syncthreads();
-  if (lane == 0) s_has[wave] = slots;
-  __syncthreads();
-  if (tid == 0 && blockIdx.y == 0) {
-    int all = 0;
-    for (int w = 0; w < WAVES; ++w) all += s_has[w];
-    filled[blockIdx.x] = all;
+  if constexpr (!SRC::kSegments) {
+    // s_has is free again: the waves' slot counts meet there
+    __syncthreads();
+    if (lane == 0) s_has[wave] = slots;
+    __syncthreads();
+    if (tid == 0 && blockIdx.y == 0) {
+      int all = 0;
+      for (int w = 0; w < WAVES; ++w) all += s_has[w];
+      source.filled[blockIdx.x] = all;
+    }
   }
 }
 
@@ -1473,7 +1976,17 @@ GatherDims gatherDims(const ConvProblem &p, GatherDirection dir) {
   return d;
 }
 
+// The list kernels take the per-offset tables by value and are asked for only when the
+// caller has reason to believe the result-row column in order; a row map announced for
+// the call is used instead.
+bool listsUsable(const ConvProblem &p, const GatherDims &d) {
+  (void)d;
+  return p.lists_in_order && p.K <= kMaxInlineK && p.row_map == nullptr;
+}
+
 struct GatherWorkspace {
+  int32_t *cuts = nullptr;              // [K, tiles + 1] cut positions of the pair lists
+  unsigned long long *verdict = nullptr;
   int32_t *dev_counts = nullptr;
   int32_t *filled = nullptr;  // map slots the gather kernel's workgroups found filled
   int32_t *shadow = nullptr;  // repairLostPairs' scratch, touched only when pairs collide
@@ -1494,6 +2007,11 @@ GatherWorkspace carveGather(const ConvProblem &p, const GatherDims &d, void *bas
     return r;
   };
   if (p.K > kMaxInlineK) ws.dev_counts = reinterpret_cast<int32_t *>(take((size_t)p.K * 4));
+  if (p.K <= kMaxInlineK) {
+    // tiles of the narrowest kind (64 rows) bound the table
+    ws.cuts = reinterpret_cast<int32_t *>(take((size_t)p.K * ((size_t)d.R / 64 + 2) * 4));
+    ws.verdict = reinterpret_cast<unsigned long long *>(take(8));
+  }
   ws.filled = reinterpret_cast<int32_t *>(take(((size_t)d.R / 32 + 16) * 4));
   ws.shadow = reinterpret_cast<int32_t *>(take((size_t)d.R * 4));
   ws.pool_row = reinterpret_cast<int32_t *>(take((size_t)kRepairPoolRows * 4));
@@ -1552,13 +2070,6 @@ int mfmaTileCols(const ConvProblem &p, const GatherDims &d) {
   return per_tile_offset < 8.0 ? 64 : 128;
 }
 
-// The row map and, per workgroup of a gather kernel (blockIdx.x), the number of slots it
-// found filled in its tile.
-struct RowMap {
-  const int32_t *entries;
-  int32_t *filled;
-};
-
 // Workgroups along x: tiles rounded up to a multiple of the XCD count.
 int mfmaGridX(int R, int tile_cols) {
   const int tr = mfmaTileRows(tile_cols);
@@ -1566,45 +2077,80 @@ int mfmaGridX(int R, int tile_cols) {
 }
 int denseGridX(int R) { return ((R + kDenseTileRows - 1) / kDenseTileRows + 7) / 8 * 8; }
 
-template <typename E, int Q, int C>
+template <typename E, int Q, int C, typename SRC>
 void launchMfmaInstance(const LaunchCtx &lc, const void *A, const void *packed,
-                        RowMap map, int R, int K, int ldc, void *result) {
+                        const SRC &source, int R, int K, int ldc, void *result) {
   constexpr int NT = mfmaThreads(C);
-  constexpr int TR = mfmaTileRows(C);
-  static_assert(TR == mfmaTileRows(C), "grid helper and kernel agree");
   const dim3 grid(mfmaGridX(R, C), ldc / C);
   lc.begin("gatherConvMfma");
-  gatherConvMfma<E, Q, C><<<grid, NT, 0, lc.stream>>>(
+  gatherConvMfma<E, Q, C, SRC><<<grid, NT, 0, lc.stream>>>(
       static_cast<const typename E::storage *>(A),
-      static_cast<const typename E::storage *>(packed), map.entries, R, K, ldc, map.filled,
+      static_cast<const typename E::storage *>(packed), source, R, K, ldc,
       static_cast<typename E::storage *>(result));
   lc.end();
 }
 
 // `tile_cols` result columns per workgroup out of C: a narrower tile has more
 // rows, so sparse rulebooks fill their 16-pair blocks better.
-template <typename E, int Q>
+template <typename E, int Q, typename SRC>
 void launchMfmaByC(const LaunchCtx &lc, int C, int tile_cols, const void *A, const void *packed,
-                   RowMap map, int R, int K, void *result) {
+                   const SRC &source, int R, int K, void *result) {
   switch (tile_cols) {
-    case 16: launchMfmaInstance<E, Q, 16>(lc, A, packed, map, R, K, C, result); break;
-    case 32: launchMfmaInstance<E, Q, 32>(lc, A, packed, map, R, K, C, result); break;
-    case 64: launchMfmaInstance<E, Q, 64>(lc, A, packed, map, R, K, C, result); break;
-    case 128: launchMfmaInstance<E, Q, 128>(lc, A, packed, map, R, K, C, result); break;
+    case 16: launchMfmaInstance<E, Q, 16, SRC>(lc, A, packed, source, R, K, C, result); break;
+    case 32: launchMfmaInstance<E, Q, 32, SRC>(lc, A, packed, source, R, K, C, result); break;
+    case 64: launchMfmaInstance<E, Q, 64, SRC>(lc, A, packed, source, R, K, C, result); break;
+    case 128: launchMfmaInstance<E, Q, 128, SRC>(lc, A, packed, source, R, K, C, result); break;
     default: break;
   }
 }
 
-template <typename E>
+template <typename E, typename SRC>
 void launchMfma(const LaunchCtx &lc, int Q, int C, int tile_cols, const void *A, const void *packed,
-                RowMap map, int R, int K, void *result) {
+                const SRC &source, int R, int K, void *result) {
   switch (Q) {
-    case 16: launchMfmaByC<E, 16>(lc, C, tile_cols, A, packed, map, R, K, result); break;
-    case 32: launchMfmaByC<E, 32>(lc, C, tile_cols, A, packed, map, R, K, result); break;
-    case 64: launchMfmaByC<E, 64>(lc, C, tile_cols, A, packed, map, R, K, result); break;
-    case 128: launchMfmaByC<E, 128>(lc, C, tile_cols, A, packed, map, R, K, result); break;
+    case 16: launchMfmaByC<E, 16, SRC>(lc, C, tile_cols, A, packed, source, R, K, result); break;
+    case 32: launchMfmaByC<E, 32, SRC>(lc, C, tile_cols, A, packed, source, R, K, result); break;
+    case 64: launchMfmaByC<E, 64, SRC>(lc, C, tile_cols, A, packed, source, R, K, result); break;
+    case 128: launchMfmaByC<E, 128, SRC>(lc, C, tile_cols, A, packed, source, R, K, result); break;
     default: break;
   }
+}
+
+template <typename E, int Q, int C>
+void launchWaveInstance(const LaunchCtx &lc, const void *A, const void *packed,
+                        const SegmentSource &source, int R, int K, void *result) {
+  if constexpr (waveKernelShape((int)sizeof(typename E::storage), Q, C)) {
+    const int grid = ((R + kWaveTileRows - 1) / kWaveTileRows + 7) / 8 * 8;
+    lc.begin("gatherConvWave");
+    gatherConvWave<E, Q, C><<<grid, 64, 0, lc.stream>>>(
+        static_cast<const typename E::storage *>(A), static_cast<const typename E::storage *>(packed),
+        source, R, K, static_cast<typename E::storage *>(result));
+    lc.end();
+  }
+}
+
+template <typename E>
+void launchWave(const LaunchCtx &lc, int Q, int C, const void *A, const void *packed,
+                const SegmentSource &source, int R, int K, void *result) {
+#define WAVE_CASE(q)                                                                      \
+  case q:                                                                                 \
+    if (C == 16) launchWaveInstance<E, q, 16>(lc, A, packed, source, R, K, result);       \
+    else launchWaveInstance<E, q, 32>(lc, A, packed, source, R, K, result);               \
+    break;
+  switch (Q) {
+    WAVE_CASE(16)
+    WAVE_CASE(32)
+    WAVE_CASE(64)
+    WAVE_CASE(128)
+    default: break;
+  }
+#undef WAVE_CASE
+}
+
+bool useWaveKernel(ElemType t, int Q, int C) {
+  const char *e = getenv("MLUOP_SPCONV_WAVE");
+  if (e != nullptr && e[0] == '0') return false;
+  return waveKernelShape((int)elemSize(t), Q, C);
 }
 
 // The register-accumulating kernel pays when a quarter or more of all (row, offset)
@@ -1629,39 +2175,39 @@ bool useDenseKernel(const ConvProblem &p, const GatherDims &d) {
   return pairs >= 0.25 * (double)d.R * p.K;
 }
 
-template <typename E, int Q, int C>
-void launchDenseInstance(const LaunchCtx &lc, const void *A, const void *packed, RowMap map,
+template <typename E, int Q, int C, typename SRC>
+void launchDenseInstance(const LaunchCtx &lc, const void *A, const void *packed, const SRC &source,
                          int R, int K, void *result) {
   const dim3 grid(denseGridX(R), 1);
   lc.begin("gatherConvDense");
-  gatherConvDense<E, Q, C><<<grid, denseThreads(C), 0, lc.stream>>>(
+  gatherConvDense<E, Q, C, SRC><<<grid, denseThreads(C), 0, lc.stream>>>(
       static_cast<const typename E::storage *>(A), static_cast<const typename E::storage *>(packed),
-      map.entries, R, K, C, map.filled, static_cast<typename E::storage *>(result));
+      source, R, K, C, static_cast<typename E::storage *>(result));
   lc.end();
 }
 
-template <typename E>
+template <typename E, typename SRC>
 void launchDense(const LaunchCtx &lc, int Q, int C, const void *A, const void *packed,
-                 RowMap map, int R, int K, void *result) {
+                 const SRC &source, int R, int K, void *result) {
   constexpr bool is_float = std::is_same<E, FloatElem>::value;
-#define DENSE_CASE(q)                                                                      \
-  case q:                                                                                  \
-    if (C == 64) launchDenseInstance<E, q, 64>(lc, A, packed, map, R, K, result);          \
-    else launchDenseInstance<E, q, 128>(lc, A, packed, map, R, K, result);                 \
+#define DENSE_CASE(q)                                                                           \
+  case q:                                                                                       \
+    if (C == 64) launchDenseInstance<E, q, 64, SRC>(lc, A, packed, source, R, K, result);       \
+    else launchDenseInstance<E, q, 128, SRC>(lc, A, packed, source, R, K, result);              \
     break;
   switch (Q) {
     case 16:
       if constexpr (is_float) {
-        if (C == 64) launchDenseInstance<E, 16, 64>(lc, A, packed, map, R, K, result);
-        else launchDenseInstance<E, 16, 128>(lc, A, packed, map, R, K, result);
+        if (C == 64) launchDenseInstance<E, 16, 64, SRC>(lc, A, packed, source, R, K, result);
+        else launchDenseInstance<E, 16, 128, SRC>(lc, A, packed, source, R, K, result);
       }
       break;
     DENSE_CASE(32)
     DENSE_CASE(64)
     case 128:
       if constexpr (!is_float) {
-        if (C == 64) launchDenseInstance<E, 128, 64>(lc, A, packed, map, R, K, result);
-        else launchDenseInstance<E, 128, 128>(lc, A, packed, map, R, K, result);
+        if (C == 64) launchDenseInstance<E, 128, 64, SRC>(lc, A, packed, source, R, K, result);
+        else launchDenseInstance<E, 128, 128, SRC>(lc, A, packed, source, R, K, result);
       }
       break;
     default: break;
@@ -1716,6 +2262,52 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
   // B(k, q, c): forward q = ci, c = co; backward data q = co, c = ci.
   const int64_t sQ = d.filter_forward ? f.stride_ci : f.stride_co;
   const int64_t sC = d.filter_forward ? f.stride_co : f.stride_ci;
+  if (use_mfma && listsUsable(p, d)) {
+    // Pair lists in order (as far as the caller knows: the first kernel checks): the
+    // gather kernel reads them cut by tile, no row map.
+    const bool dense = useDenseKernel(p, d);
+    const int tile_cols = dense ? d.C : mfmaTileCols(p, d);
+    const int tile_rows = dense ? kDenseTileRows : mfmaTileRows(tile_cols);
+    int tile_shift = 0;
+    while ((1 << tile_shift) < tile_rows) ++tile_shift;
+    const int n_tiles = (d.R + tile_rows - 1) / tile_rows;
+    OffsetBlocks ob;
+    int list_blocks = 0;
+    for (int k = 0; k < kMaxInlineK; ++k) {
+      ob.first[k] = list_blocks;
+      if (k < p.K) list_blocks += inl.n[k] > 0 ? (inl.n[k] + 255) / 256 : 1;
+    }
+    const size_t frags = (size_t)p.K * (d.C / 16) * ((d.Q + E::kChunk - 1) / E::kChunk) * 64;
+    const int pack_blocks = gridFor(frags, 512);
+    lc.begin("packFilterCutPairLists");
+    packFilterCutPairLists<E><<<pack_blocks + list_blocks, 256, 0, lc.stream>>>(
+        static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K, d.Q, d.C, static_cast<S *>(ws.packed),
+        pack_blocks, p.indice_pairs, p.L, inl, ob, d.row_col, d.src_col, d.R, d.n_src, tile_shift,
+        n_tiles, ws.cuts, ws.verdict, p.ticket);
+    lc.end();
+    SegmentSource src;
+    src.pairs = p.indice_pairs;
+    src.cuts = ws.cuts;
+    src.verdict = ws.verdict;
+    src.ticket = p.ticket;
+    src.L = p.L;
+    src.row_col = d.row_col;
+    src.src_col = d.src_col;
+    src.n_src = d.n_src;
+    src.cut_stride = n_tiles + 1;
+    src.W = f.base;
+    src.sK = f.stride_k;
+    src.sQ = sQ;
+    src.sC = sC;
+    src.counts = inl;
+    if (dense)
+      launchDense<E, SegmentSource>(lc, d.Q, d.C, gathered, ws.packed, src, d.R, p.K, result);
+    else if (tile_cols == d.C && useWaveKernel(p.dtype, d.Q, d.C))
+      launchWave<E>(lc, d.Q, d.C, gathered, ws.packed, src, d.R, p.K, result);
+    else
+      launchMfma<E, SegmentSource>(lc, d.Q, d.C, tile_cols, gathered, ws.packed, src, d.R, p.K, result);
+    return;
+  }
   const size_t map_elems = (size_t)p.K * d.R;
   const bool own_map = p.row_map == nullptr;  // else: built ahead, nothing to clear or fill
   const int32_t *entries = own_map ? ws.map : p.row_map;
@@ -1730,14 +2322,14 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
         d.Q, d.C, static_cast<S *>(ws.packed));
     lc.end();
     if (own_map) launchScatterRowMap(lc, p, d, ws, inl, max_count);
-    const RowMap map = {entries, ws.filled};
+    const MapSource map = {entries, ws.filled};
     if (useDenseKernel(p, d)) {
       n_filled = denseGridX(d.R);
-      launchDense<E>(lc, d.Q, d.C, gathered, ws.packed, map, d.R, p.K, result);
+      launchDense<E, MapSource>(lc, d.Q, d.C, gathered, ws.packed, map, d.R, p.K, result);
     } else {
       const int tile_cols = mfmaTileCols(p, d);
       n_filled = mfmaGridX(d.R, tile_cols);
-      launchMfma<E>(lc, d.Q, d.C, tile_cols, gathered, ws.packed, map, d.R, p.K, result);
+      launchMfma<E, MapSource>(lc, d.Q, d.C, tile_cols, gathered, ws.packed, map, d.R, p.K, result);
     }
   } else {
     if (own_map) {

@@ -8,6 +8,7 @@
 #include "core/core.h"
 #include "sparse_conv/indice_conv.h"
 #include "sparse_conv/row_map.h"
+#include "sparse_conv/rulebook_notes.h"
 
 namespace {
 
@@ -299,6 +300,8 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardData(
   p.distinct_pairs = handle->distinct_pairs_promised;
   st = mluop::sparse_conv::takeRowMap(api, handle, announced_map, GatherDirection::kBackwardData, &p);
   if (st != MLUOP_STATUS_SUCCESS) return st;
+  // result rows are named by pair column 0 (the other one in an inverse convolution)
+  mluop::sparse_conv::consultRulebookNotes(handle, p.inverse ? 1 : 0, &p);
   const size_t need =
       mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kBackwardData);
   if (workspace_size < need || workspace == NULL) {

@@ -7,6 +7,7 @@
 #include "core/core.h"
 #include "sparse_conv/indice_conv.h"
 #include "sparse_conv/row_map.h"
+#include "sparse_conv/rulebook_notes.h"
 
 namespace {
 
@@ -242,6 +243,8 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionForward(
   p.distinct_pairs = handle->distinct_pairs_promised;
   st = mluop::sparse_conv::takeRowMap(api, handle, announced_map, GatherDirection::kForward, &p);
   if (st != MLUOP_STATUS_SUCCESS) return st;
+  // result rows are named by pair column 1 (the other one in an inverse convolution)
+  mluop::sparse_conv::consultRulebookNotes(handle, p.inverse ? 0 : 1, &p);
   const size_t need = mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kForward);
   if (workspace_size < need || workspace == nullptr) {
     MLUOP_LOG(ERROR) << api << " workspace of " << workspace_size

@@ -27,13 +27,22 @@ struct RulebookGeom {
   bool sub_m;
 };
 
+// Where the last kernel of a rulebook reports (pinned host memory, written from the device):
+// whether the input rows were strictly ascending in (n, d, h, w) order, then the stamp that
+// tells the host the report is the one it waits for.  Null words: no report.
+struct RulebookReportTarget {
+  unsigned long long *stamp_word = nullptr;
+  unsigned int *order_word = nullptr;
+  unsigned long long stamp = 0;
+};
+
 // Bytes of device workspace the kernel set needs for this geometry.
 size_t rulebookWorkspaceBytes(const RulebookGeom &g);
 
 // Enqueues submanifold rulebook construction on the context's stream.
 hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const int32_t *indices,
                               void *workspace, int32_t *indice_pairs, int32_t *out_indices,
-                              int32_t *indice_num);
+                              int32_t *indice_num, const RulebookReportTarget &report);
 
 // Enqueues regular (strided / dilated) rulebook construction and
 // an asynchronous copy of the number of active outputs into `host_num_act_out`
@@ -41,7 +50,7 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
 hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                  const int32_t *indices, void *workspace, int32_t *indice_pairs,
                                  int32_t *out_indices, int32_t *indice_num,
-                                 int32_t *host_num_act_out);
+                                 int32_t *host_num_act_out, const RulebookReportTarget &report);
 
 }  // namespace sparse_conv
 }  // namespace mluop

@@ -112,7 +112,24 @@ __device__ __forceinline__ int axisOut(int i, int pad, int kk, int dil, int stri
   return o < osize ? o : -1;
 }
 
-__global__ __launch_bounds__(kBlock) void rbFill32(uint32_t *dst, size_t n, uint32_t value) {
+// Strictly below in (n, d, h, w) order, which is the order of linear cell indices.
+__device__ __forceinline__ bool coordBelow(int4 a, int4 b) {
+  if (a.x != b.x) return a.x < b.x;
+  if (a.y != b.y) return a.y < b.y;
+  if (a.z != b.z) return a.z < b.z;
+  return a.w < b.w;
+}
+
+// Row j and the row before it are out of cell order (or equal): the rulebook's report
+// will say so.  *rows_in_order was set to 1 by the first launch.
+__device__ __forceinline__ void noteRowOrder(const int32_t *indices, int j, int4 c, bool aligned,
+                                             int32_t *rows_in_order) {
+  if (j > 0 && !coordBelow(loadCoord(indices, j - 1, aligned), c)) *rows_in_order = 0;
+}
+
+__global__ __launch_bounds__(kBlock) void rbFill32(uint32_t *dst, size_t n, uint32_t value,
+                                                   int32_t *rows_in_order) {
+  if (blockIdx.x == 0 && threadIdx.x == 0) *rows_in_order = 1;
   // 16-byte stores; n is a multiple of 4 and dst is 16-byte aligned (workspace blocks are).
   uint4 *d4 = reinterpret_cast<uint4 *>(dst);
   const size_t n4 = n / 4;
@@ -150,10 +167,12 @@ __device__ __forceinline__ void decodeOffset(const OffsetTable &tab, const GeomD
 __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t *indices,
                                                        bool aligned, uint32_t *keys,
                                                        int32_t *vals, uint32_t mask,
-                                                       int32_t *out_indices, int out_rows) {
+                                                       int32_t *out_indices, int out_rows,
+                                                       int32_t *rows_in_order) {
   int j = blockIdx.x * kBlock + threadIdx.x;
   if (j < g.L) {
     int4 c = loadCoord(indices, j, aligned);
+    noteRowOrder(indices, j, c, aligned, rows_in_order);
     if (j < out_rows) storeCoord(out_indices, j, c, aligned);
     bool in_range = (unsigned)c.x < (unsigned)g.batch && (unsigned)c.y < (unsigned)g.out[0] &&
                     (unsigned)c.z < (unsigned)g.out[1] && (unsigned)c.w < (unsigned)g.out[2];
@@ -186,7 +205,8 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
                                                        const uint32_t *keys, const int32_t *vals,
                                                        uint32_t mask, unsigned long long *bitmap,
                                                        int32_t *cand, int32_t *counts,
-                                                       int n_wave, int k_per_slice) {
+                                                       int n_wave, int k_per_slice,
+                                                       int32_t *rows_in_order) {
   const int j = blockIdx.x * kBlock + threadIdx.x;
   // blockIdx.y selects a slice of the offsets: more waves in flight than rows alone give
   const int k_lo = blockIdx.y * k_per_slice;
@@ -197,6 +217,7 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
   const bool active = j < g.L;
   int4 c = make_int4(-1, 0, 0, 0);
   if (active) c = loadCoord(indices, j, aligned);
+  if (!SUBM && active && blockIdx.y == 0) noteRowOrder(indices, j, c, aligned, rows_in_order);
   const bool n_ok = active && (unsigned)c.x < (unsigned)g.batch;
   for (int k0 = k_lo; k0 < k_hi; k0 += kGroup) {
     uint32_t cell[kGroup];
@@ -568,7 +589,15 @@ __global__ __launch_bounds__(kBlock) void rbEmitPairs(int L, int K, const int32_
                                                       const int32_t *indice_num,
                                                       const unsigned long long *bitmap,
                                                       const uint32_t *word_rank,
-                                                      int32_t *pairs, int k_per_slice) {
+                                                      int32_t *pairs, int k_per_slice,
+                                                      const int32_t *rows_in_order,
+                                                      RulebookReportTarget report) {
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && report.stamp_word != nullptr) {
+    // the host reads the stamp first and takes the flag only when the stamp is its own
+    *report.order_word = (unsigned int)*rows_in_order;
+    __threadfence_system();
+    __hip_atomic_store(report.stamp_word, report.stamp, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
   const int j = blockIdx.x * kBlock + threadIdx.x;
   const int k_lo = blockIdx.y * k_per_slice;
   const int k_hi = k_lo + k_per_slice < K ? k_lo + k_per_slice : K;
@@ -749,6 +778,7 @@ struct Workspace {
   // both
   int32_t *cand = nullptr;
   int32_t *counts = nullptr;
+  int32_t *rows_in_order = nullptr;  // 1 until a kernel finds two rows out of cell order
   int n_wave = 0;
   size_t bytes = 0;
 };
@@ -781,6 +811,7 @@ Workspace carve(const RulebookGeom &g, void *base) {
   }
   ws.cand = reinterpret_cast<int32_t *>(take((size_t)g.K * g.L * 4));
   ws.counts = reinterpret_cast<int32_t *>(take((size_t)g.K * ws.n_wave * 4));
+  ws.rows_in_order = reinterpret_cast<int32_t *>(take(4));
   ws.bytes = off + 256;
   return ws;
 }
@@ -828,7 +859,7 @@ size_t rulebookWorkspaceBytes(const RulebookGeom &g) { return carve(g, nullptr).
 
 hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const int32_t *indices,
                               void *workspace, int32_t *indice_pairs, int32_t *out_indices,
-                              int32_t *indice_num) {
+                              int32_t *indice_num, const RulebookReportTarget &report) {
   const Workspace ws = carve(g, workspace);
   const GeomDev d = toDev(g);
   const bool al = aligned16(indices, out_indices);
@@ -840,11 +871,11 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
   // cells become kEmptyKey and rows -1 with the same all-ones pattern
   lc.begin("rbFill32");
   rbFill32<<<fillBlocks((size_t)ws.table_cap / 2), kBlock, 0, lc.stream>>>(
-      ws.keys, (size_t)ws.table_cap * 2, kEmptyKey);
+      ws.keys, (size_t)ws.table_cap * 2, kEmptyKey, ws.rows_in_order);
   lc.end();
   lc.begin("rbSubmInsert");
   rbSubmInsert<<<row_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.keys, ws.vals, mask,
-                                                     out_indices, g.out_rows);
+                                                     out_indices, g.out_rows, ws.rows_in_order);
   lc.end();
   const int k_per = offsetsPerSlice(g.K);
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
@@ -887,7 +918,7 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
     lc.begin("rbProbeCount");
     rbProbeCount<true><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al, ws.keys, ws.vals,
                                                              mask, nullptr, ws.cand, ws.counts,
-                                                             ws.n_wave, k_per);
+                                                             ws.n_wave, k_per, ws.rows_in_order);
     lc.end();
   }
   lc.begin("rbScanRows");
@@ -896,7 +927,7 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
   lc.begin("rbEmitPairs");
   rbEmitPairs<true><<<slice_grid, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
                                                        indice_num, nullptr, nullptr, indice_pairs,
-                                                       k_per);
+                                                       k_per, ws.rows_in_order, report);
   lc.end();
   return hipGetLastError();
 }
@@ -904,7 +935,7 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
 hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                  const int32_t *indices, void *workspace, int32_t *indice_pairs,
                                  int32_t *out_indices, int32_t *indice_num,
-                                 int32_t *host_num_act_out) {
+                                 int32_t *host_num_act_out, const RulebookReportTarget &report) {
   const Workspace ws = carve(g, workspace);
   const GeomDev d = toDev(g);
   const bool al_in = aligned16(indices, indices);
@@ -914,14 +945,15 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
   const OffsetTable tab = makeOffsetTable(g);
   lc.begin("rbFill32");
   rbFill32<<<fillBlocks(ws.n_words / 2 + 1), kBlock, 0, lc.stream>>>(
-      reinterpret_cast<uint32_t *>(ws.bitmap), ws.bitmap_fill_words, 0u);
+      reinterpret_cast<uint32_t *>(ws.bitmap), ws.bitmap_fill_words, 0u, ws.rows_in_order);
   lc.end();
   lc.begin("rbProbeCount");
   const int k_per = offsetsPerSlice(g.K);
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
   rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al_in, nullptr,
                                                             nullptr, 0, ws.bitmap, ws.cand,
-                                                            ws.counts, ws.n_wave, k_per);
+                                                            ws.counts, ws.n_wave, k_per,
+                                                            ws.rows_in_order);
   lc.end();
   lc.begin("rbScanRows");
   rbScanRows<<<g.K, kScanBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
@@ -945,7 +977,8 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
   lc.begin("rbEmitPairs");
   rbEmitPairs<false><<<slice_grid, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
                                                         indice_num, ws.bitmap, ws.word_rank,
-                                                        indice_pairs, k_per);
+                                                        indice_pairs, k_per, ws.rows_in_order,
+                                                        report);
   lc.end();
   return hipGetLastError();
 }

@@ -1,0 +1,45 @@
+// Notes about rulebooks built on a handle: which pair tensors came from
+// mluOpGetIndicePairs, and whether their input rows were in cell order.
+#include "sparse_conv/rulebook_notes.h"
+
+namespace mluop {
+namespace sparse_conv {
+
+RulebookReportTarget openRulebookNote(mluOpContext *handle, const void *pairs, int K, int L) {
+  // an older note about the same address describes a tensor that is being overwritten
+  for (auto &n : handle->rulebook_notes)
+    if (n.pairs == pairs) n.pairs = nullptr;
+  const int slot = handle->next_rulebook_note;
+  handle->next_rulebook_note = (slot + 1) % mluOpContext::kRulebookNotes;
+  mluOpContext::RulebookNote &note = handle->rulebook_notes[slot];
+  note.pairs = pairs;
+  note.K = K;
+  note.L = L;
+  note.stamp = handle->next_stamp++;
+  RulebookReportTarget t;
+  t.stamp_word = &handle->rulebook_reports[slot].stamp;
+  t.order_word = &handle->rulebook_reports[slot].rows_in_order;
+  t.stamp = note.stamp;
+  return t;
+}
+
+void consultRulebookNotes(mluOpContext *handle, int row_column, ConvProblem *p) {
+  p->ticket = handle->next_stamp++;
+  p->lists_in_order = false;
+  if (handle->rulebook_reports == nullptr) return;
+  for (int slot = 0; slot < mluOpContext::kRulebookNotes; ++slot) {
+    const mluOpContext::RulebookNote &note = handle->rulebook_notes[slot];
+    if (note.pairs != p->indice_pairs || note.K != p->K || note.L != p->L) continue;
+    if (row_column == 0) {
+      p->lists_in_order = true;
+      return;
+    }
+    const volatile mluOpContext::RulebookReport *report = &handle->rulebook_reports[slot];
+    if (__atomic_load_n(&report->stamp, __ATOMIC_ACQUIRE) != note.stamp) return;
+    p->lists_in_order = report->rows_in_order != 0;
+    return;
+  }
+}
+
+}  // namespace sparse_conv
+}  // namespace mluop
