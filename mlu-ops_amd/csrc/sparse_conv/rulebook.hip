@@ -11,12 +11,14 @@
 // offset, pairs are listed by ascending input row; unused tails are -1.
 //
 // Kernel set
-//   submanifold:  clear hash -> insert rows -> probe (one wavefront per 64
-//                 rows, per-wave pair counts) -> scan counts per offset ->
-//                 emit (wave-ballot ranks, coalesced pair writes, -1 tails)
-//   regular:      clear bitmap -> mark output cells + record candidates ->
-//                 scan counts -> bitmap popcount scan (ranks, out_indices) ->
-//                 emit with rank lookup
+//   submanifold:  clear hash -> insert rows (and set every pair slot to -1) ->
+//                 probe + compact: a workgroup of 256 rows resolves its pairs,
+//                 learns how many pairs earlier rows hold at every offset by
+//                 looking back over the workgroups before it, and writes its
+//                 pairs at their final positions
+//   regular:      clear bitmap, pair slots to -1 -> mark output cells + compact
+//                 (output cell in place of the output row) -> bitmap popcount
+//                 scan (ranks, out_indices) -> cells to ranks in place
 // The stable order needs no sort: rows are visited in ascending order by
 // construction (lane = row) and positions come from exclusive prefix sums.
 #include <hip/hip_runtime.h>
@@ -127,16 +129,39 @@ __device__ __forceinline__ void noteRowOrder(const int32_t *indices, int j, int4
   if (j > 0 && !coordBelow(loadCoord(indices, j - 1, aligned), c)) *rows_in_order = 0;
 }
 
-__global__ __launch_bounds__(kBlock) void rbFill32(uint32_t *dst, size_t n, uint32_t value,
-                                                   int32_t *rows_in_order) {
+// The rulebook's report to the host: the flag first, then the stamp the host looks for.
+__device__ __forceinline__ void fileReport(const int32_t *rows_in_order, const RulebookReportTarget &report) {
+  if (report.stamp_word == nullptr) return;
+  *report.order_word = *rows_in_order != 0 ? 1u : 0u;
+  __threadfence_system();
+  __hip_atomic_store(report.stamp_word, report.stamp, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// Up to three ranges of 32-bit words, each set to its own value (16-byte stores: every
+// count is a multiple of 4 and every range 16-byte aligned, as workspace blocks are; a
+// caller's tensor that is not goes word by word).  Also raises the rows-in-order flag.
+struct FillRanges {
+  uint32_t *dst[3];
+  size_t n[3];
+  uint32_t value[3];
+};
+
+__global__ __launch_bounds__(kBlock) void rbFill(FillRanges r, int32_t *rows_in_order) {
   if (blockIdx.x == 0 && threadIdx.x == 0) *rows_in_order = 1;
-  // 16-byte stores; n is a multiple of 4 and dst is 16-byte aligned (workspace blocks are).
-  uint4 *d4 = reinterpret_cast<uint4 *>(dst);
-  const size_t n4 = n / 4;
-  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * kBlock;
-  const uint4 v = make_uint4(value, value, value, value);
-  for (; i < n4; i += stride) d4[i] = v;
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    if (r.n[i] == 0) continue;
+    const uint32_t v = r.value[i];
+    if ((reinterpret_cast<uintptr_t>(r.dst[i]) & 15u) == 0 && (r.n[i] & 3u) == 0) {
+      uint4 *d4 = reinterpret_cast<uint4 *>(r.dst[i]);
+      const size_t n4 = r.n[i] / 4;
+      for (size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x; t < n4; t += stride)
+        d4[t] = make_uint4(v, v, v, v);
+    } else {
+      for (size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x; t < r.n[i]; t += stride) r.dst[i][t] = v;
+    }
+  }
 }
 
 // Kernel offsets (kd, kh, kw) of offset index k.  Small kernel volumes carry a
@@ -168,9 +193,15 @@ __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t 
                                                        bool aligned, uint32_t *keys,
                                                        int32_t *vals, uint32_t mask,
                                                        int32_t *out_indices, int out_rows,
-                                                       int32_t *rows_in_order) {
+                                                       int32_t *rows_in_order, int32_t *pairs) {
   int j = blockIdx.x * kBlock + threadIdx.x;
   if (j < g.L) {
+    // Every pair slot starts as -1; the probe kernel overwrites the slots in front of each
+    // offset's pair count.  Plain stores that nobody waits for, under the table's atomics.
+    for (int k = 0; k < g.K; ++k) {
+      pairs[(size_t)k * 2 * g.L + j] = -1;
+      pairs[((size_t)k * 2 + 1) * g.L + j] = -1;
+    }
     int4 c = loadCoord(indices, j, aligned);
     noteRowOrder(indices, j, c, aligned, rows_in_order);
     if (j < out_rows) storeCoord(out_indices, j, c, aligned);
@@ -194,6 +225,50 @@ __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t 
   }
 }
 
+// ---- pairs to their final positions -----------------------------------------------
+//
+// A pair's position inside its offset is the number of pairs earlier rows hold there.
+// The probe kernels do not know it yet; a wave (64 consecutive rows) stages the pairs it
+// found at offset k compactly at the start of its own 64 slots of stage[k][.] and writes
+// their number to counts[k][wave], so that what crosses the kernel boundary is the pairs
+// (a few per wave and offset) and not a slot for every (row, offset).  rbPlacePairs then
+// moves them: a workgroup adds up the counts in front of its 256 waves, scans its own, and
+// copies the staged pairs to their final positions.
+// (Looking back over earlier workgroups inside the probe kernel instead, single-pass-scan
+// style, was built and measured: all workgroups finish probing at the same moment, so
+// the look-back degenerates into a chain over hundreds of workgroups per offset; 400 us.)
+struct Staging {
+  int32_t *stage;       // [K, L]: submanifold: output row << 6 | lane; regular: output cell
+  uint8_t *stage_lane;  // [K, L], regular mode only: lane of the staged pair
+  int32_t *counts;      // [K, n_wave]
+  int n_wave;
+};
+
+template <bool SUBM, int N>
+__device__ __forceinline__ void stagePairs(const int (&res)[N], int k_first, int k_end, int j, int L,
+                                           const Staging &st) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wt = j >> 6;
+  const unsigned long long lt_mask = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int u = 0; u < N; ++u) {
+    const int k = k_first + u;
+    if (k < k_end) {
+      const unsigned long long b = __ballot(res[u] >= 0);
+      if (res[u] >= 0) {
+        const size_t at = (size_t)k * L + (size_t)wt * kWave + __popcll(b & lt_mask);
+        if (SUBM) {
+          st.stage[at] = (res[u] << 6) | lane;
+        } else {
+          st.stage[at] = res[u];
+          st.stage_lane[at] = (uint8_t)lane;
+        }
+      }
+      if (lane == 0) st.counts[(size_t)k * st.n_wave + wt] = __popcll(b);
+    }
+  }
+}
+
 // One wavefront per 64 consecutive rows, offsets in groups of kGroup so that a
 // lane keeps kGroup independent table probes in flight.  For every offset:
 // resolve the pair (submanifold: table lookup -> output row; regular: output
@@ -204,16 +279,13 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
                                                        const int32_t *indices, bool aligned,
                                                        const uint32_t *keys, const int32_t *vals,
                                                        uint32_t mask, unsigned long long *bitmap,
-                                                       int32_t *cand, int32_t *counts,
-                                                       int n_wave, int k_per_slice,
+                                                       Staging staging, int k_per_slice,
                                                        int32_t *rows_in_order) {
   const int j = blockIdx.x * kBlock + threadIdx.x;
   // blockIdx.y selects a slice of the offsets: more waves in flight than rows alone give
   const int k_lo = blockIdx.y * k_per_slice;
   const int k_hi = k_lo + k_per_slice < g.K ? k_lo + k_per_slice : g.K;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wt = j >> 6;
-  if (wt >= n_wave) return;  // whole wave beyond the last row
+  if ((j >> 6) >= staging.n_wave) return;  // whole wave beyond the last row
   const bool active = j < g.L;
   int4 c = make_int4(-1, 0, 0, 0);
   if (active) c = loadCoord(indices, j, aligned);
@@ -284,15 +356,7 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
         }
       }
     }
-#pragma unroll
-    for (int u = 0; u < kGroup; ++u) {
-      const int k = k0 + u;
-      if (k < k_hi) {
-        if (active) cand[(size_t)k * g.L + j] = res[u];
-        const unsigned long long b = __ballot(res[u] >= 0);
-        if (lane == 0) counts[(size_t)k * n_wave + wt] = __popcll(b);
-      }
-    }
+    stagePairs<SUBM, kGroup>(res, k0, k_hi, j, g.L, staging);
   }
 }
 
@@ -309,14 +373,11 @@ struct UnitStrideOffsets {
 
 __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
     GeomDev g, UnitStrideOffsets tab, const int32_t *indices, bool aligned, const uint32_t *keys,
-    const int32_t *vals, uint32_t mask, int32_t *cand, int32_t *counts, int n_wave,
-    int k_per_slice) {
+    const int32_t *vals, uint32_t mask, Staging staging, int k_per_slice) {
   const int j = blockIdx.x * kBlock + threadIdx.x;
   const int k_lo = blockIdx.y * k_per_slice;
   const int k_hi = k_lo + k_per_slice < g.K ? k_lo + k_per_slice : g.K;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wt = j >> 6;
-  if (wt >= n_wave) return;  // whole wave beyond the last row
+  if ((j >> 6) >= staging.n_wave) return;  // whole wave beyond the last row
   const bool active = j < g.L;
   int4 c = make_int4(-1, 0, 0, 0);
   if (active) c = loadCoord(indices, j, aligned);
@@ -375,15 +436,7 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
     for (int u = 0; u < kGroup; ++u) {
       if (hit & (1u << u)) res[u] = vals[slot[u]];
     }
-#pragma unroll
-    for (int u = 0; u < kGroup; ++u) {
-      const int k = k0 + u;
-      if (k < k_hi) {
-        if (active) cand[(size_t)k * g.L + j] = res[u];
-        const unsigned long long b = __ballot(res[u] >= 0);
-        if (lane == 0) counts[(size_t)k * n_wave + wt] = __popcll(b);
-      }
-    }
+    stagePairs<true, kGroup>(res, k0, k_hi, j, g.L, staging);
   }
 }
 
@@ -406,17 +459,14 @@ constexpr int kGroupsPerPass = 3;  // (kd, kh) pairs resolved together per lane
 template <int KW>
 __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
     GeomDev g, UnitStrideOffsets tab, const int32_t *indices, bool aligned, const uint32_t *keys,
-    const int32_t *vals, uint32_t mask, int32_t *cand, int32_t *counts, int n_wave,
-    int groups_per_slice) {
+    const int32_t *vals, uint32_t mask, Staging staging, int groups_per_slice) {
   constexpr int N = kGroupsPerPass * KW;
   static_assert(KW <= kWindow && N <= 32, "window and bit masks");
   const int j = blockIdx.x * kBlock + threadIdx.x;
   const int n_groups = g.K / KW;
   const int t_lo = blockIdx.y * groups_per_slice;
   const int t_hi = t_lo + groups_per_slice < n_groups ? t_lo + groups_per_slice : n_groups;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wt = j >> 6;
-  if (wt >= n_wave) return;  // whole wave beyond the last row
+  if ((j >> 6) >= staging.n_wave) return;  // whole wave beyond the last row
   const bool active = j < g.L;
   int4 c = make_int4(-1, 0, 0, 0);
   if (active) c = loadCoord(indices, j, aligned);
@@ -523,16 +573,7 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
     for (int u = 0; u < N; ++u) {
       if (hit & (1u << u)) res[u] = vals[slot[u]];
     }
-#pragma unroll
-    for (int u = 0; u < N; ++u) {
-      const int t = t0 + u / KW;
-      if (t < t_hi) {
-        const int k = KW * t + u % KW;
-        if (active) cand[(size_t)k * g.L + j] = res[u];
-        const unsigned long long b = __ballot(res[u] >= 0);
-        if (lane == 0) counts[(size_t)k * n_wave + wt] = __popcll(b);
-      }
-    }
+    stagePairs<true, N>(res, KW * t0, KW * t_hi, j, g.L, staging);
   }
 }
 
@@ -578,76 +619,6 @@ __global__ __launch_bounds__(kScanBlock) void rbScanRows(int32_t *data, int n, i
     __syncthreads();
   }
   if (threadIdx.x == 0) totals[blockIdx.x] = carry;
-}
-
-// Compacts the candidates of every offset in row order: position = exclusive
-// wave prefix + rank of the lane among the wave's hits.  Lane j also owns
-// position j of every offset's tail and writes -1 there when j >= indice_num[k].
-template <bool SUBM>
-__global__ __launch_bounds__(kBlock) void rbEmitPairs(int L, int K, const int32_t *cand,
-                                                      const int32_t *wave_offs, int n_wave,
-                                                      const int32_t *indice_num,
-                                                      const unsigned long long *bitmap,
-                                                      const uint32_t *word_rank,
-                                                      int32_t *pairs, int k_per_slice,
-                                                      const int32_t *rows_in_order,
-                                                      RulebookReportTarget report) {
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && report.stamp_word != nullptr) {
-    // the host reads the stamp first and takes the flag only when the stamp is its own
-    *report.order_word = (unsigned int)*rows_in_order;
-    __threadfence_system();
-    __hip_atomic_store(report.stamp_word, report.stamp, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-  }
-  const int j = blockIdx.x * kBlock + threadIdx.x;
-  const int k_lo = blockIdx.y * k_per_slice;
-  const int k_hi = k_lo + k_per_slice < K ? k_lo + k_per_slice : K;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wt = j >> 6;
-  if (wt >= n_wave) return;
-  const bool active = j < L;
-  const unsigned long long lt_mask = (1ull << lane) - 1ull;
-  for (int k0 = k_lo; k0 < k_hi; k0 += kGroup) {
-    int r[kGroup], base[kGroup], total[kGroup];
-#pragma unroll
-    for (int u = 0; u < kGroup; ++u) {
-      const int k = k0 + u;
-      r[u] = -1;
-      base[u] = 0;
-      total[u] = 0;
-      if (k < k_hi) {
-        if (active) r[u] = cand[(size_t)k * L + j];
-        base[u] = wave_offs[(size_t)k * n_wave + wt];
-        total[u] = indice_num[k];
-      }
-    }
-    if (!SUBM) {
-#pragma unroll
-      for (int u = 0; u < kGroup; ++u) {
-        if (r[u] >= 0) {
-          const unsigned long long below = bitmap[r[u] >> 6] & ((1ull << (r[u] & 63)) - 1ull);
-          r[u] = (int)(word_rank[r[u] >> 6] + (uint32_t)__popcll(below));
-        }
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < kGroup; ++u) {
-      const int k = k0 + u;
-      if (k < k_hi) {
-        const unsigned long long b = __ballot(r[u] >= 0);
-        int32_t *in_col = pairs + (size_t)k * 2 * L;
-        int32_t *out_col = in_col + L;
-        if (r[u] >= 0) {
-          const int pos = base[u] + __popcll(b & lt_mask);
-          in_col[pos] = j;
-          out_col[pos] = r[u];
-        }
-        if (active && j >= total[u]) {
-          in_col[j] = -1;
-          out_col[j] = -1;
-        }
-      }
-    }
-  }
 }
 
 // ---- regular mode: ranks of marked cells -----------------------------------
@@ -735,6 +706,75 @@ __global__ __launch_bounds__(kBlock) void rbRankAndDecode(GeomDev g,
   }
 }
 
+// Moves the staged pairs of kPlaceWaves waves of one offset (workgroup (x, k)) to their
+// final positions: the pairs in front of the chunk are the sum of the earlier waves'
+// counts (a few kilobytes, read by every workgroup of the offset rather than scanned in a
+// launch of its own), wave 0 scans the chunk's own counts, and every wave of the
+// workgroup copies a quarter of the chunk's staged pieces, one piece per step, a lane per
+// pair.  In regular mode the staged output cell becomes the output row, its rank among
+// the marked cells.  One thread also files the rulebook's report.
+constexpr int kPlaceWaves = 64;
+template <bool SUBM>
+__global__ __launch_bounds__(kBlock) void rbPlacePairs(int L, Staging st,
+                                                        const unsigned long long *bitmap,
+                                                        const uint32_t *word_rank, int32_t *pairs,
+                                                        int32_t *indice_num,
+                                                        const int32_t *rows_in_order,
+                                                        RulebookReportTarget report) {
+  static_assert(kPlaceWaves == kWave, "one lane per wave count in the scan");
+  __shared__ int s_first[kPlaceWaves];  // staged pairs in front of each wave of the chunk
+  __shared__ int s_count[kPlaceWaves];
+  __shared__ int s_wave_sum[kBlock / kWave];
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) fileReport(rows_in_order, report);
+  const int k = blockIdx.y;
+  const int w0 = blockIdx.x * kPlaceWaves;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int32_t *counts = st.counts + (size_t)k * st.n_wave;
+  // pairs of the waves in front of the chunk
+  int part = 0;
+  for (int i = tid; i < w0; i += kBlock) part += counts[i];
+  part = waveInclusiveScan(part);
+  if (lane == kWave - 1) s_wave_sum[wave] = part;
+  if (wave == 0) {
+    const int mine = w0 + lane < st.n_wave ? counts[w0 + lane] : 0;
+    const int incl = waveInclusiveScan(mine);
+    s_count[lane] = mine;
+    s_first[lane] = incl - mine;
+  }
+  __syncthreads();
+  int before = 0;
+#pragma unroll
+  for (int w = 0; w < kBlock / kWave; ++w) before += s_wave_sum[w];
+  if (blockIdx.x == gridDim.x - 1 && tid == 0)
+    indice_num[k] = before + s_first[kPlaceWaves - 1] + s_count[kPlaceWaves - 1];
+  int32_t *in_col = pairs + (size_t)k * 2 * L;
+  int32_t *out_col = in_col + L;
+  constexpr int kPieces = kPlaceWaves / (kBlock / kWave);  // staged pieces per wave
+#pragma unroll 4
+  for (int i = 0; i < kPieces; ++i) {
+    const int seg = wave * kPieces + i;
+    if (lane < s_count[seg]) {
+      const int first_row = (w0 + seg) * kWave;
+      const size_t at = (size_t)k * L + (size_t)first_row + lane;
+      const int v = st.stage[at];
+      int row, out;
+      if (SUBM) {
+        row = first_row + (v & 63);
+        out = v >> 6;
+      } else {
+        row = first_row + (int)st.stage_lane[at];
+        const unsigned long long below = bitmap[v >> 6] & ((1ull << (v & 63)) - 1ull);
+        out = (int)(word_rank[v >> 6] + (uint32_t)__popcll(below));
+      }
+      const int to = before + s_first[seg] + lane;
+      in_col[to] = row;
+      out_col[to] = out;
+    }
+  }
+}
+
 // ---- host side ---------------------------------------------------------------
 
 inline size_t alignUp(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
@@ -776,10 +816,11 @@ struct Workspace {
   size_t bitmap_fill_words = 0;  // 32-bit words to clear, rounded up to a multiple of 4
   int n_bitmap_blocks = 0;
   // both
-  int32_t *cand = nullptr;
-  int32_t *counts = nullptr;
-  int32_t *rows_in_order = nullptr;  // 1 until a kernel finds two rows out of cell order
+  int32_t *stage = nullptr;          // [K, L] staged pairs (see Staging)
+  uint8_t *stage_lane = nullptr;     // [K, L], regular mode only
+  int32_t *counts = nullptr;         // [K, n_wave]
   int n_wave = 0;
+  int32_t *rows_in_order = nullptr;  // 1 until a kernel finds two rows out of cell order
   size_t bytes = 0;
 };
 
@@ -809,7 +850,8 @@ Workspace carve(const RulebookGeom &g, void *base) {
     ws.block_sum = reinterpret_cast<int32_t *>(take((size_t)ws.n_bitmap_blocks * 4));
     ws.num_act_out = reinterpret_cast<int32_t *>(take(4));
   }
-  ws.cand = reinterpret_cast<int32_t *>(take((size_t)g.K * g.L * 4));
+  ws.stage = reinterpret_cast<int32_t *>(take((size_t)g.K * g.L * 4));
+  if (!g.sub_m) ws.stage_lane = reinterpret_cast<uint8_t *>(take((size_t)g.K * g.L));
   ws.counts = reinterpret_cast<int32_t *>(take((size_t)g.K * ws.n_wave * 4));
   ws.rows_in_order = reinterpret_cast<int32_t *>(take(4));
   ws.bytes = off + 256;
@@ -869,14 +911,19 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
   const int l_blocks = (g.L + kBlock - 1) / kBlock;
 
   // cells become kEmptyKey and rows -1 with the same all-ones pattern
-  lc.begin("rbFill32");
-  rbFill32<<<fillBlocks((size_t)ws.table_cap / 2), kBlock, 0, lc.stream>>>(
-      ws.keys, (size_t)ws.table_cap * 2, kEmptyKey, ws.rows_in_order);
+  FillRanges fill = {};
+  fill.dst[0] = ws.keys;
+  fill.n[0] = (size_t)ws.table_cap * 2;
+  fill.value[0] = kEmptyKey;
+  lc.begin("rbFill");
+  rbFill<<<fillBlocks((size_t)ws.table_cap / 2), kBlock, 0, lc.stream>>>(fill, ws.rows_in_order);
   lc.end();
   lc.begin("rbSubmInsert");
   rbSubmInsert<<<row_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.keys, ws.vals, mask,
-                                                     out_indices, g.out_rows, ws.rows_in_order);
+                                                     out_indices, g.out_rows, ws.rows_in_order,
+                                                     indice_pairs);
   lc.end();
+  const Staging staging = {ws.stage, nullptr, ws.counts, ws.n_wave};
   const int k_per = offsetsPerSlice(g.K);
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
   const bool unit_stride = g.stride[0] == 1 && g.stride[1] == 1 && g.stride[2] == 1 &&
@@ -902,32 +949,28 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
       lc.begin("rbSubmProbeRuns");
       if (g.ksize[2] == 3)
         rbSubmProbeRuns<3><<<grid, kBlock, 0, lc.stream>>>(d, ut, indices, al, ws.keys, ws.vals, mask,
-                                                           ws.cand, ws.counts, ws.n_wave, t_per);
+                                                           staging, t_per);
       else
         rbSubmProbeRuns<5><<<grid, kBlock, 0, lc.stream>>>(d, ut, indices, al, ws.keys, ws.vals, mask,
-                                                           ws.cand, ws.counts, ws.n_wave, t_per);
+                                                           staging, t_per);
       lc.end();
     } else {
       lc.begin("rbSubmProbeUnitStride");
-      rbSubmProbeUnitStride<<<slice_grid, kBlock, 0, lc.stream>>>(
-          d, ut, indices, al, ws.keys, ws.vals, mask, ws.cand, ws.counts, ws.n_wave, k_per);
+      rbSubmProbeUnitStride<<<slice_grid, kBlock, 0, lc.stream>>>(d, ut, indices, al, ws.keys, ws.vals,
+                                                                  mask, staging, k_per);
       lc.end();
     }
   } else {
     const OffsetTable tab = makeOffsetTable(g);
     lc.begin("rbProbeCount");
     rbProbeCount<true><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al, ws.keys, ws.vals,
-                                                             mask, nullptr, ws.cand, ws.counts,
-                                                             ws.n_wave, k_per, ws.rows_in_order);
+                                                             mask, nullptr, staging, k_per,
+                                                             ws.rows_in_order);
     lc.end();
   }
-  lc.begin("rbScanRows");
-  rbScanRows<<<g.K, kScanBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
-  lc.end();
-  lc.begin("rbEmitPairs");
-  rbEmitPairs<true><<<slice_grid, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
-                                                       indice_num, nullptr, nullptr, indice_pairs,
-                                                       k_per, ws.rows_in_order, report);
+  lc.begin("rbPlacePairs");
+  rbPlacePairs<true><<<dim3((ws.n_wave + kPlaceWaves - 1) / kPlaceWaves, g.K), kBlock, 0, lc.stream>>>(
+      g.L, staging, nullptr, nullptr, indice_pairs, indice_num, ws.rows_in_order, report);
   lc.end();
   return hipGetLastError();
 }
@@ -943,20 +986,25 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
   const int l_blocks = (g.L + kBlock - 1) / kBlock;
 
   const OffsetTable tab = makeOffsetTable(g);
-  lc.begin("rbFill32");
-  rbFill32<<<fillBlocks(ws.n_words / 2 + 1), kBlock, 0, lc.stream>>>(
-      reinterpret_cast<uint32_t *>(ws.bitmap), ws.bitmap_fill_words, 0u, ws.rows_in_order);
+  // bitmap 0, every pair slot -1
+  FillRanges fill = {};
+  fill.dst[0] = reinterpret_cast<uint32_t *>(ws.bitmap);
+  fill.n[0] = ws.bitmap_fill_words;
+  fill.value[0] = 0u;
+  fill.dst[1] = reinterpret_cast<uint32_t *>(indice_pairs);
+  fill.n[1] = (size_t)g.K * 2 * g.L;
+  fill.value[1] = 0xffffffffu;
+  lc.begin("rbFill");
+  rbFill<<<fillBlocks((ws.bitmap_fill_words + fill.n[1]) / 4 + 1), kBlock, 0, lc.stream>>>(
+      fill, ws.rows_in_order);
   lc.end();
+  const Staging staging = {ws.stage, ws.stage_lane, ws.counts, ws.n_wave};
   lc.begin("rbProbeCount");
   const int k_per = offsetsPerSlice(g.K);
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
   rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al_in, nullptr,
-                                                            nullptr, 0, ws.bitmap, ws.cand,
-                                                            ws.counts, ws.n_wave, k_per,
+                                                            nullptr, 0, ws.bitmap, staging, k_per,
                                                             ws.rows_in_order);
-  lc.end();
-  lc.begin("rbScanRows");
-  rbScanRows<<<g.K, kScanBlock, 0, lc.stream>>>(ws.counts, ws.n_wave, indice_num);
   lc.end();
   lc.begin("rbBitmapBlockSum");
   rbBitmapBlockSum<<<ws.n_bitmap_blocks, kBlock, 0, lc.stream>>>(ws.bitmap, ws.n_words,
@@ -974,11 +1022,9 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                                              ws.word_rank, out_indices, al_out,
                                                              g.out_rows);
   lc.end();
-  lc.begin("rbEmitPairs");
-  rbEmitPairs<false><<<slice_grid, kBlock, 0, lc.stream>>>(g.L, g.K, ws.cand, ws.counts, ws.n_wave,
-                                                        indice_num, ws.bitmap, ws.word_rank,
-                                                        indice_pairs, k_per, ws.rows_in_order,
-                                                        report);
+  lc.begin("rbPlacePairs");
+  rbPlacePairs<false><<<dim3((ws.n_wave + kPlaceWaves - 1) / kPlaceWaves, g.K), kBlock, 0, lc.stream>>>(
+      g.L, staging, ws.bitmap, ws.word_rank, indice_pairs, indice_num, ws.rows_in_order, report);
   lc.end();
   return hipGetLastError();
 }

@@ -16,6 +16,9 @@ RulebookReportTarget openRulebookNote(mluOpContext *handle, const void *pairs, i
   note.K = K;
   note.L = L;
   note.stamp = handle->next_stamp++;
+  // the device ORs its flags into a cleared word and stores the stamp last
+  handle->rulebook_reports[slot].stamp = 0;
+  handle->rulebook_reports[slot].rows_in_order = 0;
   RulebookReportTarget t;
   t.stamp_word = &handle->rulebook_reports[slot].stamp;
   t.order_word = &handle->rulebook_reports[slot].rows_in_order;
