@@ -1,10 +1,13 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-convolution hot path on one MI355X.
 
-A step is one pass of the path over one synthetic voxel set already resident in HBM:
-mluOpGetIndicePairs (rulebook) followed by mluOpIndiceConvolutionForward, called through the
+A step is one pass of the path over one synthetic voxel set already resident in HBM, in the call
+sequence the API prescribes: mluOpGetIndicePairs (rulebook), the copy of indice_num to the host
+(the convolutions take the counts as a host array), mluOpIndiceConvolutionForward; all through the
 library's C ABI with descriptors and workspaces prepared once.  The default workload is BASELINE
-configuration 4 (submanifold 3x3x3, 120 000 clustered voxels in 1x41x1600x1408, Ci=Co=64 fp16).
+configuration 4 (submanifold 3x3x3, 120 000 clustered voxels in 1x41x1600x1408, Ci=Co=64 fp16);
+--workload names the other BASELINE layers (regular ones included: their rulebook call waits for
+num_act_out inside, as the reference's does) and four layers of a detection network.
 
 Prints one JSON line: `value` is the forward operator's algorithmic TFLOP/s (2*P*Ci*Co per call
 over its device time), `rulebook_mvoxels_per_s` the second half of the metric, `roofline`
@@ -26,9 +29,10 @@ for _p in (os.path.join(ROOT, "mlu-ops_amd", "python"), os.path.join(ROOT, "orac
 METRIC = "indice_conv fwd TFLOP/s + get_indice_pairs Mvoxels/s, 120k voxels Ci=Co=64"
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
+MFMA_F32_PEAK_TFLOPS = 157.3
 
 WORKLOADS = {
-    # name: (grid N,D,H,W, voxels per batch, generator, seed, Ci, Co, dtype, kernel)
+    # name: grid N,D,H,W, rows, generator, seed, channels, dtype, kernel / stride / padding, mode
     "config4": dict(grid=(1, 41, 1600, 1408), per_batch=120000, gen="clustered", seed=4, ci=64, co=64,
                     dtype="float16", ks=(3, 3, 3),
                     text="BASELINE config 4: subm 3x3x3, 120000 clustered voxels in 1x41x1600x1408, "
@@ -40,15 +44,66 @@ WORKLOADS = {
     "config1": dict(grid=(1, 40, 400, 352), per_batch=20000, gen="uniform", seed=1, ci=16, co=16,
                     dtype="float32", ks=(3, 3, 3),
                     text="BASELINE config 1: subm 3x3x3, 20000 uniform voxels in 1x40x400x352, Ci=Co=16 fp32"),
+    "config3": dict(grid=(4, 41, 1600, 1408), per_batch=30000, gen="clustered", seed=3, ci=64, co=64,
+                    dtype="bfloat16", ks=(3, 3, 3), sub_m=False, stride=(2, 2, 2), pad=(1, 1, 1),
+                    text="BASELINE config 3: regular 3x3x3 stride 2 pad 1, 4x30000 clustered voxels in "
+                         "4x41x1600x1408 -> 4x21x800x704, Ci=Co=64 bf16"),
     "config5a": dict(grid=(1, 64, 1024, 1024), per_batch=400000, gen="surface", seed=5, ci=128, co=128,
                      dtype="float16", ks=(5, 5, 5),
                      text="BASELINE config 5, first layer: subm 5x5x5, 400000 voxels on 50 planes and spheres "
                           "(5 % uniform noise) in 1x64x1024x1024, Ci=Co=128 fp16"),
+    "config5a_fp32": dict(grid=(1, 64, 1024, 1024), per_batch=400000, gen="surface", seed=5, ci=128, co=128,
+                          dtype="float32", ks=(5, 5, 5),
+                          text="BASELINE config 5, first layer in fp32: subm 5x5x5, 400000 voxels on 50 planes "
+                               "and spheres in 1x64x1024x1024, Ci=Co=128"),
+    "config5b": dict(grid=(1, 64, 1024, 1024), per_batch=400000, gen="surface", seed=5, ci=128, co=128,
+                     dtype="float16", ks=(2, 2, 2), sub_m=False, stride=(2, 2, 2), pad=(0, 0, 0),
+                     text="BASELINE config 5, second layer: regular 2x2x2 stride 2 pad 0 on the first layer's "
+                          "400000 output voxels, 1x64x1024x1024 -> 1x32x512x512, Ci=Co=128 fp16"),
+    "config5b_fp32": dict(grid=(1, 64, 1024, 1024), per_batch=400000, gen="surface", seed=5, ci=128, co=128,
+                          dtype="float32", ks=(2, 2, 2), sub_m=False, stride=(2, 2, 2), pad=(0, 0, 0),
+                          text="BASELINE config 5, second layer in fp32: regular 2x2x2 stride 2 pad 0, "
+                               "1x64x1024x1024 -> 1x32x512x512, Ci=Co=128"),
+    # the shapes the reference's design documents quote from a detection network
+    # (docs/design_docs/get_indice_pairs/get_indice_pairs.md:331-368,
+    # docs/design_docs/indice_convolution_forward/indice_convolution_forward.md:229-234)
+    "network_subm16": dict(grid=(4, 41, 1440, 1440), rows=248636, gen="scene", seed=11, ci=16, co=16,
+                           dtype="float16", ks=(3, 3, 3),
+                           text="network layer: subm 3x3x3, 248636 scene voxels (11 pairs a voxel) in "
+                                "4x41x1440x1440, Ci=Co=16 fp16"),
+    "network_subm64": dict(grid=(4, 41, 1440, 1440), rows=248636, gen="scene", seed=11, ci=64, co=64,
+                           dtype="float16", ks=(3, 3, 3),
+                           text="network layer: subm 3x3x3, 248636 scene voxels (11 pairs a voxel) in "
+                                "4x41x1440x1440, Ci=Co=64 fp16"),
+    "network_subm128": dict(grid=(4, 41, 1440, 1440), rows=248636, gen="scene", seed=11, ci=128, co=128,
+                            dtype="float16", ks=(3, 3, 3),
+                            text="network layer: subm 3x3x3, 248636 scene voxels (11 pairs a voxel) in "
+                                 "4x41x1440x1440, Ci=Co=128 fp16"),
+    "network_strided": dict(grid=(4, 11, 360, 360), rows=149100, gen="scene", seed=12, ci=64, co=128,
+                            dtype="float16", ks=(3, 3, 3), sub_m=False, stride=(2, 2, 2), pad=(0, 1, 1),
+                            scene=dict(sheet_frac=0.68, wall_frac=0.30),
+                            text="network layer: regular 3x3x3 stride 2 pad (0,1,1), 149100 scene voxels in "
+                                 "4x11x360x360 -> 4x5x180x180 (about 59000 outputs), 64 -> 128 channels fp16"),
 }
 
 
+def library_fingerprint():
+    """sha256 over the library's sources: what a committed counter summary was measured on."""
+    import hashlib
+    h = hashlib.sha256()
+    base = os.path.join(ROOT, "mlu-ops_amd")
+    files = [os.path.join(base, "Makefile")]
+    for d, _, names in sorted(os.walk(os.path.join(base, "csrc"))):
+        files += [os.path.join(d, n) for n in sorted(names)]
+    for f in files:
+        with open(f, "rb") as fh:
+            h.update(os.path.relpath(f, base).encode())
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 class Step:
-    """Descriptors, buffers and workspaces of one submanifold layer, built once."""
+    """Descriptors, buffers and workspaces of one sparse-convolution layer, built once."""
 
     def __init__(self, handle, wl):
         import numpy as np
@@ -60,6 +115,8 @@ class Step:
             idx = m.datagen.clustered_voxels(grid, wl["per_batch"], wl["seed"])
         elif wl["gen"] == "surface":
             idx = m.datagen.surface_voxels(grid, wl["per_batch"], wl["seed"])
+        elif wl["gen"] == "scene":
+            idx = m.datagen.scene_voxels(grid, wl["rows"], wl["seed"], **wl.get("scene", {}))
         else:
             idx = m.datagen.uniform_voxels(grid, wl["per_batch"] * grid[0], wl["seed"])
         self.idx_np = idx
@@ -68,36 +125,38 @@ class Step:
         K = ks[0] * ks[1] * ks[2]
         ci, co = wl["ci"], wl["co"]
         self.L, self.K, self.ci, self.co = L, K, ci, co
+        self.sub_m = wl.get("sub_m", True)
+        self.space = list(grid[1:])
+        self.stride = list(wl.get("stride", (1, 1, 1)))
+        self.pad = list(wl.get("pad", tuple(k // 2 for k in ks)))
+        self.out_space = self.space if self.sub_m else m.regular_output_space(
+            self.space, list(ks), self.pad, self.stride, [1, 1, 1])
         tdt = getattr(torch, wl["dtype"])
+        self.tdt = tdt
         self.elem = 4 if wl["dtype"] == "float32" else 2
         rng = np.random.default_rng(wl["seed"])
         self.feats_np = rng.standard_normal((L, ci)).astype(np.float32)
         self.w_np = m.datagen.kaiming_uniform_filters(ks, ci, co, wl["seed"])
-        self.dy_np = (rng.standard_normal((L, co)) * 0.1).astype(np.float32)
         dev = "cuda"
         self.indices = torch.from_numpy(idx).to(dev)
         self.features = torch.from_numpy(self.feats_np).to(dev, tdt)
         self.filters = torch.from_numpy(self.w_np).to(dev, tdt)
-        self.dy = torch.from_numpy(self.dy_np).to(dev, tdt)
         self.pairs = torch.empty((K, 2, L), dtype=torch.int32, device=dev)
-        self.out_indices = torch.empty((L, 4), dtype=torch.int32, device=dev)
+        out_cells = grid[0] * self.out_space[0] * self.out_space[1] * self.out_space[2]
+        self.out_rows = L if self.sub_m else min(out_cells, K * L)
+        self.out_indices = torch.empty((self.out_rows, 4), dtype=torch.int32, device=dev)
         self.indice_num = torch.empty((K,), dtype=torch.int32, device=dev)
-        self.out = torch.empty((L, co), dtype=tdt, device=dev)
-        self.dx = torch.empty((L, ci), dtype=tdt, device=dev)
-        self.dw = torch.empty(tuple(ks) + (ci, co), dtype=tdt, device=dev)
-        space = list(grid[1:])
-        pad = [k // 2 for k in ks]
+        self.num_pinned = torch.empty((K,), dtype=torch.int32).pin_memory()
         code = m.torch_dtype_code(tdt)
-        self.sdesc = m.SparseConvDescriptor(grid[0], pad, [1, 1, 1], [1, 1, 1], space, list(ks), space, 1)
+        self.code = code
+        self.sdesc = m.SparseConvDescriptor(grid[0], self.pad, self.stride, [1, 1, 1], self.space, list(ks),
+                                            self.out_space, 1 if self.sub_m else 0)
         self.d_idx = m.TensorDescriptor(m.LAYOUT_ARRAY, m.DTYPE_INT32, [L, 4])
         self.d_pairs = m.TensorDescriptor(m.LAYOUT_ARRAY, m.DTYPE_INT32, [K, 2, L])
-        self.d_oidx = m.TensorDescriptor(m.LAYOUT_ARRAY, m.DTYPE_INT32, [L, 4])
+        self.d_oidx = m.TensorDescriptor(m.LAYOUT_ARRAY, m.DTYPE_INT32, [self.out_rows, 4])
         self.d_num = m.TensorDescriptor(m.LAYOUT_ARRAY, m.DTYPE_INT32, [K])
         self.d_feat = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [L, ci])
         self.d_filt = m.TensorDescriptor(m.LAYOUT_ARRAY, code, list(ks) + [ci, co])
-        self.d_out = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [L, co])
-        self.d_dy = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [L, co])
-        self.d_dx = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [L, ci])
         self.d_dw = m.TensorDescriptor(m.LAYOUT_ARRAY, code, list(ks) + [ci, co], onchip_dtype=m.DTYPE_FLOAT)
         lib = m.lib()
         size = ctypes.c_size_t(0)
@@ -105,14 +164,23 @@ class Step:
                                                      self.d_oidx.ptr, self.d_num.ptr, ctypes.byref(size)))
         self.ws_rb_size = size.value
         self.ws_rb = torch.empty(max(size.value, 1), dtype=torch.uint8, device=dev)
-        # one rulebook build to learn indice_num (the host-side hand-off a framework does once per layer)
+        # one rulebook build to learn the shapes that depend on it
         self.rulebook()
-        torch.cuda.synchronize()
-        self.num_host = self.indice_num.cpu().tolist()
-        self.P = int(sum(self.num_host))
-        self.counts = (ctypes.c_int64 * K)(*self.num_host)
+        self.read_counts()
+        self.n_out = L if self.sub_m else self.sdesc.num_act_out()
+        self.P = int(sum(self.counts))
+        n_out = self.n_out
+        self.dy_np = (rng.standard_normal((n_out, co)) * 0.1).astype(np.float32)
+        self.dy = torch.from_numpy(self.dy_np).to(dev, tdt)
+        self.out = torch.empty((n_out, co), dtype=tdt, device=dev)
+        self.dx = torch.empty((L, ci), dtype=tdt, device=dev)
+        self.dw = torch.empty(tuple(ks) + (ci, co), dtype=tdt, device=dev)
+        self.d_out = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [n_out, co])
+        self.d_dy = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [n_out, co])
+        self.d_dx = m.TensorDescriptor(m.LAYOUT_ARRAY, code, [L, ci])
+        sm = 1 if self.sub_m else 0
         m.check(lib.mluOpGetIndiceConvolutionForwardWorkspaceSize(
-            handle.ptr, self.d_feat.ptr, self.d_filt.ptr, self.d_pairs.ptr, self.d_out.ptr, self.counts, L, 0, 1,
+            handle.ptr, self.d_feat.ptr, self.d_filt.ptr, self.d_pairs.ptr, self.d_out.ptr, self.counts, n_out, 0, sm,
             ctypes.byref(size)))
         self.ws_fwd_size = size.value
         self.ws_fwd = torch.empty(max(size.value, 1), dtype=torch.uint8, device=dev)
@@ -122,7 +190,7 @@ class Step:
         self.ws_bd_size = size.value
         self.ws_bd = torch.empty(max(size.value, 1), dtype=torch.uint8, device=dev)
         m.check(lib.mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize(
-            handle.ptr, self.d_feat.ptr, self.d_dy.ptr, self.d_pairs.ptr, self.d_dw.ptr, self.counts, 0, 1,
+            handle.ptr, self.d_feat.ptr, self.d_dy.ptr, self.d_pairs.ptr, self.d_dw.ptr, self.counts, 0, sm,
             ctypes.byref(size)))
         self.ws_bf_size = size.value
         self.ws_bf = torch.empty(max(size.value, 1), dtype=torch.uint8, device=dev)
@@ -134,37 +202,45 @@ class Step:
             self.ws_rb_size, self.d_pairs.ptr, self.pairs.data_ptr(), self.d_oidx.ptr, self.out_indices.data_ptr(),
             self.d_num.ptr, self.indice_num.data_ptr()), "mluOpGetIndicePairs")
 
+    def read_counts(self):
+        """The hand-off the API prescribes between the rulebook and the convolutions: indice_num
+        leaves the device and becomes the host array of 64-bit counts the operators take."""
+        self.num_pinned.copy_(self.indice_num, non_blocking=True)
+        self.torch.cuda.current_stream().synchronize()
+        self.counts = (ctypes.c_int64 * self.K)(*self.num_pinned.tolist())
+
     def forward(self):
         m = self.m
         m.check(m.lib().mluOpIndiceConvolutionForward(
             self.handle.ptr, self.d_feat.ptr, self.features.data_ptr(), self.d_filt.ptr, self.filters.data_ptr(),
-            self.d_pairs.ptr, self.pairs.data_ptr(), self.counts, self.L, 0, 1, self.ws_fwd.data_ptr(),
-            self.ws_fwd_size, self.d_out.ptr, self.out.data_ptr()), "mluOpIndiceConvolutionForward")
+            self.d_pairs.ptr, self.pairs.data_ptr(), self.counts, self.n_out, 0, 1 if self.sub_m else 0,
+            self.ws_fwd.data_ptr(), self.ws_fwd_size, self.d_out.ptr, self.out.data_ptr()),
+            "mluOpIndiceConvolutionForward")
 
     def backward_data(self):
         m = self.m
         m.check(m.lib().mluOpIndiceConvolutionBackwardData(
             self.handle.ptr, self.d_dy.ptr, self.dy.data_ptr(), self.d_filt.ptr, self.filters.data_ptr(),
-            self.d_pairs.ptr, self.pairs.data_ptr(), self.counts, 0, 1, self.ws_bd.data_ptr(), self.ws_bd_size,
-            self.d_dx.ptr, self.dx.data_ptr()), "mluOpIndiceConvolutionBackwardData")
+            self.d_pairs.ptr, self.pairs.data_ptr(), self.counts, 0, 1 if self.sub_m else 0, self.ws_bd.data_ptr(),
+            self.ws_bd_size, self.d_dx.ptr, self.dx.data_ptr()), "mluOpIndiceConvolutionBackwardData")
 
     def backward_filter(self):
         m = self.m
         m.check(m.lib().mluOpIndiceConvolutionBackwardFilter(
             self.handle.ptr, self.d_feat.ptr, self.features.data_ptr(), self.d_dy.ptr, self.dy.data_ptr(),
-            self.d_pairs.ptr, self.pairs.data_ptr(), self.counts, 0, 1, self.ws_bf.data_ptr(), self.ws_bf_size,
-            self.d_dw.ptr, self.dw.data_ptr()), "mluOpIndiceConvolutionBackwardFilter")
+            self.d_pairs.ptr, self.pairs.data_ptr(), self.counts, 0, 1 if self.sub_m else 0, self.ws_bf.data_ptr(),
+            self.ws_bf_size, self.d_dw.ptr, self.dw.data_ptr()), "mluOpIndiceConvolutionBackwardFilter")
 
     # algorithmic work (per call)
     def conv_flops(self):
         return 2.0 * self.P * self.ci * self.co
 
     def rulebook_bytes(self):
-        return 16.0 * self.L + 8.0 * self.K * self.L + 4.0 * self.K + 16.0 * self.L
+        return 16.0 * self.L + 8.0 * self.K * self.L + 4.0 * self.K + 16.0 * self.n_out
 
     def forward_bytes(self):
         s = self.elem
-        return self.L * self.ci * s + self.L * self.co * s + self.K * self.ci * self.co * s + 8.0 * self.P
+        return self.L * self.ci * s + self.n_out * self.co * s + self.K * self.ci * self.co * s + 8.0 * self.P
 
 
 def median(v):
@@ -190,32 +266,43 @@ def time_ops(torch, ops, steps):
     return wall, per
 
 
-def cpu_baseline(step, reps=3):
+def cpu_baseline(step):
     """The CPU oracle (plain-C restatement of the reference's cpuCompute) on the same workload,
-    one thread: rulebook, then forward on the device-rounded inputs."""
+    one thread: rulebook, then forward on the device-rounded inputs.  Workloads whose forward is
+    more than a few seconds of CPU work are timed once, and on a prefix of the pairs of every offset
+    (the oracle's cost is linear in the pairs)."""
     import numpy as np
     import sparse_conv_oracle as oracle
     wl = step.wl
-    space = list(wl["grid"][1:])
     ks = list(wl["ks"])
-    pad = [k // 2 for k in ks]
-    rnd = oracle.round_through_half if wl["dtype"] == "float16" else (lambda a: a)
+    if wl["dtype"] == "float16":
+        rnd = oracle.round_through_half
+    elif wl["dtype"] == "bfloat16":
+        rnd = oracle.round_through_bf16
+    else:
+        rnd = lambda a: a
     feats, w = rnd(step.feats_np), rnd(step.w_np).reshape(step.K, step.ci, step.co)
+    macs = float(step.P) * step.ci * step.co
+    reps = 3 if macs < 3e9 else 1
+    keep = 1.0 if macs < 6e10 else 6e10 / macs   # at most about 15 s of forward
     t_rb, t_fw = [], []
     for _ in range(reps):
         t0 = time.perf_counter()
-        pairs, oidx, num, n_out = oracle.get_indice_pairs(step.idx_np, wl["grid"][0], pad, [1, 1, 1], [1, 1, 1],
-                                                          ks, space, True)
+        pairs, oidx, num, n_out = oracle.get_indice_pairs(step.idx_np, wl["grid"][0], step.pad, step.stride,
+                                                          [1, 1, 1], ks, step.out_space, step.sub_m)
         t1 = time.perf_counter()
-        oracle.forward(feats, w, pairs, num, n_out)
+        num_s = np.maximum((np.asarray(num) * keep).astype(np.asarray(num).dtype), np.minimum(num, 1))
+        t1b = time.perf_counter()
+        oracle.forward(feats, w, pairs, num_s, n_out)
         t2 = time.perf_counter()
         t_rb.append(t1 - t0)
-        t_fw.append(t2 - t1)
-    P = int(np.sum(num))
+        t_fw.append(t2 - t1b)
+    P_timed = int(np.sum(num_s))
     fw, rb = median(t_fw), median(t_rb)
-    return {"value": 2.0 * P * step.ci * step.co / fw / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
-            "sample": "full workload (%d voxels, %d pairs), median of %d runs, gcc -O2 single thread, "
-                      "host has %d logical cores" % (step.L, P, reps, os.cpu_count()),
+    sample = "full workload" if keep == 1.0 else "rulebook in full, forward on the first %.0f %% of every offset's pairs" % (keep * 100)
+    return {"value": 2.0 * P_timed * step.ci * step.co / fw / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": "%s (%d voxels, %d pairs timed), median of %d, gcc -O2 single thread, host has %d logical "
+                      "cores" % (sample, step.L, P_timed, reps, os.cpu_count()),
             "forward_ms": fw * 1e3, "rulebook_ms": rb * 1e3,
             "rulebook_mvoxels_per_s": step.L / rb / 1e6}
 
@@ -254,14 +341,18 @@ def graph_replay_step(torch, m, handle, step, step_ops, steps):
 
 
 def measured_traffic(workload, kernel):
-    """HBM bytes per launch of `kernel` from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary
-    of this workload (counters cannot be read from inside the process), or None."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "pmc_traffic_%s.json" % workload)
+    """(HBM bytes per launch of `kernel`, note) from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE
+    summary of this workload (counters cannot be read from inside the process).  The summary names
+    the library sources it was measured on; for other sources the figure is withheld."""
+    path = os.path.join(ROOT, "profiles", "pmc_traffic_%s.json" % workload)
     try:
         with open(path) as f:
-            return json.load(f)["kernels"][kernel]["total_bytes"]
+            doc = json.load(f)
+        if doc.get("library_fingerprint") != library_fingerprint():
+            return None, "profiles/pmc_traffic_%s.json was measured on other library sources" % workload
+        return doc["kernels"][kernel]["total_bytes"], None
     except (OSError, KeyError, ValueError):
-        return None
+        return None, "no counter summary for this kernel and workload"
 
 
 UPSTREAM = {
@@ -422,7 +513,9 @@ def main():
         return
     wl = WORKLOADS[args.workload]
     step = Step(handle, wl)
-    step_ops = [("get_indice_pairs", step.rulebook), ("forward", step.forward)]
+    # The step as the API prescribes it: the rulebook, the copy of indice_num to the host (the
+    # convolutions take it as a host array), the forward convolution.
+    step_ops = [("get_indice_pairs", step.rulebook), ("read_counts", step.read_counts), ("forward", step.forward)]
 
     for _ in range(args.warmup):
         for _, fn in step_ops:
@@ -430,17 +523,26 @@ def main():
     torch.cuda.synchronize()
 
     # timed region: exactly --steps steps
-    wall, per = time_ops(torch, step_ops, args.steps)
+    wall, _ = time_ops(torch, step_ops, args.steps)
     ms_per_step = wall * 1e3 / args.steps
+    # Device time of the two operators: the same number of calls of each, back to back, events on
+    # the handle's stream between them.  (Inside a step the forward call follows a wait for the
+    # queue, so an event pair around it there would also count the host's way to the first launch.)
+    _, per_rb = time_ops(torch, [("get_indice_pairs", step.rulebook)], args.steps)
+    step.read_counts()
+    _, per_fw = time_ops(torch, [("forward", step.forward)], args.steps)
+    per = {"forward": per_fw["forward"], "get_indice_pairs": per_rb["get_indice_pairs"]}
     fwd_ms = sum(per["forward"]) / args.steps
     rb_ms = sum(per["get_indice_pairs"]) / args.steps
     result = {
         "metric": METRIC, "value": step.conv_flops() / (fwd_ms * 1e-3) / 1e12, "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if wl["dtype"] == "float32" else "f16", "data": "synthetic",
-        "config": {"workload": wl["text"] + "; step = get_indice_pairs + indice_convolution_forward",
-                   "voxels": step.L, "pairs": step.P, "Ci": step.ci, "Co": step.co, "kernel_volume": step.K},
+        "dtype": {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[wl["dtype"]], "data": "synthetic",
+        "config": {"workload": wl["text"] + "; step = get_indice_pairs + copy of indice_num to the host + "
+                               "indice_convolution_forward",
+                   "voxels": step.L, "outputs": step.n_out, "pairs": step.P, "Ci": step.ci, "Co": step.co,
+                   "kernel_volume": step.K},
         "rulebook_mvoxels_per_s": step.L / (rb_ms * 1e-3) / 1e6,
         "forward_ms": fwd_ms, "forward_ms_min": min(per["forward"]),
         "rulebook_ms": rb_ms, "rulebook_ms_min": min(per["get_indice_pairs"]),
@@ -479,17 +581,31 @@ def main():
         alg_bytes, what = step.rulebook_bytes(), "rulebook bytes 16L + 8KL + 4K + 16N_out"
     else:
         alg_bytes, what = step.forward_bytes(), "forward bytes L*Ci*s + N*Co*s + K*Ci*Co*s + 8P"
-    achieved = alg_bytes / (dom_ms * 1e-3) / 1e9
-    result["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(args.workload, dominant),
-                          "kernel": dominant,
-                          "kernel_avg_us": dom_ms * 1e3, "algorithmic_bytes": alg_bytes, "bytes_model": what}
-    if "gatherConvMfma" in agg:
-        g_ms = agg["gatherConvMfma"][0] / agg["gatherConvMfma"][1]
+    # The bound that binds: a kernel that moves more than 312 FLOP per algorithmic byte (2.5 PFLOP/s
+    # over 8 TB/s) is priced against the matrix cores, any other against HBM.
+    mfma_peak = MFMA_F32_PEAK_TFLOPS if wl["dtype"] == "float32" else MFMA_F16_PEAK_TFLOPS
+    traffic, traffic_note = measured_traffic(args.workload, dominant)
+    if not dominant.startswith("rb") and step.conv_flops() / alg_bytes > mfma_peak * 1e12 / (HBM_PEAK_GBS * 1e9):
+        achieved = step.conv_flops() / (dom_ms * 1e-3) / 1e12
+        result["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": mfma_peak, "unit": "TFLOP/s",
+                              "frac": achieved / mfma_peak, "traffic": traffic, "kernel": dominant,
+                              "kernel_avg_us": dom_ms * 1e3, "algorithmic_flops": step.conv_flops(),
+                              "algorithmic_bytes": alg_bytes}
+    else:
+        achieved = alg_bytes / (dom_ms * 1e-3) / 1e9
+        result["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": dominant,
+                              "kernel_avg_us": dom_ms * 1e3, "algorithmic_bytes": alg_bytes, "bytes_model": what}
+    if traffic_note:
+        result["roofline"]["traffic_note"] = traffic_note
+    gather = [n for n in agg if n.startswith("gatherConv")]
+    if gather:
+        g = max(gather, key=lambda n: agg[n][0])
+        g_ms = agg[g][0] / agg[g][1]
         result["forward_kernel"] = {
-            "kernel": "gatherConvMfma", "avg_us": g_ms * 1e3,
+            "kernel": g, "avg_us": g_ms * 1e3,
             "hbm_frac": step.forward_bytes() / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "mfma_frac": step.conv_flops() / (g_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS}
+            "mfma_frac": step.conv_flops() / (g_ms * 1e-3) / 1e12 / mfma_peak}
 
     # the two backward operators of the same layer, reported beside the metric
     _, per_b = time_ops(torch, [("backward_data", step.backward_data), ("backward_filter", step.backward_filter)],
@@ -509,25 +625,16 @@ def main():
     result["backward_data_tflops"] = step.conv_flops() / (result["backward_data_ms"] * 1e-3) / 1e12
     result["backward_filter_tflops"] = step.conv_flops() / (result["backward_filter_ms"] * 1e-3) / 1e12
 
-    result["graph_replay"] = graph_replay_step(torch, m, handle, step, step_ops, args.steps)
-    # Not part of the metric: the forward operator for a caller that promises distinct pairs, which
-    # spares the kernel that checks for pairs of one offset sharing a result row.
-    handle.promise_distinct_pairs(True)
-    _, per_p = time_ops(torch, [("forward", step.forward)], max(args.steps // 2, 5))
-    handle.promise_distinct_pairs(False)
-    result["forward_ms_distinct_pairs_promised"] = median(per_p["forward"])
-    # Nor is this: the forward operator handed the row map of its rulebook, built once ahead
-    # (mluOpExtBuildRowMap), as layers that share a rulebook can; it then launches neither the
-    # map kernels nor that check.
-    row_map = m.RowMap(handle, step.pairs, list(step.counts), step.L, step.L, 1)
-
-    def forward_with_map():
-        row_map.announce()
-        step.forward()
-
-    _, per_m = time_ops(torch, [("forward", forward_with_map)], max(args.steps // 2, 5))
-    result["forward_ms_row_map_kept"] = median(per_m["forward"]) if row_map.usable else None
-    row_map.close()
+    # Not part of the metric: the step without the copy of indice_num (a caller that kept the counts
+    # of an identical rulebook).  The forward operator then cannot know yet whether the rulebook's
+    # input rows were in cell order and takes the way that assumes nothing.
+    wall_nr, per_nr = time_ops(torch, [("get_indice_pairs", step.rulebook), ("forward", step.forward)],
+                               max(args.steps // 2, 5))
+    result["without_count_readback"] = {"ms_per_step": wall_nr * 1e3 / max(args.steps // 2, 5),
+                                        "forward_ms": median(per_nr["forward"])}
+    if step.sub_m:
+        result["graph_replay"] = graph_replay_step(
+            torch, m, handle, step, [("get_indice_pairs", step.rulebook), ("forward", step.forward)], args.steps)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(step)
     print(json.dumps(result))

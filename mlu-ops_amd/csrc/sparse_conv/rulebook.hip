@@ -37,7 +37,8 @@ constexpr int kWave = 64;
 constexpr uint32_t kEmptyKey = 0xffffffffu;  // no cell index reaches 2^31
 constexpr int kGroup = 8;                    // offsets resolved together per lane
 constexpr int kMaxInlineOffsets = 128;       // kernel volumes with an in-argument offset table
-constexpr int kWordsPerBlock = 1024;  // bitmap words (64 cells each) per block
+constexpr int kWordsPerBlock = 256;  // bitmap words (64 cells each) per block, one a thread
+constexpr int kSelfScanBlocks = 4096;  // up to here every workgroup sums the block counts in front of it
 
 // Division of a non-negative int by a divisor fixed for the launch:
 // n / d = (n * mul) >> (31 + shift) for every 0 <= n < 2^31, with shift = ceil(log2 d)
@@ -164,28 +165,6 @@ __global__ __launch_bounds__(kBlock) void rbFill(FillRanges r, int32_t *rows_in_
   }
 }
 
-// Kernel offsets (kd, kh, kw) of offset index k.  Small kernel volumes carry a
-// table in the kernel arguments; larger ones are decoded by division.
-struct OffsetTable {
-  uint32_t packed[kMaxInlineOffsets];  // kd | kh << 8 | kw << 16
-};
-
-__device__ __forceinline__ void decodeOffset(const OffsetTable &tab, const GeomDev &g, int k,
-                                             int *kd, int *kh, int *kw) {
-  if (g.K <= kMaxInlineOffsets) {
-    const uint32_t p = tab.packed[k];
-    *kd = p & 0xff;
-    *kh = (p >> 8) & 0xff;
-    *kw = p >> 16;
-  } else {
-    const int hw = g.ks[1] * g.ks[2];
-    *kd = k / hw;
-    const int rem = k - *kd * hw;
-    *kh = rem / g.ks[2];
-    *kw = rem - *kh * g.ks[2];
-  }
-}
-
 // Open-addressing table over linear cell indices: keys[] holds the cell (or
 // kEmptyKey), vals[] the highest row index stored for that cell.  32-bit
 // atomics only: a 64-bit compare-and-swap costs several times more here.
@@ -275,12 +254,12 @@ __device__ __forceinline__ void stagePairs(const int (&res)[N], int k_first, int
 // cell, marked in the bitmap), store it as a candidate at [k][row] and record
 // how many lanes of the wave produced one.
 template <bool SUBM>
-__global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable tab,
+__global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g,
                                                        const int32_t *indices, bool aligned,
                                                        const uint32_t *keys, const int32_t *vals,
                                                        uint32_t mask, unsigned long long *bitmap,
                                                        Staging staging, int k_per_slice,
-                                                       int32_t *rows_in_order) {
+                                                       int32_t *rows_in_order, int32_t *pairs) {
   const int j = blockIdx.x * kBlock + threadIdx.x;
   // blockIdx.y selects a slice of the offsets: more waves in flight than rows alone give
   const int k_lo = blockIdx.y * k_per_slice;
@@ -291,6 +270,16 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
   if (active) c = loadCoord(indices, j, aligned);
   if (!SUBM && active && blockIdx.y == 0) noteRowOrder(indices, j, c, aligned, rows_in_order);
   const bool n_ok = active && (unsigned)c.x < (unsigned)g.batch;
+  // (kd, kh, kw) of the slice's first offset, advanced by one offset a step: all of it
+  // the same for every lane
+  int kd = k_lo / (g.ks[1] * g.ks[2]);
+  int kh = (k_lo - kd * g.ks[1] * g.ks[2]) / g.ks[2];
+  int kw = k_lo - (kd * g.ks[1] + kh) * g.ks[2];
+  // The cell of (row, offset) is plane + ow: `plane` (the cell of w = 0 in the output line,
+  // or -1 when (kd, kh) has no output line for this row) is computed again only when kh or
+  // kd changes, once in ks[2] offsets.
+  int base_d = 0, plane = -1;
+  bool new_d = true, new_h = true;
   for (int k0 = k_lo; k0 < k_hi; k0 += kGroup) {
     uint32_t cell[kGroup];
     int res[kGroup];
@@ -300,13 +289,27 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
       res[u] = -1;
       const int k = k0 + u;
       if (k < k_hi) {
-        int kd, kh, kw;
-        decodeOffset(tab, g, k, &kd, &kh, &kw);
-        const int od = axisOut(c.y, g.pad[0], kd, g.dil[0], g.stride[0], g.by_stride[0], g.out[0]);
-        const int oh = axisOut(c.z, g.pad[1], kh, g.dil[1], g.stride[1], g.by_stride[1], g.out[1]);
+        if (new_d) {
+          const int od = axisOut(c.y, g.pad[0], kd, g.dil[0], g.stride[0], g.by_stride[0], g.out[0]);
+          base_d = n_ok && od >= 0 ? (c.x * g.out[0] + od) * g.out[1] : -1;
+        }
+        if (new_h) {
+          const int oh = axisOut(c.z, g.pad[1], kh, g.dil[1], g.stride[1], g.by_stride[1], g.out[1]);
+          plane = base_d >= 0 && oh >= 0 ? (base_d + oh) * g.out[2] : -1;
+        }
         const int ow = axisOut(c.w, g.pad[2], kw, g.dil[2], g.stride[2], g.by_stride[2], g.out[2]);
-        if (n_ok && (od | oh | ow) >= 0)
-          cell[u] = (uint32_t)(((c.x * g.out[0] + od) * g.out[1] + oh) * g.out[2] + ow);
+        if ((plane | ow) >= 0) cell[u] = (uint32_t)(plane + ow);
+        new_d = false;
+        new_h = false;
+        if (++kw == g.ks[2]) {
+          kw = 0;
+          new_h = true;
+          if (++kh == g.ks[1]) {
+            kh = 0;
+            ++kd;
+            new_d = true;
+          }
+        }
       }
     }
     if (SUBM) {
@@ -345,14 +348,57 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g, OffsetTable ta
         if (hit & (1u << u)) res[u] = vals[slot[u]];
       }
     } else {
+      // Rows in cell order walk along w, so the lanes of a wavefront mark runs of cells
+      // in the same bitmap word: a run's bits are gathered at its last lane, which alone
+      // goes to memory (atomics on the bitmap are what this kernel would wait for).  Lanes
+      // with no output cell join the run in front of them; a lane whose word is below one
+      // in front of it (rows out of order) marks its cell by itself.
+      const int lane = threadIdx.x & (kWave - 1);
+      uint32_t word_at[kGroup];
+      unsigned long long bits[kGroup];
+      uint32_t alone = 0;
 #pragma unroll
       for (int u = 0; u < kGroup; ++u) {
-        if (cell[u] != kEmptyKey) {
-          res[u] = (int)cell[u];
-          const unsigned long long bit = 1ull << (cell[u] & 63);
-          unsigned long long *word = bitmap + (cell[u] >> 6);
-          if ((__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & bit) == 0)
-            atomicOr(word, bit);
+        const bool valid = cell[u] != kEmptyKey;
+        if (valid) res[u] = (int)cell[u];
+        const uint32_t mine = cell[u] >> 6;
+        const uint32_t run = waveInclusiveMax(valid ? mine : 0u);
+        const bool joins = valid && run == mine;
+        if (valid && !joins) alone |= 1u << u;
+        uint32_t lo = 0, hi = 0;
+        if (joins) {
+          lo = (cell[u] & 32u) ? 0u : 1u << (cell[u] & 31u);
+          hi = (cell[u] & 32u) ? 1u << (cell[u] & 31u) : 0u;
+        }
+        waveRunInclusiveOr(run, &lo, &hi);
+        const uint32_t run_next = __shfl_down(run, 1, kWave);
+        const bool last = lane == kWave - 1 || run_next != run;
+        word_at[u] = run;
+        bits[u] = last ? ((unsigned long long)hi << 32) | lo : 0ull;
+      }
+      // (a stale word from the cache only costs an atomic that changes nothing)
+      unsigned long long seen[kGroup];
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) seen[u] = bits[u] ? bitmap[word_at[u]] : ~0ull;
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u)
+        if ((seen[u] & bits[u]) != bits[u]) atomicOr(bitmap + word_at[u], bits[u]);
+      if (__any(alone != 0)) {
+#pragma unroll
+        for (int u = 0; u < kGroup; ++u) {
+          if (alone & (1u << u)) {
+            const unsigned long long bit = 1ull << (cell[u] & 63);
+            unsigned long long *word = bitmap + (cell[u] >> 6);
+            if ((*word & bit) == 0) atomicOr(word, bit);
+          }
+        }
+      }
+      // every pair slot of this row and these offsets starts out as -1; the kernel that
+      // places the pairs overwrites the front of each list afterwards
+      if (active) {
+        for (int k = k0; k < k0 + kGroup && k < k_hi; ++k) {
+          pairs[(size_t)(2 * k) * g.L + j] = -1;
+          pairs[(size_t)(2 * k + 1) * g.L + j] = -1;
         }
       }
     }
@@ -577,6 +623,8 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
   }
 }
 
+// ---- regular mode: ranks of marked cells -----------------------------------
+
 // Exclusive prefix sum over `n` ints per row of `data` (one block of 1024
 // threads per row, four consecutive elements per thread and pass), the row
 // total goes to totals[row].
@@ -621,88 +669,104 @@ __global__ __launch_bounds__(kScanBlock) void rbScanRows(int32_t *data, int n, i
   if (threadIdx.x == 0) totals[blockIdx.x] = carry;
 }
 
-// ---- regular mode: ranks of marked cells -----------------------------------
-
+// Marked cells per block of kWordsPerBlock bitmap words, one word a thread.
 __global__ __launch_bounds__(kBlock) void rbBitmapBlockSum(const unsigned long long *bitmap,
                                                            size_t n_words, int32_t *block_sum) {
   __shared__ int s_wsum[kBlock / kWave];
-  const size_t base = (size_t)blockIdx.x * kWordsPerBlock;
-  int cnt = 0;
+  const size_t w = (size_t)blockIdx.x * kWordsPerBlock + threadIdx.x;
+  int cnt = w < n_words ? __popcll(bitmap[w]) : 0;
 #pragma unroll
-  for (int i = 0; i < kWordsPerBlock / kBlock; ++i) {
-    size_t w = base + (size_t)i * kBlock + threadIdx.x;
-    if (w < n_words) cnt += __popcll(bitmap[w]);
-  }
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) cnt += __shfl_down(cnt, off, kWave);
+  for (int off = kWave / 2; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off, kWave);
   if ((threadIdx.x & (kWave - 1)) == 0) s_wsum[threadIdx.x >> 6] = cnt;
   __syncthreads();
   if (threadIdx.x == 0) {
     int t = 0;
-    for (int w = 0; w < kBlock / kWave; ++w) t += s_wsum[w];
+    for (int x = 0; x < kBlock / kWave; ++x) t += s_wsum[x];
     block_sum[blockIdx.x] = t;
   }
 }
 
 // Per bitmap word: number of marked cells before it (word_rank).  Every marked
-// cell is decoded to (n, d, h, w) and written at its rank; rows from
-// num_act_out up to out_rows are set to -1.
+// cell is decoded to (n, d, h, w) and written at its rank.  A thread owns one word; where
+// a wavefront's 64 words hold many cells (a small dense grid) the wavefront decodes them
+// word by word, a lane per cell, instead of each lane walking its own word's bits.  Rows
+// of out_indices from the number of marked cells on are left as the caller passed them,
+// as the reference's decode kernel leaves them (normal_get_indice_pairs.cpp:1143-1150).
+// block_count holds the marked cells of every block of kWordsPerBlock words: either as
+// counted, then each workgroup sums the counts in front of its block itself and the last
+// one writes the total to num_act_out, or, for bitmaps of more blocks than that is worth,
+// already scanned (`scanned`, total already in num_act_out).
 __global__ __launch_bounds__(kBlock) void rbRankAndDecode(GeomDev g,
                                                           const unsigned long long *bitmap,
                                                           size_t n_words,
-                                                          const int32_t *block_excl,
-                                                          const int32_t *num_act_out,
+                                                          const int32_t *block_count,
+                                                          bool scanned, int32_t *num_act_out,
                                                           uint32_t *word_rank,
                                                           int32_t *out_indices, bool aligned,
                                                           int out_rows) {
   __shared__ int s_wsum[kBlock / kWave];
-  constexpr int kPerThread = kWordsPerBlock / kBlock;  // consecutive words of one thread
-  static_assert(kPerThread == 4, "one 32-byte load and one 16-byte rank store per thread");
+  static_assert(kWordsPerBlock == kBlock, "one bitmap word per thread");
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
-  const size_t w0 = (size_t)blockIdx.x * kWordsPerBlock + (size_t)threadIdx.x * kPerThread;
+  __shared__ int s_front[kBlock / kWave];
+  int front = 0;  // marked cells in the blocks before this one
+  if (scanned) {
+    front = block_count[blockIdx.x];
+  } else {
+    int part = 0;
+    for (int i = threadIdx.x; i < (int)blockIdx.x; i += kBlock) part += block_count[i];
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, kWave);
+    if (lane == 0) s_front[wave] = part;
+  }
+  const size_t w = (size_t)blockIdx.x * kWordsPerBlock + threadIdx.x;
   const int hw = g.out[1] * g.out[2];
   const int vol = g.out[0] * hw;
-  unsigned long long bits[kPerThread];
-  int mine = 0;
-#pragma unroll
-  for (int i = 0; i < kPerThread; ++i) {
-    bits[i] = w0 + i < n_words ? bitmap[w0 + i] : 0ull;
-    mine += __popcll(bits[i]);
-  }
+  const unsigned long long bits = w < n_words ? bitmap[w] : 0ull;
+  const int mine = __popcll(bits);
   const int incl = waveInclusiveScan(mine);
   if (lane == kWave - 1) s_wsum[wave] = incl;
   __syncthreads();
-  int rank = block_excl[blockIdx.x] + incl - mine;
+  if (!scanned) {
+#pragma unroll
+    for (int x = 0; x < kBlock / kWave; ++x) front += s_front[x];
+  }
+  int rank = front + incl - mine;
 #pragma unroll
   for (int x = 0; x < kBlock / kWave; ++x)
     if (x < wave) rank += s_wsum[x];
-#pragma unroll
-  for (int i = 0; i < kPerThread; ++i) {
-    if (w0 + i < n_words) word_rank[w0 + i] = (uint32_t)rank;
-    unsigned long long b = bits[i];
+  if (!scanned && blockIdx.x == gridDim.x - 1 && threadIdx.x == kBlock - 1) *num_act_out = rank + mine;
+  if (w < n_words) word_rank[w] = (uint32_t)rank;
+  auto put = [&](size_t cell64, int r) {
+    if (r >= out_rows) return;
+    int cell = (int)cell64;
+    int4 o;
+    o.x = fastDiv(cell, g.by_out_volume);
+    cell -= o.x * vol;
+    o.y = fastDiv(cell, g.by_out_plane);
+    cell -= o.y * hw;
+    o.z = fastDiv(cell, g.by_out_width);
+    o.w = cell - o.z * g.out[2];
+    storeCoord(out_indices, r, o, aligned);
+  };
+  const int wave_cells = __shfl(incl, kWave - 1, kWave);
+  if (wave_cells > 4 * kWave) {
+    unsigned long long todo = __ballot(bits != 0ull);
+    const size_t w_first = w - lane;
+    while (todo) {
+      const int src = __ffsll((long long)todo) - 1;
+      todo &= todo - 1;
+      const unsigned long long b = __shfl(bits, src, kWave);
+      const int r0 = __shfl(rank, src, kWave);
+      if ((b >> lane) & 1ull) put((w_first + src) * 64 + lane, r0 + __popcll(b & ((1ull << lane) - 1ull)));
+    }
+  } else {
+    unsigned long long b = bits;
     while (b) {
       const int bit = __ffsll((long long)b) - 1;
       b &= b - 1;
-      if (rank < out_rows) {
-        int cell = (int)((w0 + i) * 64 + bit);
-        int4 o;
-        o.x = fastDiv(cell, g.by_out_volume);
-        cell -= o.x * vol;
-        o.y = fastDiv(cell, g.by_out_plane);
-        cell -= o.y * hw;
-        o.z = fastDiv(cell, g.by_out_width);
-        o.w = cell - o.z * g.out[2];
-        storeCoord(out_indices, rank, o, aligned);
-      }
-      ++rank;
+      put(w * 64 + bit, rank++);
     }
-  }
-  const int n_out = *num_act_out;
-  const size_t gstride = (size_t)gridDim.x * kBlock;
-  for (size_t r = (size_t)n_out + (size_t)blockIdx.x * kBlock + threadIdx.x; r < (size_t)out_rows;
-       r += gstride) {
-    storeCoord(out_indices, (int)r, make_int4(-1, -1, -1, -1), aligned);
   }
 }
 
@@ -789,18 +853,6 @@ inline uint32_t tableCapacity(int L) {
   return cap;
 }
 
-OffsetTable makeOffsetTable(const RulebookGeom &g) {
-  OffsetTable t;
-  for (int k = 0; k < kMaxInlineOffsets; ++k) t.packed[k] = 0;
-  if (g.K <= kMaxInlineOffsets) {
-    int k = 0;
-    for (int kd = 0; kd < g.ksize[0]; ++kd)
-      for (int kh = 0; kh < g.ksize[1]; ++kh)
-        for (int kw = 0; kw < g.ksize[2]; ++kw, ++k)
-          t.packed[k] = (uint32_t)kd | ((uint32_t)kh << 8) | ((uint32_t)kw << 16);
-  }
-  return t;
-}
 
 struct Workspace {
   // submanifold
@@ -849,6 +901,7 @@ Workspace carve(const RulebookGeom &g, void *base) {
     ws.word_rank = reinterpret_cast<uint32_t *>(take(ws.n_words * 4));
     ws.block_sum = reinterpret_cast<int32_t *>(take((size_t)ws.n_bitmap_blocks * 4));
     ws.num_act_out = reinterpret_cast<int32_t *>(take(4));
+
   }
   ws.stage = reinterpret_cast<int32_t *>(take((size_t)g.K * g.L * 4));
   if (!g.sub_m) ws.stage_lane = reinterpret_cast<uint8_t *>(take((size_t)g.K * g.L));
@@ -961,11 +1014,10 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
       lc.end();
     }
   } else {
-    const OffsetTable tab = makeOffsetTable(g);
     lc.begin("rbProbeCount");
-    rbProbeCount<true><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al, ws.keys, ws.vals,
+    rbProbeCount<true><<<slice_grid, kBlock, 0, lc.stream>>>(d, indices, al, ws.keys, ws.vals,
                                                              mask, nullptr, staging, k_per,
-                                                             ws.rows_in_order);
+                                                             ws.rows_in_order, nullptr);
     lc.end();
   }
   lc.begin("rbPlacePairs");
@@ -985,15 +1037,11 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
   const bool al_out = aligned16(out_indices, out_indices);
   const int l_blocks = (g.L + kBlock - 1) / kBlock;
 
-  const OffsetTable tab = makeOffsetTable(g);
-  // bitmap 0, every pair slot -1
+  // bitmap 0
   FillRanges fill = {};
   fill.dst[0] = reinterpret_cast<uint32_t *>(ws.bitmap);
   fill.n[0] = ws.bitmap_fill_words;
   fill.value[0] = 0u;
-  fill.dst[1] = reinterpret_cast<uint32_t *>(indice_pairs);
-  fill.n[1] = (size_t)g.K * 2 * g.L;
-  fill.value[1] = 0xffffffffu;
   lc.begin("rbFill");
   rbFill<<<fillBlocks((ws.bitmap_fill_words + fill.n[1]) / 4 + 1), kBlock, 0, lc.stream>>>(
       fill, ws.rows_in_order);
@@ -1002,26 +1050,27 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
   lc.begin("rbProbeCount");
   const int k_per = offsetsPerSlice(g.K);
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
-  rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, tab, indices, al_in, nullptr,
+  rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, indices, al_in, nullptr,
                                                             nullptr, 0, ws.bitmap, staging, k_per,
-                                                            ws.rows_in_order);
+                                                            ws.rows_in_order, indice_pairs);
   lc.end();
   lc.begin("rbBitmapBlockSum");
-  rbBitmapBlockSum<<<ws.n_bitmap_blocks, kBlock, 0, lc.stream>>>(ws.bitmap, ws.n_words,
-                                                              ws.block_sum);
+  rbBitmapBlockSum<<<ws.n_bitmap_blocks, kBlock, 0, lc.stream>>>(ws.bitmap, ws.n_words, ws.block_sum);
   lc.end();
-  lc.begin("rbScanRows");
-  rbScanRows<<<1, kScanBlock, 0, lc.stream>>>(ws.block_sum, ws.n_bitmap_blocks, ws.num_act_out);
+  const bool scanned = ws.n_bitmap_blocks > kSelfScanBlocks;
+  if (scanned) {
+    lc.begin("rbScanRows");
+    rbScanRows<<<1, kScanBlock, 0, lc.stream>>>(ws.block_sum, ws.n_bitmap_blocks, ws.num_act_out);
+    lc.end();
+  }
+  lc.begin("rbRankAndDecode");
+  rbRankAndDecode<<<ws.n_bitmap_blocks, kBlock, 0, lc.stream>>>(d, ws.bitmap, ws.n_words, ws.block_sum,
+                                                             scanned, ws.num_act_out, ws.word_rank,
+                                                             out_indices, al_out, g.out_rows);
   lc.end();
   hipError_t err = hipMemcpyAsync(host_num_act_out, ws.num_act_out, sizeof(int32_t),
                                   hipMemcpyDeviceToHost, lc.stream);
   if (err != hipSuccess) return err;
-  lc.begin("rbRankAndDecode");
-  rbRankAndDecode<<<ws.n_bitmap_blocks, kBlock, 0, lc.stream>>>(d, ws.bitmap, ws.n_words,
-                                                             ws.block_sum, ws.num_act_out,
-                                                             ws.word_rank, out_indices, al_out,
-                                                             g.out_rows);
-  lc.end();
   lc.begin("rbPlacePairs");
   rbPlacePairs<false><<<dim3((ws.n_wave + kPlaceWaves - 1) / kPlaceWaves, g.K), kBlock, 0, lc.stream>>>(
       g.L, staging, ws.bitmap, ws.word_rank, indice_pairs, indice_num, ws.rows_in_order, report);

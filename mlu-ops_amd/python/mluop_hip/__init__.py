@@ -303,11 +303,13 @@ def _workspace(nbytes, device):
 
 
 def get_indice_pairs(handle, indices, batch, input_space, filter_space, output_space, pad, stride,
-                     dilation, sub_m, out_rows=None):
+                     dilation, sub_m, out_rows=None, out_indices=None):
     """Builds the rulebook for `indices` (int32 [L, 4] device tensor).
 
     Returns (indice_pairs [K,2,L], out_indices [out_rows,4], indice_num [K] device int32,
-    num_act_out).  In submanifold mode num_act_out is L."""
+    num_act_out).  In submanifold mode num_act_out is L.  Rows of out_indices from
+    num_act_out on are -1: this wrapper allocates the tensor that way, the operator leaves
+    them alone (the reference decodes num_act_out rows, normal_get_indice_pairs.cpp:1143-1150)."""
     torch = _torch()
     L = indices.shape[0]
     K = 1
@@ -323,7 +325,11 @@ def get_indice_pairs(handle, indices, batch, input_space, filter_space, output_s
             out_rows = min(vol, K * L)
     dev = indices.device
     pairs = torch.empty((K, 2, L), dtype=torch.int32, device=dev)
-    out_indices = torch.empty((out_rows, 4), dtype=torch.int32, device=dev)
+    # the operator writes the first num_act_out rows only; the rest keep this initial -1
+    if out_indices is None:
+        out_indices = torch.full((out_rows, 4), -1, dtype=torch.int32, device=dev)
+    else:
+        out_rows = out_indices.shape[0]
     indice_num = torch.empty((K,), dtype=torch.int32, device=dev)
     desc = SparseConvDescriptor(batch, pad, stride, dilation, input_space, filter_space,
                                 output_space, sub_m)

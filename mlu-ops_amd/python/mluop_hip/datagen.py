@@ -114,6 +114,58 @@ def surface_voxels(grid, L, seed, n_shapes=50, noise_frac=0.05, shuffle=False):
     return _finish(cells, grid, L, rng, shuffle)
 
 
+def scene_voxels(grid, L, seed, sheet_frac=0.6, wall_frac=0.3, shuffle=False):
+    """L cells of a driving scene as a voxelizer leaves it, over all batches of ``grid``:
+    ``sheet_frac`` of them in filled rectangles one or two cells thick along D (ground, roofs),
+    ``wall_frac`` in filled upright rectangles one or two cells thick along H or W (walls,
+    vehicles' sides), the rest uniform.  A cell of a filled sheet has 8 to 17 occupied neighbours in
+    a 3x3x3 window, which is what the layers of a detection backbone see (against about one for
+    cells strewn uniformly)."""
+    rng = np.random.default_rng(seed)
+    N, D, H, W = grid
+    vol = D * H * W
+    want_sheet, want_wall = int(L * sheet_frac), int(L * wall_frac)
+
+    def rectangles(quota, upright):
+        got, cells = 0, []
+        while got < quota:
+            n = rng.integers(0, N)
+            thick = rng.integers(1, 3)
+            if not upright:
+                eh, ew = rng.integers(max(4, H // 36), max(6, H // 7) + 1), rng.integers(max(4, W // 36), max(6, W // 7) + 1)
+                d0 = rng.integers(0, D - thick + 1)
+                h0, w0 = rng.integers(0, H - eh + 1), rng.integers(0, W - ew + 1)
+                dd, hh, ww = np.meshgrid(np.arange(d0, d0 + thick), np.arange(h0, h0 + eh),
+                                         np.arange(w0, w0 + ew), indexing="ij")
+            else:
+                ed = rng.integers(min(3, D), min(D, 12) + 1)
+                el = rng.integers(max(4, W // 72), max(6, W // 14) + 1)
+                d0 = rng.integers(0, D - ed + 1)
+                if rng.integers(0, 2):
+                    h0, w0 = rng.integers(0, H - thick + 1), rng.integers(0, W - el + 1)
+                    dd, hh, ww = np.meshgrid(np.arange(d0, d0 + ed), np.arange(h0, h0 + thick),
+                                             np.arange(w0, w0 + el), indexing="ij")
+                else:
+                    el = min(el, H)
+                    h0, w0 = rng.integers(0, H - el + 1), rng.integers(0, W - thick + 1)
+                    dd, hh, ww = np.meshgrid(np.arange(d0, d0 + ed), np.arange(h0, h0 + el),
+                                             np.arange(w0, w0 + thick), indexing="ij")
+            c = n * vol + (dd.ravel() * H + hh.ravel()) * W + ww.ravel()
+            cells.append(c)
+            got += c.size
+        return np.concatenate(cells)
+
+    cells = np.unique(np.concatenate([rectangles(want_sheet, False), rectangles(want_wall, True)]))
+    if cells.size > want_sheet + want_wall:
+        cells = cells[np.sort(rng.choice(cells.size, size=want_sheet + want_wall, replace=False))]
+    while cells.size < L:
+        extra = rng.integers(0, N * vol, size=(L - cells.size) + 16)
+        cells = np.unique(np.concatenate([cells, extra]))
+    if cells.size > L:
+        cells = np.delete(cells, rng.choice(cells.size, size=cells.size - L, replace=False))
+    return _finish(cells, grid, L, rng, shuffle)
+
+
 def kaiming_uniform_filters(K_shape, Ci, Co, seed):
     """Weights U(-b, b), b = 1/sqrt(K*Ci), laid out [kd, kh, kw, Ci, Co] (fp32)."""
     rng = np.random.default_rng(seed)

@@ -117,6 +117,38 @@ def test_regular_rulebook_matches_oracle(gpu_handle, case):
     assert np.all(np.diff(lin) > 0)
 
 
+def test_regular_rulebook_in_a_grid_of_many_bitmap_blocks(gpu_handle):
+    """2 x 41 x 1024 x 1024 output cells at stride 1: a bitmap of more than 5000 blocks of 256 words,
+    whose per-block counts are scanned by a launch of their own instead of summed by every workgroup."""
+    rng = np.random.default_rng(131)
+    space = (41, 1024, 1024)
+    idx = random_voxels(rng, 2, space, 20000, shuffle=True)
+    print("regular many blocks", flush=True)
+    p, o, n, n_out = compare(gpu_handle, idx, 2, space, (3, 3, 3), [1, 1, 1], [1, 1, 1], [1, 1, 1], False)
+    assert n_out > 20000
+
+
+def test_regular_mode_leaves_the_rows_behind_the_active_outputs_alone(gpu_handle):
+    """Like the reference's decode kernel (normal_get_indice_pairs.cpp:1143-1150), which is launched
+    over num_act_out rows, the operator writes no row of out_indices from num_act_out on."""
+    import torch
+    import mluop_hip
+    rng = np.random.default_rng(132)
+    space, ks = (9, 40, 40), (3, 3, 3)
+    idx = random_voxels(rng, 2, space, 900, shuffle=True)
+    ospace = out_space(space, ks, (1, 1, 1), (2, 2, 2), (1, 1, 1))
+    mine = torch.full((2 * int(np.prod(ospace)), 4), 12345, dtype=torch.int32, device="cuda")
+    _, o, _, n_out = mluop_hip.get_indice_pairs(gpu_handle, torch.from_numpy(idx).cuda(), 2, space, ks, ospace,
+                                               [1, 1, 1], [2, 2, 2], [1, 1, 1], False, out_indices=mine)
+    torch.cuda.synchronize()
+    o = o.cpu().numpy()
+    _, ro, _, rn_out = oracle.get_indice_pairs(idx, 2, [1, 1, 1], [2, 2, 2], [1, 1, 1], list(ks), ospace, False,
+                                               out_rows=o.shape[0], exact_count=True)
+    assert n_out == rn_out and 0 < n_out < o.shape[0]
+    assert np.array_equal(o[:n_out], ro[:n_out])
+    assert np.all(o[n_out:] == 12345)
+
+
 def test_regular_out_indices_smaller_tensor_is_rejected_cleanly(gpu_handle):
     """A caller-supplied out_indices with fewer rows than active outputs must not be overrun."""
     import mluop_hip
