@@ -117,9 +117,14 @@ mluOpStatus_t MLUOP_WIN_API mluOpGetQueue(mluOpHandle_t handle, mluOpQueue_t *qu
 mluOpStatus_t MLUOP_WIN_API mluOpSetQuantizeRoundMode(mluOpHandle_t handle,
                                                       mluOpQuantizeRoundMode_t round_mode) {
   PARAM_CHECK("[mluOpSetQuantizeRoundMode]", handle != NULL);
-  PARAM_CHECK("[mluOpSetQuantizeRoundMode]", round_mode == MLUOP_ROUND_HALF_TO_EVEN ||
-                                                 round_mode == MLUOP_ROUND_HALF_OFF_ZERO ||
-                                                 round_mode == MLUOP_ROUND_HALF_UP);
+  // A C caller can pass any integer here; it is looked at as one before it is used as the
+  // enumeration.
+  int as_int = 0;
+  static_assert(sizeof(as_int) == sizeof(round_mode), "enumeration passed as an int");
+  std::memcpy(&as_int, &round_mode, sizeof(as_int));
+  PARAM_CHECK("[mluOpSetQuantizeRoundMode]", as_int == MLUOP_ROUND_HALF_TO_EVEN ||
+                                                 as_int == MLUOP_ROUND_HALF_OFF_ZERO ||
+                                                 as_int == MLUOP_ROUND_HALF_UP);
   handle->round_mode = round_mode;
   return MLUOP_STATUS_SUCCESS;
 }

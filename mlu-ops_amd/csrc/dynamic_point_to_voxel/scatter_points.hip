@@ -240,10 +240,13 @@ struct Workspace {
 
 Workspace carve(void *base, const ScatterShape &s, size_t library_bytes) {
   const size_t n = (size_t)s.num_points;
-  char *p = static_cast<char *>(base);
+  // Blocks start at the caller's pointer rounded up to 256 bytes (64-bit keys, packed sort
+  // keys and the library's temporary storage need their alignment whatever the caller
+  // passes); the reported size includes that slack.  A null base only measures.
+  char *p = base ? reinterpret_cast<char *>(alignUp(reinterpret_cast<uintptr_t>(base))) : nullptr;
   size_t off = 0;
   auto take = [&](size_t bytes) {
-    char *q = p + off;
+    char *q = p ? p + off : nullptr;
     off += alignUp(bytes);
     return q;
   };
@@ -257,7 +260,7 @@ Workspace carve(void *base, const ScatterShape &s, size_t library_bytes) {
   w.first_pos = reinterpret_cast<int32_t *>(take(4 * (n + 1)));
   w.axis_max = reinterpret_cast<int32_t *>(take(16));
   w.library = take(library_bytes);
-  w.total = off;
+  w.total = off + 256;
   return w;
 }
 

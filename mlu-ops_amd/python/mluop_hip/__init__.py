@@ -12,12 +12,15 @@ computation runs in the library's own HIP kernels.  There is no CPU fallback: a
 missing library raises at import of the first symbol.
 """
 import ctypes
+import threading
 import os
 
 from . import datagen  # noqa: F401
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "..", "lib", "libmluops.so"))
+# MLUOP_LIBRARY names another build of the library (the sanitizer build of `make asan`).
+LIB_PATH = os.environ.get("MLUOP_LIBRARY") or os.path.normpath(
+    os.path.join(_HERE, "..", "..", "lib", "libmluops.so"))
 
 # mluOpStatus_t
 STATUS_SUCCESS = 0
@@ -297,9 +300,88 @@ def make_handle_on_current_stream():
     return Handle(queue=torch.cuda.current_stream().cuda_stream)
 
 
-def _workspace(nbytes, device):
+# Guard bands for tests (the reference's test runner does the same around every device buffer,
+# pb_gtest/src/runtime.cpp:99-145): with GUARD_BYTES > 0 every output tensor and workspace these
+# wrappers allocate sits between two bands of GUARD_BYTES bytes holding GUARD_PATTERN, and after
+# every operator call the wrappers wait for the queue and raise if a band has changed.
+GUARD_BYTES = 0
+GUARD_PATTERN = 0xA5
+_guard_state = threading.local()   # .bands: (whole buffer, payload bytes, what) of this thread's next call
+
+
+def _bands():
+    if not hasattr(_guard_state, "bands"):
+        _guard_state.bands = []
+    return _guard_state.bands
+
+
+def _capturing():
+    """Inside a stream capture nothing runs, so bands could be neither filled nor checked."""
     torch = _torch()
-    return torch.empty((max(int(nbytes), 1),), dtype=torch.uint8, device=device)
+    return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+
+
+def _guarded_bytes(nbytes, device, what):
+    torch = _torch()
+    nbytes = int(nbytes)
+    if GUARD_BYTES <= 0 or _capturing():
+        return torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=device)
+    whole = torch.empty((nbytes + 2 * GUARD_BYTES,), dtype=torch.uint8, device=device)
+    whole[:GUARD_BYTES] = GUARD_PATTERN
+    whole[GUARD_BYTES + nbytes:] = GUARD_PATTERN
+    _bands().append((whole, nbytes, what))
+    return whole[GUARD_BYTES:GUARD_BYTES + max(nbytes, 1)]
+
+
+# Tests of workspaces the caller did not align: every workspace starts this many bytes behind
+# an aligned address.
+WORKSPACE_SKEW = 0
+
+
+def _workspace(nbytes, device):
+    if WORKSPACE_SKEW:
+        return _guarded_bytes(int(nbytes) + WORKSPACE_SKEW, device, "workspace")[WORKSPACE_SKEW:]
+    return _guarded_bytes(nbytes, device, "workspace")
+
+
+def _output(shape, dtype, device, what, fill=None):
+    """An output tensor of the operator `what` is about to write (between guard bands in guard mode)."""
+    torch = _torch()
+    shape = tuple(int(v) for v in shape)
+    if GUARD_BYTES <= 0 or _capturing():
+        if fill is None:
+            return torch.empty(shape, dtype=dtype, device=device)
+        return torch.full(shape, fill, dtype=dtype, device=device)
+    n = 1
+    for v in shape:
+        n *= v
+    item = torch.empty((), dtype=dtype).element_size()
+    raw = _guarded_bytes(n * item, device, what)
+    t = raw[:n * item].view(dtype).view(shape)
+    if fill is not None:
+        t.fill_(fill)
+    return t
+
+
+def _guards_intact(call):
+    """After operator `call`: in guard mode, waits for the GPU and checks every band allocated for it."""
+    bands = _bands()
+    if not bands:
+        return
+    torch = _torch()
+    if torch.cuda.is_available():
+        torch.cuda.synchronize()
+    bad = []
+    for whole, nbytes, what in bands:
+        front = whole[:GUARD_BYTES]
+        back = whole[GUARD_BYTES + nbytes:]
+        if not bool((front == GUARD_PATTERN).all()):
+            bad.append("%s: bytes in front of it were written" % what)
+        if not bool((back == GUARD_PATTERN).all()):
+            bad.append("%s: bytes behind it were written" % what)
+    del bands[:]
+    if bad:
+        raise AssertionError("%s wrote outside its buffers: %s" % (call, "; ".join(bad)))
 
 
 def get_indice_pairs(handle, indices, batch, input_space, filter_space, output_space, pad, stride,
@@ -324,13 +406,13 @@ def get_indice_pairs(handle, indices, batch, input_space, filter_space, output_s
                 vol *= int(o)
             out_rows = min(vol, K * L)
     dev = indices.device
-    pairs = torch.empty((K, 2, L), dtype=torch.int32, device=dev)
+    pairs = _output((K, 2, L), torch.int32, dev, "indice_pairs")
     # the operator writes the first num_act_out rows only; the rest keep this initial -1
     if out_indices is None:
-        out_indices = torch.full((out_rows, 4), -1, dtype=torch.int32, device=dev)
+        out_indices = _output((out_rows, 4), torch.int32, dev, "out_indices", fill=-1)
     else:
         out_rows = out_indices.shape[0]
-    indice_num = torch.empty((K,), dtype=torch.int32, device=dev)
+    indice_num = _output((K,), torch.int32, dev, "indice_num")
     desc = SparseConvDescriptor(batch, pad, stride, dilation, input_space, filter_space,
                                 output_space, sub_m)
     d_in = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [L, 4])
@@ -346,6 +428,7 @@ def get_indice_pairs(handle, indices, batch, input_space, filter_space, output_s
                                     ws.data_ptr(), size.value, d_pairs.ptr, pairs.data_ptr(),
                                     d_out.ptr, out_indices.data_ptr(), d_num.ptr,
                                     indice_num.data_ptr()), "mluOpGetIndicePairs")
+    _guards_intact("mluOpGetIndicePairs")
     num_act_out = L if sub_m else desc.num_act_out()
     return pairs, out_indices, indice_num, num_act_out
 
@@ -370,13 +453,14 @@ class RowMap:
         check(lib().mluOpExtGetRowMapSize(d_pairs.ptr, int(rows), ctypes.byref(size)), "mluOpExtGetRowMapSize")
         self.handle = handle
         self.pairs = indice_pairs          # the map is valid for this tensor only: keep it alive
-        self.buffer = torch.empty((size.value,), dtype=torch.uint8, device=indice_pairs.device)
+        self.buffer = _guarded_bytes(size.value, indice_pairs.device, "row map")
         lost = ctypes.c_int64(0)
         check(lib().mluOpExtBuildRowMap(handle.ptr, d_pairs.ptr, indice_pairs.data_ptr(),
                                         _host_counts(indice_num_host), int(rows), int(source_rows),
                                         int(row_column), self.buffer.data_ptr(), size.value,
                                         ctypes.byref(lost) if verify else None),
               "mluOpExtBuildRowMap")
+        _guards_intact("mluOpExtBuildRowMap")
         self.lost_pairs = int(lost.value) if verify else None
         self.usable = not verify or self.lost_pairs == 0
 
@@ -407,7 +491,7 @@ def indice_conv_forward(handle, features, filters, filters_layout, indice_pairs,
         co = filters.shape[4]
     else:
         co = filters.shape[0]
-    out = torch.empty((num_act_out, co), dtype=features.dtype, device=features.device)
+    out = _output((num_act_out, co), features.dtype, features.device, "features_out")
     d_feat = TensorDescriptor(LAYOUT_ARRAY, code, list(features.shape))
     d_filt = TensorDescriptor(filters_layout, code, list(filters.shape))
     d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
@@ -424,6 +508,7 @@ def indice_conv_forward(handle, features, filters, filters_layout, indice_pairs,
         handle.ptr, d_feat.ptr, features.data_ptr(), d_filt.ptr, filters.data_ptr(), d_pairs.ptr,
         indice_pairs.data_ptr(), counts, num_act_out, inverse, int(sub_m), ws.data_ptr(),
         size.value, d_out.ptr, out.data_ptr()), "mluOpIndiceConvolutionForward")
+    _guards_intact("mluOpIndiceConvolutionForward")
     return out
 
 
@@ -434,7 +519,7 @@ def indice_conv_backward_data(handle, output_grad, filters, filters_layout, indi
     code = torch_dtype_code(output_grad.dtype)
     K, _, L = indice_pairs.shape
     rows = L if rows is None else int(rows)
-    dx = torch.empty((rows, ci), dtype=output_grad.dtype, device=output_grad.device)
+    dx = _output((rows, ci), output_grad.dtype, output_grad.device, "input_grad")
     d_dy = TensorDescriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
     d_filt = TensorDescriptor(filters_layout, code, list(filters.shape))
     d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
@@ -451,6 +536,7 @@ def indice_conv_backward_data(handle, output_grad, filters, filters_layout, indi
         handle.ptr, d_dy.ptr, output_grad.data_ptr(), d_filt.ptr, filters.data_ptr(), d_pairs.ptr,
         indice_pairs.data_ptr(), counts, inverse, int(sub_m), ws.data_ptr(), size.value, d_dx.ptr,
         dx.data_ptr()), "mluOpIndiceConvolutionBackwardData")
+    _guards_intact("mluOpIndiceConvolutionBackwardData")
     return dx
 
 
@@ -469,7 +555,7 @@ def indice_conv_backward_filter(handle, features, output_grad, indice_pairs, ind
         shape = (co, ci) + tuple(filter_space)
     else:
         shape = tuple(filter_space) + (ci, co)
-    dw = torch.empty(shape, dtype=features.dtype, device=features.device)
+    dw = _output(shape, features.dtype, features.device, "filters_grad")
     d_x = TensorDescriptor(LAYOUT_ARRAY, code, list(features.shape))
     d_dy = TensorDescriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
     d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
@@ -485,6 +571,7 @@ def indice_conv_backward_filter(handle, features, output_grad, indice_pairs, ind
         handle.ptr, d_x.ptr, features.data_ptr(), d_dy.ptr, output_grad.data_ptr(), d_pairs.ptr,
         indice_pairs.data_ptr(), counts, inverse, int(sub_m), ws.data_ptr(), size.value, d_dw.ptr,
         dw.data_ptr()), "mluOpIndiceConvolutionBackwardFilter")
+    _guards_intact("mluOpIndiceConvolutionBackwardFilter")
     return dw
 
 
@@ -507,6 +594,7 @@ def indice_conv_backward_filter_no_alloc(handle, features, output_grad, indice_p
         handle.ptr, d_x.ptr, features.data_ptr(), d_dy.ptr, output_grad.data_ptr(), d_pairs.ptr,
         indice_pairs.data_ptr(), _host_counts(indice_num_host), inverse, int(sub_m), d_dw.ptr,
         filters_grad.data_ptr()), "mluOpExtIndiceConvolutionBackwardFilterNoAlloc")
+    _guards_intact("mluOpExtIndiceConvolutionBackwardFilterNoAlloc")
     return filters_grad
 
 
@@ -519,9 +607,9 @@ def voxelization(handle, points, voxel_size, coors_range, max_points, max_voxels
     torch = _torch()
     n, f = points.shape
     dev = points.device
-    voxels = torch.empty((max_voxels, max_points, f), dtype=torch.float32, device=dev)
-    coors = torch.empty((max_voxels, 3), dtype=torch.int32, device=dev)
-    npv = torch.empty((max_voxels,), dtype=torch.int32, device=dev)
+    voxels = _output((max_voxels, max_points, f), torch.float32, dev, "voxels")
+    coors = _output((max_voxels, 3), torch.int32, dev, "coors")
+    npv = _output((max_voxels,), torch.int32, dev, "num_points_per_voxel")
     voxel_num = torch.zeros((1,), dtype=torch.int32, device=dev)
     d_points = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, f])
     d_vs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [3])
@@ -541,6 +629,7 @@ def voxelization(handle, points, voxel_size, coors_range, max_points, max_voxels
         coors_range.data_ptr(), max_points, max_voxels, 3, bool(deterministic), ws.data_ptr(), size.value,
         d_voxels.ptr, voxels.data_ptr(), d_coors.ptr, coors.data_ptr(), d_npv.ptr, npv.data_ptr(), d_num.ptr,
         voxel_num.data_ptr()), "mluOpVoxelization")
+    _guards_intact("mluOpVoxelization")
     return voxels, coors, npv, voxel_num
 
 
@@ -554,10 +643,10 @@ def dynamic_point_to_voxel_forward(handle, feats, coors, reduce_type="max", rows
     n, c = feats.shape
     m = n if rows is None else int(rows)
     dev = feats.device
-    voxel_feats = torch.empty((m, c), dtype=torch.float32, device=dev)
-    voxel_coors = torch.empty((m, 3), dtype=torch.int32, device=dev)
-    p2v = torch.empty((n,), dtype=torch.int32, device=dev)
-    count = torch.empty((m,), dtype=torch.int32, device=dev)
+    voxel_feats = _output((m, c), torch.float32, dev, "voxel_feats")
+    voxel_coors = _output((m, 3), torch.int32, dev, "voxel_coors")
+    p2v = _output((n,), torch.int32, dev, "point2voxel_map")
+    count = _output((m,), torch.int32, dev, "voxel_points_count")
     voxel_num = torch.zeros((1,), dtype=torch.int32, device=dev)
     mode = {"max": REDUCE_DMAX, "mean": REDUCE_DMEAN, "sum": REDUCE_DSUM}[reduce_type]
     d_feats = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
@@ -577,6 +666,7 @@ def dynamic_point_to_voxel_forward(handle, feats, coors, reduce_type="max", rows
         size.value, d_vf.ptr, voxel_feats.data_ptr(), d_vc.ptr, voxel_coors.data_ptr(), d_p2v.ptr,
         p2v.data_ptr(), d_cnt.ptr, count.data_ptr(), d_num.ptr, voxel_num.data_ptr()),
         "mluOpDynamicPointToVoxelForward")
+    _guards_intact("mluOpDynamicPointToVoxelForward")
     return voxel_feats, voxel_coors, p2v, count, voxel_num
 
 
@@ -586,7 +676,7 @@ def dynamic_point_to_voxel_backward(handle, grad_voxel_feats, feats, voxel_feats
     torch = _torch()
     n, c = feats.shape
     m = grad_voxel_feats.shape[0]
-    grad_feats = torch.empty((n, c), dtype=torch.float32, device=feats.device)
+    grad_feats = _output((n, c), torch.float32, feats.device, "grad_feats")
     mode = {"max": REDUCE_DMAX, "mean": REDUCE_DMEAN, "sum": REDUCE_DSUM}[reduce_type]
     d_g = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [m, c])
     d_feats = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
@@ -605,4 +695,5 @@ def dynamic_point_to_voxel_backward(handle, grad_voxel_feats, feats, voxel_feats
         voxel_feats.data_ptr(), d_p2v.ptr, point2voxel_map.data_ptr(), d_cnt.ptr,
         voxel_points_count.data_ptr(), d_num.ptr, voxel_num.data_ptr(), ws.data_ptr(), size.value, d_out.ptr,
         grad_feats.data_ptr()), "mluOpDynamicPointToVoxelBackward")
+    _guards_intact("mluOpDynamicPointToVoxelBackward")
     return grad_feats

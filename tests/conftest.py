@@ -21,6 +21,9 @@ def gpu_handle():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     torch.cuda.set_device(0)
+    # every output tensor and workspace the wrappers allocate sits between 4 KiB guard bands,
+    # checked after each operator call (the reference's test runner: pb_gtest/src/runtime.cpp:99-145)
+    mluop_hip.GUARD_BYTES = 4096
     h = mluop_hip.make_handle_on_current_stream()
     yield h
     torch.cuda.synchronize()

@@ -133,10 +133,35 @@ def test_config5a_subm_5x5x5_rulebook_and_forward(gpu_handle, config5_voxels):
         grade_sample(from_torch(out[torch.from_numpy(rows).cuda()]), ref, dtype_name, "config5a " + dtype_name)
         del out
 
+    # backward data and backward filter on the same rulebook, fp16: input-gradient rows of a sample
+    # (the forward sum with the pair columns swapped and every filter slice transposed), and the filter
+    # gradient of four offsets (centre, both ends, one in between) as X[in]^T dY[out] over their pairs
+    print("config5a backward data", flush=True)
+    dy = round_to((rng.standard_normal((n_out, 128)) * 0.1).astype(np.float32), "float16")
+    w = round_to(w32, "float16")
+    feats = round_to(feats32, "float16")
+    t_dy, t_w, t_f = (to_torch(a, "float16", "cuda") for a in (dy, w, feats))
+    dx = mluop_hip.indice_conv_backward_data(gpu_handle, t_dy, t_w, mluop_hip.LAYOUT_ARRAY, pairs, num_host, True,
+                                             128)
+    torch.cuda.synchronize()
+    swapped = np.ascontiguousarray(pairs_np[:, ::-1, :])
+    w_t = np.ascontiguousarray(w.reshape(125, 128, 128).transpose(0, 2, 1))
+    ref = sampled_rows_reference(dy, w_t, swapped, num_host, rows)
+    grade_sample(from_torch(dx[torch.from_numpy(rows).cuda()]), ref, "float16", "config5a backward data")
+    del dx
+    print("config5a backward filter", flush=True)
+    dw = mluop_hip.indice_conv_backward_filter(gpu_handle, t_f, t_dy, pairs, num_host, ks, True)
+    torch.cuda.synchronize()
+    dw_np = from_torch(dw).reshape(125, 128, 128)
+    for k in (0, 37, 62, 124):
+        n = num_host[k]
+        ref_k = feats[pairs_np[k, 0, :n]].astype(np.float64).T @ dy[pairs_np[k, 1, :n]].astype(np.float64)
+        grade_sample(dw_np[k], ref_k, "float16", "config5a backward filter, offset %d" % k)
+
 
 def test_config5b_regular_2x2x2_stride2_on_5a_outputs(gpu_handle, config5_voxels):
     """Config 5b: regular 2x2x2 stride 2 pad 0 over the rows 5a leaves (a submanifold layer keeps
-    its input coordinates), out 1x32x512x512, Ci=Co=128 fp16."""
+    its input coordinates), out 1x32x512x512, Ci=Co=128, fp16 and fp32."""
     import torch
     import mluop_hip
     idx = config5_voxels
@@ -148,16 +173,20 @@ def test_config5b_regular_2x2x2_stride2_on_5a_outputs(gpu_handle, config5_voxels
     num_host = num.cpu().tolist()
     assert sum(num_host) == idx.shape[0]  # stride = kernel edge: every input row lands in exactly one pair
     rng = np.random.default_rng(6)
-    feats = round_to(rng.standard_normal((idx.shape[0], 128)).astype(np.float32), "float16")
-    w = round_to(mluop_hip.datagen.kaiming_uniform_filters(ks, 128, 128, seed=6), "float16")
-    out = mluop_hip.indice_conv_forward(gpu_handle, to_torch(feats, "float16", "cuda"),
-                                        to_torch(w, "float16", "cuda"), mluop_hip.LAYOUT_ARRAY, pairs, num_host,
-                                        n_out, False)
-    torch.cuda.synchronize()
+    feats32 = rng.standard_normal((idx.shape[0], 128)).astype(np.float32)
+    w32 = mluop_hip.datagen.kaiming_uniform_filters(ks, 128, 128, seed=6)
     rows = np.sort(rng.choice(n_out, size=3000, replace=False))
-    ref = sampled_rows_reference(feats, w.reshape(8, 128, 128), pairs.cpu().numpy(), num_host, rows)
-    grade_sample(from_torch(out[torch.from_numpy(rows).cuda()]), ref, "float16", "config5b fp16")
-
+    pairs_np = pairs.cpu().numpy()
+    for dtype_name in ("float16", "float32"):
+        print("config5b forward", dtype_name, flush=True)
+        feats, w = round_to(feats32, dtype_name), round_to(w32, dtype_name)
+        out = mluop_hip.indice_conv_forward(gpu_handle, to_torch(feats, dtype_name, "cuda"),
+                                            to_torch(w, dtype_name, "cuda"), mluop_hip.LAYOUT_ARRAY, pairs, num_host,
+                                            n_out, False)
+        torch.cuda.synchronize()
+        ref = sampled_rows_reference(feats, w.reshape(8, 128, 128), pairs_np, num_host, rows)
+        grade_sample(from_torch(out[torch.from_numpy(rows).cuda()]), ref, dtype_name, "config5b " + dtype_name)
+        del out
 
 @pytest.mark.timeout(600)
 def test_convolutions_at_one_million_rows(gpu_handle):

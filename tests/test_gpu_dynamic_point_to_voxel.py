@@ -162,9 +162,13 @@ def test_inputs_at_odd_addresses(gpu_handle):
     cv = cc[1:1 + coors.size].view(coors.shape)
     cv.copy_(torch.from_numpy(coors))
     assert fv.data_ptr() % 16 != 0 and cv.data_ptr() % 16 != 0
-    for mode in ("max", "mean"):
+    for mode, skew in (("max", 0), ("mean", 0), ("max", 4), ("mean", 12)):   # skew: workspace off alignment too
         cv.copy_(torch.from_numpy(coors))
-        out = mluop_hip.dynamic_point_to_voxel_forward(gpu_handle, fv, cv, mode)
+        mluop_hip.WORKSPACE_SKEW = skew
+        try:
+            out = mluop_hip.dynamic_point_to_voxel_forward(gpu_handle, fv, cv, mode)
+        finally:
+            mluop_hip.WORKSPACE_SKEW = 0
         torch.cuda.synchronize()
         got = [t.cpu().numpy() for t in out[:4]] + [int(out[4].item()), cv.cpu().numpy()]
         assert_same(got, dpv.forward(mode, feats, coors))

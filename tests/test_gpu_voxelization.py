@@ -110,8 +110,14 @@ def test_points_at_an_odd_address(gpu_handle):
     view = flat[1:1 + pts.size].view(pts.shape)
     view.copy_(torch.from_numpy(pts))
     assert view.data_ptr() % 16 != 0
-    out = mluop_hip.voxelization(gpu_handle, view, torch.tensor(vs, dtype=torch.float32).cuda(),
-                                 torch.tensor(cr, dtype=torch.float32).cuda(), 5, 2000)
-    torch.cuda.synchronize()
-    got = (out[0].cpu().numpy(), out[1].cpu().numpy(), out[2].cpu().numpy(), int(out[3].item()))
-    assert_same(got, vox.voxelization(pts, vs, cr, 5, 2000))
+    expect = vox.voxelization(pts, vs, cr, 5, 2000)
+    for skew in (0, 4):   # and a workspace that is only 4-byte aligned
+        mluop_hip.WORKSPACE_SKEW = skew
+        try:
+            out = mluop_hip.voxelization(gpu_handle, view, torch.tensor(vs, dtype=torch.float32).cuda(),
+                                         torch.tensor(cr, dtype=torch.float32).cuda(), 5, 2000)
+        finally:
+            mluop_hip.WORKSPACE_SKEW = 0
+        torch.cuda.synchronize()
+        got = (out[0].cpu().numpy(), out[1].cpu().numpy(), out[2].cpu().numpy(), int(out[3].item()))
+        assert_same(got, expect)
