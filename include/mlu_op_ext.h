@@ -19,6 +19,23 @@ extern "C" {
  * costs two event records per launch, so leave it off in production. */
 mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelTiming(mluOpHandle_t handle, int enable);
 
+/* Kernel choices of the sparse convolution operators.  Where two kernels compute the same
+ * result the shape decides between them; the parity tests switch each one on and off through
+ * this call and compare.  value: -1 the shape decides (the default), 0 never, 1 whenever the
+ * kernel can run the shape.  The choice belongs to the handle and holds until changed.  (The
+ * reference selects kernels by shape only; its test-time switches are environment variables
+ * of the test runner, pb_gtest/src/runtime.cpp.) */
+typedef enum {
+  MLUOP_EXT_KERNEL_GATHER_SIMT = 0,    /* plain SIMT kernels instead of the MFMA ones */
+  MLUOP_EXT_KERNEL_DENSE_TILES = 1,    /* register-accumulating gather kernel */
+  MLUOP_EXT_KERNEL_WAVE_PER_TILE = 2,  /* one-wavefront-per-tile gather kernel */
+  MLUOP_EXT_KERNEL_FLAT_SLICE_SUM = 3, /* backward filter: partial tiles summed on a flat grid */
+  MLUOP_EXT_KERNEL_FLAT_SCATTER = 4    /* row maps built on a flat grid */
+} mluOpExtKernelChoice_t;
+
+mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelChoice(mluOpHandle_t handle,
+                                                    mluOpExtKernelChoice_t which, int value);
+
 /* Waits for the handle's queue, then reports how many launches were recorded. */
 mluOpStatus_t MLUOP_WIN_API mluOpExtGetKernelTimingCount(mluOpHandle_t handle, int *count);
 

@@ -160,6 +160,27 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelTiming(mluOpHandle_t handle, int en
   return MLUOP_STATUS_SUCCESS;
 }
 
+mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelChoice(mluOpHandle_t handle,
+                                                    mluOpExtKernelChoice_t which, int value) {
+  PARAM_CHECK("[mluOpExtSetKernelChoice]", handle != NULL);
+  PARAM_CHECK("[mluOpExtSetKernelChoice]", value >= -1 && value <= 1);
+  int as_int = 0;
+  static_assert(sizeof(as_int) == sizeof(which), "enumeration passed as an int");
+  std::memcpy(&as_int, &which, sizeof(as_int));
+  mluop::KernelChoices &c = handle->kernel_choices;
+  switch (as_int) {
+    case MLUOP_EXT_KERNEL_GATHER_SIMT: c.gather_simt = value; break;
+    case MLUOP_EXT_KERNEL_DENSE_TILES: c.dense_tiles = value; break;
+    case MLUOP_EXT_KERNEL_WAVE_PER_TILE: c.wave_per_tile = value; break;
+    case MLUOP_EXT_KERNEL_FLAT_SLICE_SUM: c.flat_slice_sum = value; break;
+    case MLUOP_EXT_KERNEL_FLAT_SCATTER: c.flat_scatter = value; break;
+    default:
+      MLUOP_LOG(ERROR) << "[mluOpExtSetKernelChoice] unknown kernel choice " << as_int;
+      return MLUOP_STATUS_BAD_PARAM;
+  }
+  return MLUOP_STATUS_SUCCESS;
+}
+
 mluOpStatus_t MLUOP_WIN_API mluOpExtSetSparseConvExtendedModes(mluOpHandle_t handle,
                                                                int enable) {
   PARAM_CHECK("[mluOpExtSetSparseConvExtendedModes]", handle != NULL);

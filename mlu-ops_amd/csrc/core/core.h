@@ -73,7 +73,10 @@ struct mluOpContext {
   unsigned long long next_stamp = 1;   // also the source of per-call tickets
 
   // What the kernel launchers need: the stream, and the timer while it is on.
-  mluop::LaunchCtx launchCtx() { return mluop::LaunchCtx(queue, timer.enabled ? &timer : nullptr); }
+  mluop::KernelChoices kernel_choices;
+  mluop::LaunchCtx launchCtx() {
+    return mluop::LaunchCtx(queue, timer.enabled ? &timer : nullptr, &kernel_choices);
+  }
 };
 
 // ---------------------------------------------------------------------------

@@ -45,10 +45,24 @@ struct KernelTimer {
   }
 };
 
+// Which kernel the sparse convolution launchers take where more than one computes the same
+// result: -1 lets the shape decide, 0 / 1 switch a kernel off / on for every shape it can
+// run.  A handle holds one set (mluOpExtSetKernelChoice); the parity tests use it to run
+// both kernels of a pair on one shape.
+struct KernelChoices {
+  int gather_simt = -1;     // 1: the plain SIMT gather and filter-gradient kernels instead of MFMA
+  int dense_tiles = -1;     // the register-accumulating gather kernel
+  int wave_per_tile = -1;   // the one-wavefront-per-tile gather kernel
+  int flat_slice_sum = -1;  // backward filter: partial tiles summed on the flat grid
+  int flat_scatter = -1;    // 1: row maps built on the flat grid
+};
+
 class LaunchCtx {
  public:
-  LaunchCtx(hipStream_t s, KernelTimer *t) : stream(s), timer_(t) {}
+  LaunchCtx(hipStream_t s, KernelTimer *t, const KernelChoices *c = nullptr)
+      : stream(s), choices(c ? *c : KernelChoices()), timer_(t) {}
   hipStream_t stream;
+  KernelChoices choices;
 
   // Call right before / right after enqueueing kernel `name`.
   void begin(const char *name) const {

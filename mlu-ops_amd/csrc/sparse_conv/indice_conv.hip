@@ -26,7 +26,6 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
-#include <cstdlib>
 #include <type_traits>
 
 #include "core/wave_scan.h"
@@ -1925,20 +1924,9 @@ inline int gridFor(size_t n, int cap = 8192) {
   return (int)(b < 1 ? 1 : (b > (size_t)cap ? (size_t)cap : b));
 }
 
-// Test switch: "1" sums the backward filter's partial tiles on the flat grid whatever
-// the shape, "0" never does (the two kernels must give the same bits); unset, the
-// grid's size decides.
+// The backward filter's partial tiles are summed on the flat grid from this many
+// workgroups on (or as the handle's kernel choice says; the two kernels give the same bits).
 constexpr int kFlatSumFromBlocks = 2048;
-int sliceSumMode() {
-  const char *v = getenv("MLUOP_SPCONV_FLAT_SLICE_SUM");
-  if (v == nullptr || (v[0] != '0' && v[0] != '1')) return -1;
-  return v[0] - '0';
-}
-
-bool forceSimt() {
-  const char *v = getenv("MLUOP_SPCONV_FORCE_SIMT");
-  return v != nullptr && v[0] == '1';
-}
 
 // fp16/bf16: 16x16x32 MFMA; float: 16x16x4 MFMA; reduction channels in {16, 32, 64, 128}.
 bool mfmaShapeOk(ElemType t, int Q, int C) {
@@ -2027,36 +2015,36 @@ GatherWorkspace carveGather(const ConvProblem &p, const GatherDims &d, void *bas
   return ws;
 }
 
-// Fills the by-value counts (K <= kMaxInlineK) or uploads them.  The int32
-// staging vector is consumed by a synchronous-with-host pageable copy.
+// Writes n counts, carried in the kernel arguments, to dst.
+__global__ void storeCounts(OffsetCounts c, int n, int32_t *dst) {
+  const int i = threadIdx.x;
+  if (i < n) dst[i] = c.n[i];
+}
+
+// Fills the by-value counts (K <= kMaxInlineK) or puts them into device memory: kMaxInlineK
+// counts ride in the arguments of one small launch each, so the host neither allocates nor
+// waits, and the call can be captured into a graph like any other.
 hipError_t prepareCounts(const LaunchCtx &lc, const ConvProblem &p, OffsetCounts *inl,
                          int32_t *dev_counts, int *max_count) {
+  auto clamped = [&](int k) {
+    const int64_t n = p.indice_num[k];
+    return (int)(n < 0 ? 0 : (n > p.L ? p.L : n));
+  };
   int mx = 0;
-  for (int k = 0; k < p.K; ++k) {
-    int64_t n = p.indice_num[k];
-    if (n < 0) n = 0;
-    if (n > p.L) n = p.L;
-    if ((int)n > mx) mx = (int)n;
-  }
+  for (int k = 0; k < p.K; ++k) mx = clamped(k) > mx ? clamped(k) : mx;
   *max_count = mx;
   for (int k = 0; k < kMaxInlineK; ++k) inl->n[k] = 0;
   if (p.K <= kMaxInlineK) {
-    for (int k = 0; k < p.K; ++k) {
-      int64_t n = p.indice_num[k];
-      inl->n[k] = (int)(n < 0 ? 0 : (n > p.L ? p.L : n));
-    }
+    for (int k = 0; k < p.K; ++k) inl->n[k] = clamped(k);
     return hipSuccess;
   }
-  int32_t *tmp = static_cast<int32_t *>(malloc((size_t)p.K * 4));
-  if (tmp == nullptr) return hipErrorOutOfMemory;
-  for (int k = 0; k < p.K; ++k) {
-    int64_t n = p.indice_num[k];
-    tmp[k] = (int)(n < 0 ? 0 : (n > p.L ? p.L : n));
+  for (int k0 = 0; k0 < p.K; k0 += kMaxInlineK) {
+    OffsetCounts part;
+    const int n = p.K - k0 < kMaxInlineK ? p.K - k0 : kMaxInlineK;
+    for (int i = 0; i < kMaxInlineK; ++i) part.n[i] = i < n ? clamped(k0 + i) : 0;
+    storeCounts<<<1, kMaxInlineK, 0, lc.stream>>>(part, n, dev_counts + k0);
   }
-  hipError_t err = hipMemcpyAsync(dev_counts, tmp, (size_t)p.K * 4, hipMemcpyHostToDevice, lc.stream);
-  if (err == hipSuccess) err = hipStreamSynchronize(lc.stream);
-  free(tmp);
-  return err;
+  return hipGetLastError();
 }
 
 // A 128-column result with few pairs per (64-row tile, offset) runs as two
@@ -2147,9 +2135,8 @@ void launchWave(const LaunchCtx &lc, int Q, int C, const void *A, const void *pa
 #undef WAVE_CASE
 }
 
-bool useWaveKernel(ElemType t, int Q, int C) {
-  const char *e = getenv("MLUOP_SPCONV_WAVE");
-  if (e != nullptr && e[0] == '0') return false;
+bool useWaveKernel(const LaunchCtx &lc, ElemType t, int Q, int C) {
+  if (lc.choices.wave_per_tile == 0) return false;
   return waveKernelShape((int)elemSize(t), Q, C);
 }
 
@@ -2163,10 +2150,9 @@ bool denseShapeOk(ElemType t, int Q, int C) {
   return (C == 64 || C == 128) && Q % chunk == 0 && (Q == 16 || Q == 32 || Q == 64 || Q == 128);
 }
 
-bool useDenseKernel(const ConvProblem &p, const GatherDims &d) {
+bool useDenseKernel(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d) {
   if (!denseShapeOk(p.dtype, d.Q, d.C)) return false;
-  // MLUOP_SPCONV_DENSE=1 / 0 forces the choice (the parity tests run both kernels on one shape)
-  if (const char *e = getenv("MLUOP_SPCONV_DENSE")) return e[0] == '1';
+  if (lc.choices.dense_tiles >= 0) return lc.choices.dense_tiles == 1;
   // measured: 128 result columns gain (128 -> 128 at 0.73 pairs per slot: 250 us against
   // 305 us), 64 result columns tie with the pair-list kernel
   if (d.C != 128) return false;
@@ -2215,21 +2201,18 @@ void launchDense(const LaunchCtx &lc, int Q, int C, const void *A, const void *p
 #undef DENSE_CASE
 }
 
-// Test switch: "1" builds every row map on the flat grid.
+// Row maps are built on the flat grid from this many workgroups of the per-offset grid on.
 constexpr int kFlatScatterFromBlocks = 16384;
-bool forceFlatScatter() {
-  const char *v = getenv("MLUOP_SPCONV_FLAT_SCATTER");
-  return v != nullptr && v[0] == '1';
-}
 
 // Caller brackets this with its timing marks.  dev_counts != nullptr: more offsets
 // than the inline tables hold, counts in device memory, grid kernel only.
-void enqueueScatterRowMap(hipStream_t stream, const int32_t *pairs, int L, int K,
+void enqueueScatterRowMap(const LaunchCtx &lc, const int32_t *pairs, int L, int K,
                           const OffsetCounts &inl, const int32_t *dev_counts, int max_count,
                           int row_col, int src_col, int n_rows, int n_src, int32_t *map) {
   const int gx = (max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256;
   if (dev_counts == nullptr && K <= kMaxInlineK &&
-      ((long long)gx * K > kFlatScatterFromBlocks || forceFlatScatter())) {
+      (lc.choices.flat_scatter == 1 ||
+       (lc.choices.flat_scatter != 0 && (long long)gx * K > kFlatScatterFromBlocks))) {
     OffsetBlocks ob;
     int blocks = 0;
     for (int k = 0; k < K; ++k) {
@@ -2237,11 +2220,11 @@ void enqueueScatterRowMap(hipStream_t stream, const int32_t *pairs, int L, int K
       blocks += inl.n[k] > 0 ? (inl.n[k] + 255) / 256 : 0;
     }
     if (blocks > 0)
-      scatterRowMapFlat<<<blocks, 256, 0, stream>>>(pairs, L, inl, ob, K, row_col, src_col, n_rows,
+      scatterRowMapFlat<<<blocks, 256, 0, lc.stream>>>(pairs, L, inl, ob, K, row_col, src_col, n_rows,
                                                    n_src, map);
     return;
   }
-  scatterRowMap<<<dim3(gx, K), 256, 0, stream>>>(pairs, L, inl, dev_counts, row_col, src_col,
+  scatterRowMap<<<dim3(gx, K), 256, 0, lc.stream>>>(pairs, L, inl, dev_counts, row_col, src_col,
                                                  n_rows, n_src, map);
 }
 
@@ -2249,7 +2232,7 @@ void launchScatterRowMap(const LaunchCtx &lc, const ConvProblem &p, const Gather
                          const GatherWorkspace &ws, const OffsetCounts &inl, int max_count) {
   if (max_count <= 0) return;
   lc.begin("scatterRowMap");
-  enqueueScatterRowMap(lc.stream, p.indice_pairs, p.L, p.K, inl, ws.dev_counts, max_count, d.row_col,
+  enqueueScatterRowMap(lc, p.indice_pairs, p.L, p.K, inl, ws.dev_counts, max_count, d.row_col,
                        d.src_col, d.R, d.n_src, ws.map);
   lc.end();
 }
@@ -2265,7 +2248,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
   if (use_mfma && listsUsable(p, d)) {
     // Pair lists in order (as far as the caller knows: the first kernel checks): the
     // gather kernel reads them cut by tile, no row map.
-    const bool dense = useDenseKernel(p, d);
+    const bool dense = useDenseKernel(lc, p, d);
     const int tile_cols = dense ? d.C : mfmaTileCols(p, d);
     const int tile_rows = dense ? kDenseTileRows : mfmaTileRows(tile_cols);
     int tile_shift = 0;
@@ -2302,7 +2285,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
     src.counts = inl;
     if (dense)
       launchDense<E, SegmentSource>(lc, d.Q, d.C, gathered, ws.packed, src, d.R, p.K, result);
-    else if (tile_cols == d.C && useWaveKernel(p.dtype, d.Q, d.C))
+    else if (tile_cols == d.C && useWaveKernel(lc, p.dtype, d.Q, d.C))
       launchWave<E>(lc, d.Q, d.C, gathered, ws.packed, src, d.R, p.K, result);
     else
       launchMfma<E, SegmentSource>(lc, d.Q, d.C, tile_cols, gathered, ws.packed, src, d.R, p.K, result);
@@ -2323,7 +2306,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
     lc.end();
     if (own_map) launchScatterRowMap(lc, p, d, ws, inl, max_count);
     const MapSource map = {entries, ws.filled};
-    if (useDenseKernel(p, d)) {
+    if (useDenseKernel(lc, p, d)) {
       n_filled = denseGridX(d.R);
       launchDense<E, MapSource>(lc, d.Q, d.C, gathered, ws.packed, map, d.R, p.K, result);
     } else {
@@ -2437,7 +2420,7 @@ void launchFilterMfmaInstance(const LaunchCtx &lc, const ConvProblem &p, const S
     sg.first[k] = blocks;
     blocks += sl <= kThinSlices ? (kChunks + kSliceSumWaves - 1) / kSliceSumWaves : kChunks;
   }
-  const int flat_mode = sliceSumMode();
+  const int flat_mode = lc.choices.flat_slice_sum;
   const bool flat = flat_mode == 1 || (flat_mode < 0 && kChunks * p.K > kFlatSumFromBlocks);
   lc.begin("sliceSum");
   if (flat)
@@ -2501,7 +2484,7 @@ void launchFilterGradTyped(const LaunchCtx &lc, const ConvProblem &p,
   // The MFMA path moves rows with 16-byte loads.
   const bool ptr_ok = ((reinterpret_cast<uintptr_t>(features) |
                         reinterpret_cast<uintptr_t>(output_grad)) & 15u) == 0;
-  if (filterMfmaShapeOk(p) && ptr_ok && !forceSimt()) {
+  if (filterMfmaShapeOk(p) && ptr_ok && lc.choices.gather_simt != 1) {
     launchFilterMfma<E>(lc, p, ws, inl, features, output_grad, filters_grad);
     return;
   }
@@ -2543,7 +2526,7 @@ hipError_t launchGatherConv(const LaunchCtx &lc, const ConvProblem &p, GatherDir
   const bool ptr_ok =
       ((reinterpret_cast<uintptr_t>(gathered) | reinterpret_cast<uintptr_t>(result)) & 15u) == 0;
   const bool use_mfma = mfmaShapeOk(p.dtype, d.Q, d.C) && ptr_ok && d.n_src <= (1 << 24) &&
-                        !forceSimt();
+                        lc.choices.gather_simt != 1;
   switch (p.dtype) {
     case ElemType::kHalf:
       launchGatherTyped<HalfElem>(lc, p, d, ws, inl, max_count, gathered, filters, use_mfma, result);
@@ -2589,7 +2572,7 @@ hipError_t buildRowMap(const LaunchCtx &lc, const int32_t *indice_pairs, const i
   fillInt32<<<1, 256, 0, lc.stream>>>(counter, 1, 0);
   if (max_count > 0) {
     lc.begin("scatterRowMap");
-    enqueueScatterRowMap(lc.stream, indice_pairs, shape.L, shape.K, inl,
+    enqueueScatterRowMap(lc, indice_pairs, shape.L, shape.K, inl,
                          shape.K > kMaxInlineK ? dev_counts : nullptr, max_count, shape.row_column,
                          1 - shape.row_column, shape.rows, shape.source_rows, map);
     lc.end();

@@ -123,6 +123,7 @@ SIGNATURES = {
                        ctypes.c_size_t, _vp, _vp]),
     # mlu_op_ext.h
     "mluOpExtSetKernelTiming": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "mluOpExtSetKernelChoice": (ctypes.c_int, [_vp, ctypes.c_int, ctypes.c_int]),
     "mluOpExtSetSparseConvExtendedModes": (ctypes.c_int, [_vp, ctypes.c_int]),
     "mluOpExtSetDistinctPairsPromise": (ctypes.c_int, [_vp, ctypes.c_int]),
     "mluOpExtGetRowMapSize": (ctypes.c_int, [_vp, ctypes.c_int64, ctypes.POINTER(ctypes.c_size_t)]),
@@ -189,6 +190,14 @@ class Handle:
 
     def set_kernel_timing(self, enable):
         check(lib().mluOpExtSetKernelTiming(self.ptr, 1 if enable else 0))
+
+    KERNEL_CHOICES = {"gather_simt": 0, "dense_tiles": 1, "wave_per_tile": 2, "flat_slice_sum": 3,
+                      "flat_scatter": 4}   # mluOpExtKernelChoice_t
+
+    def set_kernel_choice(self, which, value):
+        """mluOpExtSetKernelChoice: value None (the shape decides), False or True."""
+        v = -1 if value is None else (1 if value else 0)
+        check(lib().mluOpExtSetKernelChoice(self.ptr, self.KERNEL_CHOICES[which], v), "mluOpExtSetKernelChoice")
 
     def set_extended_modes(self, enable):
         """Accept inverse = 1 and tagged filters_grad layouts, which the reference rejects."""

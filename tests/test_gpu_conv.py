@@ -3,7 +3,6 @@
 Inputs are seeded fp32 values rounded through the tensor dtype (so device and oracle see the
 same numbers), the oracle accumulates in fp32 and its result is rounded through the output
 dtype, then diff1/diff2 are graded at the reference's thresholds (spconv_cases.THRESH)."""
-import os
 
 import numpy as np
 import pytest
@@ -38,10 +37,7 @@ def conv_case(seed, batch, space, L, ks, ci, co, sub_m, stride=(1, 1, 1)):
 def run_all_ops(handle, c, dtype_name, force_simt=False, check=("fwd", "bwd_data", "bwd_filter")):
     import torch
     import mluop_hip
-    if force_simt:
-        os.environ["MLUOP_SPCONV_FORCE_SIMT"] = "1"
-    else:
-        os.environ.pop("MLUOP_SPCONV_FORCE_SIMT", None)
+    handle.set_kernel_choice("gather_simt", True if force_simt else None)
     try:
         dev = "cuda"
         feats_r = round_to(c["feats"], dtype_name)
@@ -75,7 +71,7 @@ def run_all_ops(handle, c, dtype_name, force_simt=False, check=("fwd", "bwd_data
                                             "backward_filter")
         return res
     finally:
-        os.environ.pop("MLUOP_SPCONV_FORCE_SIMT", None)
+        handle.set_kernel_choice("gather_simt", None)
 
 
 SHAPES = [
@@ -130,12 +126,12 @@ def test_dense_kernel_matches_oracle(gpu_handle, shape, dtype_name):
     batch, space, L, ks, ci, co, sub_m, stride = shape
     print("dense conv case", shape, dtype_name, flush=True)
     c = conv_case(12, batch, space, L, ks, ci, co, sub_m, stride)
-    for force in ("1", "0"):
-        os.environ["MLUOP_SPCONV_DENSE"] = force
+    for force in (True, False):
+        gpu_handle.set_kernel_choice("dense_tiles", force)
         try:
             run_all_ops(gpu_handle, c, dtype_name, check=("fwd", "bwd_data"))
         finally:
-            os.environ.pop("MLUOP_SPCONV_DENSE", None)
+            gpu_handle.set_kernel_choice("dense_tiles", None)
 
 
 @pytest.mark.parametrize("layout_name", ["NDHWC", "NCDHW", "ARRAY"])
@@ -279,11 +275,11 @@ def test_repeated_coordinates_are_all_added(gpu_handle, shape, dtype_name):
              w=rng.uniform(-b, b, size=tuple(ks) + (ci, co)).astype(np.float32),
              dy=(rng.standard_normal((n_out, co)) * 1e-1).astype(np.float32))
     if dense:
-        os.environ["MLUOP_SPCONV_DENSE"] = "1"
+        gpu_handle.set_kernel_choice("dense_tiles", True)
     try:
         run_all_ops(gpu_handle, c, dtype_name)
     finally:
-        os.environ.pop("MLUOP_SPCONV_DENSE", None)
+        gpu_handle.set_kernel_choice("dense_tiles", None)
 
 
 @pytest.mark.parametrize("ci,co", [(64, 64), (13, 70)])
@@ -396,14 +392,14 @@ def test_flat_slice_sum_gives_the_bits_of_the_grid_one(gpu_handle, case, dtype_n
     got = {}
     try:
         for mode in ("1", "0"):
-            os.environ["MLUOP_SPCONV_FLAT_SLICE_SUM"] = mode
+            gpu_handle.set_kernel_choice("flat_slice_sum", mode == "1")
             if mode == "1":
                 run_all_ops(gpu_handle, c, dtype_name, check=("bwd_filter",))
             dw = mluop_hip.indice_conv_backward_filter(gpu_handle, feats_t, dy_t, pairs_t, num_host, c["ks"], True)
             torch.cuda.synchronize()
             got[mode] = dw.view(torch.int16 if dtype_name != "float32" else torch.int32).cpu()
     finally:
-        os.environ.pop("MLUOP_SPCONV_FLAT_SLICE_SUM", None)
+        gpu_handle.set_kernel_choice("flat_slice_sum", None)
     assert torch.equal(got["1"], got["0"])
 
 
@@ -427,7 +423,7 @@ def test_flat_row_map_scatter_gives_the_same_results(gpu_handle, shape, dtype_na
     got = {}
     try:
         for mode in ("1", "0"):
-            os.environ["MLUOP_SPCONV_FLAT_SCATTER"] = mode
+            gpu_handle.set_kernel_choice("flat_scatter", mode == "1")
             if mode == "1":
                 run_all_ops(gpu_handle, c, dtype_name, check=("fwd", "bwd_data"))
             out = mluop_hip.indice_conv_forward(gpu_handle, feats_t, w_t, mluop_hip.LAYOUT_ARRAY, pairs_t, num_host,
@@ -438,5 +434,5 @@ def test_flat_row_map_scatter_gives_the_same_results(gpu_handle, shape, dtype_na
             as_int = torch.int16 if dtype_name != "float32" else torch.int32
             got[mode] = (out.view(as_int).cpu(), dx.view(as_int).cpu())
     finally:
-        os.environ.pop("MLUOP_SPCONV_FLAT_SCATTER", None)
+        gpu_handle.set_kernel_choice("flat_scatter", None)
     assert torch.equal(got["1"][0], got["0"][0]) and torch.equal(got["1"][1], got["0"][1])

@@ -6,7 +6,6 @@ The oracle's inverse functions run the partner layer's rulebook backwards; they 
 CPU against dense conv_transpose3d (test_oracle_conv.py).  Inputs and grading are those of
 test_gpu_conv.py: seeded values rounded through the tensor dtype, diff1/diff2 at the reference's
 thresholds."""
-import os
 
 import numpy as np
 import pytest
@@ -153,15 +152,14 @@ def test_filters_grad_in_its_tagged_layout(extended_handle, shape, layout_name, 
     dy_r = round_to((rng.standard_normal((n_out, co)) * 1e-1).astype(np.float32), dtype_name)
     code = {"NDHWC": mluop_hip.LAYOUT_NDHWC, "NCDHW": mluop_hip.LAYOUT_NCDHW, "ARRAY": mluop_hip.LAYOUT_ARRAY}[
         layout_name]
-    if simt:
-        os.environ["MLUOP_SPCONV_FORCE_SIMT"] = "1"
+    extended_handle.set_kernel_choice("gather_simt", True if simt else None)
     try:
         dw = mluop_hip.indice_conv_backward_filter(extended_handle, to_torch(feats_r, dtype_name, "cuda"),
                                                    to_torch(dy_r, dtype_name, "cuda"), torch.from_numpy(pairs).cuda(),
                                                    [int(v) for v in num], ks, False, grad_layout=code)
         torch.cuda.synchronize()
     finally:
-        os.environ.pop("MLUOP_SPCONV_FORCE_SIMT", None)
+        extended_handle.set_kernel_choice("gather_simt", None)
     got = from_torch(dw)
     K = int(np.prod(ks))
     # back to [K, Ci, Co] with the oracle's own layout transpose (the one the forward tests pin)

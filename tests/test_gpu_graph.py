@@ -59,6 +59,54 @@ def test_captured_step_replays_bit_exactly():
     handle.close()
 
 
+def test_a_filter_of_175_offsets_is_captured_too():
+    """More offsets than the kernels carry counts for in their arguments (128): the counts reach
+    device memory through small launches, not through a copy the host waits for, so the three
+    operators can be captured with a 5x5x7 filter as well; every replay gives the eager bits."""
+    import torch
+    import mluop_hip as m
+    rng = np.random.default_rng(33)
+    batch, space, L, ci, co, ks = 1, (10, 16, 16), 1200, 32, 32, (5, 5, 7)
+    idx = torch.from_numpy(random_voxels(rng, batch, space, L)).cuda()
+    feats = torch.from_numpy(rng.standard_normal((L, ci)).astype(np.float32)).cuda().half()
+    w = torch.from_numpy((rng.standard_normal(ks + (ci, co)) * 0.05).astype(np.float32)).cuda().half()
+    dy = torch.from_numpy(rng.standard_normal((L, co)).astype(np.float32)).cuda().half()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        handle = m.make_handle_on_current_stream()
+        pairs, _, num, _ = m.get_indice_pairs(handle, idx, batch, space, ks, list(space), [2, 2, 3], [1, 1, 1],
+                                              [1, 1, 1], True)
+        side.synchronize()
+        num_host = num.cpu().tolist()
+        assert len(num_host) == 175 and num_host[87] == L
+
+        def step():
+            out = m.indice_conv_forward(handle, feats, w, m.LAYOUT_ARRAY, pairs, num_host, L, True)
+            dx = m.indice_conv_backward_data(handle, dy, w, m.LAYOUT_ARRAY, pairs, num_host, True, ci)
+            dw = m.indice_conv_backward_filter(handle, feats, dy, pairs, num_host, ks, True)
+            return out, dx, dw
+
+        eager = [t.clone() for t in step()]
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            captured = step()
+        for replay in range(3):
+            for t in captured:
+                t.fill_(0)
+            extra = step()
+            side.synchronize()
+            graph.replay()
+            side.synchronize()
+            for name, got, want in zip(("forward", "backward_data", "backward_filter"), captured, eager):
+                assert torch.equal(got, want), "replay %d: %s" % (replay, name)
+            for got, want in zip(extra, eager):
+                assert torch.equal(got, want)
+    torch.cuda.current_stream().wait_stream(side)
+    handle.close()
+
+
 def test_two_handles_on_two_streams_do_not_interfere():
     """Each handle owns its queue and its pinned read-back slot: two different problems enqueued
     alternately on two streams (default priority) give the results each gives alone."""
