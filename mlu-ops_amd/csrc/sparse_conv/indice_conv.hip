@@ -117,6 +117,7 @@ __global__ __launch_bounds__(256) void fillInt32(int32_t *dst, size_t n, int32_t
 // map[k][row] = partner row, for the first indice_num[k] pairs of every offset.
 // row_col / src_col select which pair column owns the result row (1 for
 // forward, 0 for backward data).  Indices outside their tensor are ignored.
+// Such pairs are counted: *ignored, which the map's fill left at -1, goes down by one each.
 // A map slot holds one partner.  Rulebooks built from distinct coordinates name a
 // result row once per offset at most; when coordinates repeat (or the pairs are
 // made up, as in test case files) several pairs of one offset can name the same
@@ -127,7 +128,7 @@ __global__ __launch_bounds__(256) void fillInt32(int32_t *dst, size_t n, int32_t
 __global__ __launch_bounds__(256) void scatterRowMap(const int32_t *pairs, int L,
                                                      OffsetCounts inl, const int32_t *dev_counts,
                                                      int row_col, int src_col, int n_rows,
-                                                     int n_src, int32_t *map) {
+                                                     int n_src, int32_t *map, int32_t *ignored) {
   const int k = blockIdx.y;
   const int n = offsetCount(inl, dev_counts, k);
   const int32_t *base = pairs + (size_t)k * 2 * L;
@@ -136,6 +137,8 @@ __global__ __launch_bounds__(256) void scatterRowMap(const int32_t *pairs, int L
     const int s = base[(size_t)src_col * L + p];
     if ((unsigned)r < (unsigned)n_rows && (unsigned)s < (unsigned)n_src)
       map[(size_t)k * n_rows + r] = s;
+    else
+      atomicSub(ignored, 1);  // rare: a pair outside its tensors; *ignored starts at -1
   }
 }
 
@@ -150,7 +153,8 @@ struct OffsetBlocks {
 __global__ __launch_bounds__(256) void scatterRowMapFlat(const int32_t *pairs, int L,
                                                          OffsetCounts inl, OffsetBlocks blocks,
                                                          int K, int row_col, int src_col,
-                                                         int n_rows, int n_src, int32_t *map) {
+                                                         int n_rows, int n_src, int32_t *map,
+                                                         int32_t *ignored) {
   // last offset whose first workgroup is not behind this one (an offset without
   // pairs shares its prefix with the next one and is never chosen)
   int lo = 0, hi = K - 1;
@@ -166,6 +170,8 @@ __global__ __launch_bounds__(256) void scatterRowMapFlat(const int32_t *pairs, i
   const int s = base[(size_t)src_col * L + p];
   if ((unsigned)r < (unsigned)n_rows && (unsigned)s < (unsigned)n_src)
     map[(size_t)k * n_rows + r] = s;
+  else
+    atomicSub(ignored, 1);
 }
 
 // ---- SIMT gather convolution -------------------------------------------------
@@ -1331,27 +1337,27 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
 }
 
 // ---- pairs that lost their map slot -----------------------------------------------
-// Runs behind every gather kernel as one workgroup and returns at once when the
-// kernels found as many filled map slots as there are pairs (always, for a rulebook
-// built from distinct coordinates).  Otherwise some pairs of one offset share a
-// result row, or lie outside their tensors: every pair is looked up again, the
-// first one that finds its partner in the slot claims it (the kernels have
-// multiplied that one), and each of the others is added to its result row here.
-// A touched row is rebuilt in an fp32 pool (kRepairPoolRows rows, indexed through
-// `shadow`): first the partners its map slots hold, as the kernel summed them, then
-// the lost pairs as the scan meets them, and it is rounded into the result once,
-// the same single rounding as any other row.  When more pairs are lost than the
-// pool has rows, the scan is repeated per block of kRepairPoolRows result rows and
-// looks only at the pairs of that block, so a row is never rebuilt twice.  Which
-// of the colliding pairs owned the slot depends on the order their stores landed
-// in, so the last bits of such rows can differ from run to run; rows without
-// collisions are not touched.
+// Runs behind every gather kernel and returns at once when the kernels found as many
+// filled map slots as there are pairs inside their tensors (always, for a rulebook built
+// from distinct coordinates).  Otherwise some pairs of one offset share a result row:
+// every pair is looked up again, the first one that finds its partner in the slot claims
+// it (the kernels have multiplied that one), and each of the others is added to its
+// result row here.  The result rows are split into windows of kRepairPoolRows rows; a
+// workgroup takes every gridDim.x-th window, reads all pairs and keeps those of its
+// window, so no two workgroups touch the same row, map slot or shadow entry.  A touched
+// row is rebuilt in the workgroup's fp32 pool (indexed through `shadow`): first the
+// partners its map slots hold, as the kernel summed them, then the lost pairs as the
+// scan meets them, and it is rounded into the result once, the same single rounding as
+// any other row.  Which of the colliding pairs owned the slot depends on the order their
+// stores landed in, so the last bits of such rows can differ from run to run; rows
+// without collisions are not touched.
 constexpr int kRepairPoolRows = 2048;
+constexpr int kRepairBlocks = 32;
 
 struct RepairScratch {
   int32_t *shadow;    // [R] pool row of a result row, or -1
-  int32_t *pool_row;  // [kRepairPoolRows] result row of a pool row
-  float *pool;        // [kRepairPoolRows, C]
+  int32_t *pool_row;  // [kRepairBlocks, kRepairPoolRows] result row of a pool row
+  float *pool;        // [kRepairBlocks, kRepairPoolRows, C]
 };
 
 template <typename E>
@@ -1359,7 +1365,8 @@ __global__ __launch_bounds__(256) void repairLostPairs(
     const typename E::storage *A, int Q, const typename E::storage *W, int64_t sK, int64_t sQ,
     int64_t sC, const int32_t *pairs, int L, int row_col, int src_col, int R, int n_src, int K,
     OffsetCounts inl, const int32_t *dev_counts, int32_t *map, const int32_t *filled,
-    int n_filled, int expected, int C, RepairScratch scratch, typename E::storage *result) {
+    int n_filled, int listed, const int32_t *ignored, int C, RepairScratch scratch,
+    typename E::storage *result) {
   __shared__ int s_found;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1371,22 +1378,59 @@ __global__ __launch_bounds__(256) void repairLostPairs(
   mine = waveInclusiveScan(mine);
   if (lane == 63) atomicAdd(&s_found, mine);
   __syncthreads();
-  if (s_found == expected) return;
+  // pairs the map could hold: all that are listed but those outside their tensors
+  if (s_found == listed - (-1 - *ignored)) return;
 
   __shared__ int s_row[256];
   __shared__ int s_src[256];
   __shared__ int s_wave_lost[4];
   __shared__ int s_pooled;  // pool rows in use
-  for (int i = tid; i < R; i += 256) scratch.shadow[i] = -1;
-  if (tid == 0) s_pooled = 0;
-  __syncthreads();
-  // no more rows can be touched than pairs are lost (or lie outside their tensors)
-  const int n_pass = expected - s_found <= kRepairPoolRows
-                         ? 1
-                         : (R + kRepairPoolRows - 1) / kRepairPoolRows;
-  for (int pass = 0; pass < n_pass; ++pass) {
-    const int r_lo = n_pass == 1 ? 0 : pass * kRepairPoolRows;
-    const int r_hi = n_pass == 1 ? R : (r_lo + kRepairPoolRows < R ? r_lo + kRepairPoolRows : R);
+  int32_t *pool_row = scratch.pool_row + (size_t)blockIdx.x * kRepairPoolRows;
+  float *pool = scratch.pool + (size_t)blockIdx.x * kRepairPoolRows * C;
+  // Products of gathered rows with filter slices, summed into pool row `at`: below 256
+  // result columns the workgroup is 256 / C groups of C threads, a group takes every
+  // groups-th reduction channel and the groups' sums meet in shared memory, in group order.
+  __shared__ float s_part[256];
+  const int groups = C < 256 ? 256 / C : 1;
+  const int g = C < 256 ? tid / C : 0;  // == groups: a thread without a part
+  const int c_first = C < 256 ? tid % C : tid;
+  // whole_row: every partner the map holds for result row `row` (claimed slots hold
+  // -2 - partner), stored; else gathered row `row` times slice `k_one`, added.
+  auto addProducts = [&](int at, int row, bool whole_row, int k_one) {
+    for (int c = c_first; c < C; c += 256) {
+      float part = 0.f;
+      if (g < groups) {
+        for (int kk = whole_row ? 0 : k_one; kk < (whole_row ? K : k_one + 1); ++kk) {
+          int from = row;
+          if (whole_row) {
+            const int m = map[(size_t)kk * R + row];
+            if (m == -1) continue;
+            from = m >= 0 ? m : -2 - m;
+          }
+          const typename E::storage *a = A + (size_t)from * Q;
+          const typename E::storage *w = W + (size_t)kk * sK + (size_t)c * sC;
+          for (int q = g; q < Q; q += groups) part += E::load(a + q) * E::load(w + (size_t)q * sQ);
+        }
+      }
+      if (groups > 1) {
+        s_part[tid] = part;
+        __syncthreads();
+        if (g == 0) {
+          part = 0.f;
+          for (int gg = 0; gg < groups; ++gg) part += s_part[gg * C + c];
+        }
+      }
+      if (g == 0) pool[(size_t)at * C + c] = whole_row ? part : pool[(size_t)at * C + c] + part;
+      if (groups > 1) __syncthreads();
+    }
+  };
+  const int n_windows = (R + kRepairPoolRows - 1) / kRepairPoolRows;
+  for (int window = blockIdx.x; window < n_windows; window += gridDim.x) {
+    const int r_lo = window * kRepairPoolRows;
+    const int r_hi = r_lo + kRepairPoolRows < R ? r_lo + kRepairPoolRows : R;
+    for (int i = r_lo + tid; i < r_hi; i += 256) scratch.shadow[i] = -1;
+    if (tid == 0) s_pooled = 0;
+    __syncthreads();
     for (int k = 0; k < K; ++k) {
       const int n = offsetCount(inl, dev_counts, k);
       const int32_t *base = pairs + (size_t)k * 2 * L;
@@ -1396,13 +1440,17 @@ __global__ __launch_bounds__(256) void repairLostPairs(
         bool lost = false;
         if (p < n) {
           r = base[(size_t)row_col * L + p];
-          src = base[(size_t)src_col * L + p];
-          if (r >= r_lo && r < r_hi && (unsigned)src < (unsigned)n_src) {
-            int32_t *slot = map + (size_t)k * R + r;
-            // the claimed slot holds -2 - partner: no pair finds itself there twice
-            lost = !(*slot == src && atomicCAS(slot, src, -2 - src) == src);
+          if (r >= r_lo && r < r_hi) {
+            src = base[(size_t)src_col * L + p];
+            if ((unsigned)src < (unsigned)n_src) {
+              int32_t *slot = map + (size_t)k * R + r;
+              // the claimed slot holds -2 - partner: no pair finds itself there twice
+              lost = !(*slot == src && atomicCAS(slot, src, -2 - src) == src);
+            }
           }
         }
+        // most steps hold no pair of this window at all
+        if (!__syncthreads_or(lost)) continue;
         // lost pairs of this step in pair order
         const unsigned long long b = __ballot(lost);
         if (lane == 0) s_wave_lost[wave] = __popcll(b);
@@ -1426,45 +1474,23 @@ __global__ __launch_bounds__(256) void repairLostPairs(
             __syncthreads();  // everybody has read the pool's fill state
             if (tid == 0) {
               scratch.shadow[row] = at;
-              scratch.pool_row[at] = row;
+              pool_row[at] = row;
               s_pooled = at + 1;
             }
             // what the gather kernel summed: the partner every slot of the row holds
-            // (claimed slots hold -2 - partner)
-            for (int c = tid; c < C; c += 256) {
-              float sum = 0.f;
-              for (int kk = 0; kk < K; ++kk) {
-                const int m = map[(size_t)kk * R + row];
-                if (m == -1) continue;
-                const typename E::storage *a = A + (size_t)(m >= 0 ? m : -2 - m) * Q;
-                const typename E::storage *w = W + (size_t)kk * sK + (size_t)c * sC;
-                float dot = 0.f;
-                for (int q = 0; q < Q; ++q) dot += E::load(a + q) * E::load(w + (size_t)q * sQ);
-                sum += dot;
-              }
-              scratch.pool[(size_t)at * C + c] = sum;
-            }
+            addProducts(at, row, true, 0);
           }
-          const typename E::storage *a = A + (size_t)s_src[i] * Q;
-          for (int c = tid; c < C; c += 256) {
-            const typename E::storage *w = W + (size_t)k * sK + (size_t)c * sC;
-            float dot = 0.f;
-            for (int q = 0; q < Q; ++q) dot += E::load(a + q) * E::load(w + (size_t)q * sQ);
-            scratch.pool[(size_t)at * C + c] += dot;
-          }
+          addProducts(at, s_src[i], false, k);
           __syncthreads();  // shadow and the pool row are in place for the next pair
         }
       }
     }
-    // round the rebuilt rows into the result; their pool rows are free again
+    // round the rebuilt rows into the result; the pool is free for the next window
     const int pooled = s_pooled;
     for (int i = 0; i < pooled; ++i) {
-      const int r = scratch.pool_row[i];
-      for (int c = tid; c < C; c += 256)
-        E::store(result + (size_t)r * C + c, scratch.pool[(size_t)i * C + c]);
+      const int r = pool_row[i];
+      for (int c = tid; c < C; c += 256) E::store(result + (size_t)r * C + c, pool[(size_t)i * C + c]);
     }
-    __syncthreads();
-    if (tid == 0) s_pooled = 0;
     __syncthreads();
   }
 }
@@ -1985,6 +2011,12 @@ struct GatherWorkspace {
   size_t bytes = 0;
 };
 
+// Workgroups of repairLostPairs: one per window of result rows, kRepairBlocks at most.
+int repairBlocks(int R) {
+  const int windows = (R + kRepairPoolRows - 1) / kRepairPoolRows;
+  return windows < 1 ? 1 : (windows > kRepairBlocks ? kRepairBlocks : windows);
+}
+
 GatherWorkspace carveGather(const ConvProblem &p, const GatherDims &d, void *base) {
   GatherWorkspace ws;
   char *ptr = alignPtr(base);
@@ -2002,9 +2034,11 @@ GatherWorkspace carveGather(const ConvProblem &p, const GatherDims &d, void *bas
   }
   ws.filled = reinterpret_cast<int32_t *>(take(((size_t)d.R / 32 + 16) * 4));
   ws.shadow = reinterpret_cast<int32_t *>(take((size_t)d.R * 4));
-  ws.pool_row = reinterpret_cast<int32_t *>(take((size_t)kRepairPoolRows * 4));
-  ws.pool = reinterpret_cast<float *>(take((size_t)kRepairPoolRows * d.C * 4));
-  ws.map = reinterpret_cast<int32_t *>(take((size_t)p.K * d.R * 4));
+  const size_t repair_blocks = (size_t)repairBlocks(d.R);
+  ws.pool_row = reinterpret_cast<int32_t *>(take(repair_blocks * kRepairPoolRows * 4));
+  ws.pool = reinterpret_cast<float *>(take(repair_blocks * kRepairPoolRows * d.C * 4));
+  // one word behind the map counts the pairs that lie outside their tensors
+  ws.map = reinterpret_cast<int32_t *>(take((size_t)p.K * d.R * 4 + 16));
   if (mfmaShapeOk(p.dtype, d.Q, d.C)) {
     // reduction channels are padded to whole 16-byte fragments (32 for the 2-byte types)
     const size_t chunk = 64 / elemSize(p.dtype);
@@ -2208,7 +2242,8 @@ constexpr int kFlatScatterFromBlocks = 16384;
 // than the inline tables hold, counts in device memory, grid kernel only.
 void enqueueScatterRowMap(const LaunchCtx &lc, const int32_t *pairs, int L, int K,
                           const OffsetCounts &inl, const int32_t *dev_counts, int max_count,
-                          int row_col, int src_col, int n_rows, int n_src, int32_t *map) {
+                          int row_col, int src_col, int n_rows, int n_src, int32_t *map,
+                          int32_t *ignored) {
   const int gx = (max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256;
   if (dev_counts == nullptr && K <= kMaxInlineK &&
       (lc.choices.flat_scatter == 1 ||
@@ -2221,11 +2256,11 @@ void enqueueScatterRowMap(const LaunchCtx &lc, const int32_t *pairs, int L, int 
     }
     if (blocks > 0)
       scatterRowMapFlat<<<blocks, 256, 0, lc.stream>>>(pairs, L, inl, ob, K, row_col, src_col, n_rows,
-                                                   n_src, map);
+                                                   n_src, map, ignored);
     return;
   }
   scatterRowMap<<<dim3(gx, K), 256, 0, lc.stream>>>(pairs, L, inl, dev_counts, row_col, src_col,
-                                                 n_rows, n_src, map);
+                                                 n_rows, n_src, map, ignored);
 }
 
 void launchScatterRowMap(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d,
@@ -2233,7 +2268,7 @@ void launchScatterRowMap(const LaunchCtx &lc, const ConvProblem &p, const Gather
   if (max_count <= 0) return;
   lc.begin("scatterRowMap");
   enqueueScatterRowMap(lc, p.indice_pairs, p.L, p.K, inl, ws.dev_counts, max_count, d.row_col,
-                       d.src_col, d.R, d.n_src, ws.map);
+                       d.src_col, d.R, d.n_src, ws.map, ws.map + (size_t)p.K * d.R);
   lc.end();
 }
 
@@ -2301,7 +2336,8 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
     const int pack_blocks = gridFor(frags, 512);
     lc.begin("fillMapPackFilter");
     fillMapPackFilter<E><<<fill_blocks + pack_blocks, 256, 0, lc.stream>>>(
-        ws.map, map_elems, fill_blocks, static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K,
+        ws.map, map_elems + 4 /* and the word that counts ignored pairs */, fill_blocks,
+        static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K,
         d.Q, d.C, static_cast<S *>(ws.packed));
     lc.end();
     if (own_map) launchScatterRowMap(lc, p, d, ws, inl, max_count);
@@ -2317,7 +2353,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
   } else {
     if (own_map) {
       lc.begin("fillInt32");
-      fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems, -1);
+      fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems + 4, -1);
       lc.end();
       launchScatterRowMap(lc, p, d, ws, inl, max_count);
     }
@@ -2331,17 +2367,18 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
     lc.end();
   }
   if (p.distinct_pairs || !own_map) return;  // a map built ahead was checked when it was built
-  // one workgroup that returns at once unless pairs of one offset share a result row
+  // returns at once unless pairs of one offset share a result row
   long long expected = 0;
   for (int k = 0; k < p.K; ++k) {
     const int64_t n = p.indice_num[k];
     expected += n < 0 ? 0 : (n > p.L ? p.L : n);
   }
   lc.begin("repairLostPairs");
-  repairLostPairs<E><<<1, 256, 0, lc.stream>>>(
+  repairLostPairs<E><<<repairBlocks(d.R), 256, 0, lc.stream>>>(
       static_cast<const S *>(gathered), d.Q, static_cast<const S *>(f.base), f.stride_k, sQ, sC,
       p.indice_pairs, p.L, d.row_col, d.src_col, d.R, d.n_src, p.K, inl, ws.dev_counts, ws.map,
-      ws.filled, n_filled, (int)expected, d.C, RepairScratch{ws.shadow, ws.pool_row, ws.pool},
+      ws.filled, n_filled, (int)expected, ws.map + map_elems, d.C,
+      RepairScratch{ws.shadow, ws.pool_row, ws.pool},
       static_cast<S *>(result));
   lc.end();
 }
@@ -2574,7 +2611,8 @@ hipError_t buildRowMap(const LaunchCtx &lc, const int32_t *indice_pairs, const i
     lc.begin("scatterRowMap");
     enqueueScatterRowMap(lc, indice_pairs, shape.L, shape.K, inl,
                          shape.K > kMaxInlineK ? dev_counts : nullptr, max_count, shape.row_column,
-                         1 - shape.row_column, shape.rows, shape.source_rows, map);
+                         1 - shape.row_column, shape.rows, shape.source_rows, map,
+                         counter + 1);  // nobody reads this count: the block behind `counter` is spare
     lc.end();
   }
   if (filled_host == nullptr) return hipGetLastError();

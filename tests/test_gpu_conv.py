@@ -282,6 +282,92 @@ def test_repeated_coordinates_are_all_added(gpu_handle, shape, dtype_name):
         gpu_handle.set_kernel_choice("dense_tiles", None)
 
 
+def test_a_hundred_thousand_repeated_coordinates_finish_in_bounded_time(gpu_handle):
+    """300 000 rows of which 100 000 repeat the coordinates of another row (a cloud that was
+    never made unique): about a million pairs lose their map slot.  Their repair is spread over
+    windows of result rows, each with a workgroup of its own, and must not take the queue for
+    longer than a second; forward and backward data are graded against the oracle."""
+    import time
+    import torch
+    import mluop_hip
+    rng = np.random.default_rng(43)
+    space, ks, ci, co = (24, 96, 96), (3, 3, 3), 32, 32
+    idx = random_voxels(rng, 1, space, 200000, duplicates=100000)
+    pairs, num, n_out = build_rulebook(idx, 1, space, ks, [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+    lost = sum(int(num[k]) - len(np.unique(pairs[k, 1, :num[k]])) for k in range(27))
+    print("pairs", int(num.sum()), "of which lose their slot in forward:", lost, flush=True)
+    assert lost > 500000
+    feats = round_to(rng.standard_normal((idx.shape[0], ci)).astype(np.float32), "float16")
+    w = round_to(rng.uniform(-0.05, 0.05, size=ks + (ci, co)).astype(np.float32), "float16")
+    dy = round_to((rng.standard_normal((n_out, co)) * 0.1).astype(np.float32), "float16")
+    t_pairs = torch.from_numpy(pairs).cuda()
+    num_host = [int(v) for v in num]
+    t_f, t_w, t_dy = (to_torch(a, "float16", "cuda") for a in (feats, w, dy))
+    w_k = w.reshape(27, ci, co)
+    for _ in range(2):   # the second call is the timed one
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = mluop_hip.indice_conv_forward(gpu_handle, t_f, t_w, mluop_hip.LAYOUT_ARRAY, t_pairs, num_host, n_out,
+                                            True)
+        torch.cuda.synchronize()
+        fwd_s = time.perf_counter() - t0
+    print("forward with repairs: %.1f ms" % (fwd_s * 1e3), flush=True)
+    assert fwd_s < 1.0
+    check_close(from_torch(out), oracle.forward(feats, w_k, pairs, num, n_out), "float16", "forward")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dx = mluop_hip.indice_conv_backward_data(gpu_handle, t_dy, t_w, mluop_hip.LAYOUT_ARRAY, t_pairs, num_host, True,
+                                             ci)
+    torch.cuda.synchronize()
+    assert time.perf_counter() - t0 < 1.0
+    check_close(from_torch(dx), oracle.backward_data(dy, w_k, pairs, num), "float16", "backward_data")
+
+
+def test_pairs_outside_their_tensors_do_not_start_the_repair_scan(gpu_handle):
+    """Pairs that name a row outside the tensors are skipped (the reference would read out of
+    bounds); the map can never hold them, and the check for lost pairs must not take them for
+    collisions: the repair kernel returns as fast as it does for a clean rulebook."""
+    import torch
+    import mluop_hip
+    rng = np.random.default_rng(44)
+    space, ks, ci, co, L = (16, 40, 40), (3, 3, 3), 32, 32, 20000
+    idx = random_voxels(rng, 1, space, L)
+    pairs, num, n_out = build_rulebook(idx, 1, space, ks, [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+    broken = pairs.copy()
+    for k in range(27):
+        n = int(num[k])
+        where = rng.choice(n, size=min(n, 50), replace=False)
+        broken[k, 1, where[:25]] = n_out + 5          # result row outside
+        broken[k, 0, where[25:]] = -7                 # gathered row outside
+    feats = round_to(rng.standard_normal((L, ci)).astype(np.float32), "float16")
+    w = round_to(rng.uniform(-0.05, 0.05, size=ks + (ci, co)).astype(np.float32), "float16")
+    t_f, t_w = to_torch(feats, "float16", "cuda"), to_torch(w, "float16", "cuda")
+    num_host = [int(v) for v in num]
+    times = {}
+    for name, tensor in (("clean", pairs), ("broken", broken)):
+        t_pairs = torch.from_numpy(tensor).cuda()
+        mluop_hip.indice_conv_forward(gpu_handle, t_f, t_w, mluop_hip.LAYOUT_ARRAY, t_pairs, num_host, n_out, True)
+        gpu_handle.set_kernel_timing(True)
+        try:
+            out = mluop_hip.indice_conv_forward(gpu_handle, t_f, t_w, mluop_hip.LAYOUT_ARRAY, t_pairs, num_host,
+                                                n_out, True)
+            times[name] = dict(gpu_handle.kernel_timings())["repairLostPairs"]
+        finally:
+            gpu_handle.set_kernel_timing(False)
+    valid = broken.copy()                              # the oracle's view: those pairs do not exist
+    keep_num = num.copy()
+    for k in range(27):
+        n = int(num[k])
+        ok = (broken[k, 1, :n] < n_out) & (broken[k, 0, :n] >= 0)
+        valid[k, :, :n] = -1
+        valid[k, :, :int(ok.sum())] = broken[k][:, :n][:, ok]
+        keep_num[k] = int(ok.sum())
+    check_close(from_torch(out), oracle.forward(feats, w.reshape(27, ci, co), valid, keep_num, n_out), "float16",
+                "forward")
+    print("repairLostPairs ms:", times, flush=True)
+    assert times["broken"] < 5 * times["clean"] + 0.02
+
+
 @pytest.mark.parametrize("ci,co", [(64, 64), (13, 70)])
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 def test_made_up_pairs_with_repeats_everywhere(gpu_handle, ci, co, dtype_name):
