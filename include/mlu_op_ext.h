@@ -30,7 +30,9 @@ typedef enum {
   MLUOP_EXT_KERNEL_DENSE_TILES = 1,    /* register-accumulating gather kernel */
   MLUOP_EXT_KERNEL_WAVE_PER_TILE = 2,  /* one-wavefront-per-tile gather kernel */
   MLUOP_EXT_KERNEL_FLAT_SLICE_SUM = 3, /* backward filter: partial tiles summed on a flat grid */
-  MLUOP_EXT_KERNEL_FLAT_SCATTER = 4    /* row maps built on a flat grid */
+  MLUOP_EXT_KERNEL_FLAT_SCATTER = 4,   /* row maps built on a flat grid */
+  MLUOP_EXT_KERNEL_SMALL_MAP_CHUNKS = 5 /* 1: row maps cover 2048 result rows at a time instead of
+                                           as many as 64 MiB hold (runs the chunked path on small inputs) */
 } mluOpExtKernelChoice_t;
 
 mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelChoice(mluOpHandle_t handle,

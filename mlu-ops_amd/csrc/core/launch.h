@@ -55,6 +55,7 @@ struct KernelChoices {
   int wave_per_tile = -1;   // the one-wavefront-per-tile gather kernel
   int flat_slice_sum = -1;  // backward filter: partial tiles summed on the flat grid
   int flat_scatter = -1;    // 1: row maps built on the flat grid
+  int small_map_chunks = -1;  // 1: row maps cover 2048 result rows at a time (the chunked path, on small inputs)
 };
 
 class LaunchCtx {

@@ -114,32 +114,43 @@ __global__ __launch_bounds__(256) void fillInt32(int32_t *dst, size_t n, int32_t
   for (; i < n; i += stride) dst[i] = value;
 }
 
-// map[k][row] = partner row, for the first indice_num[k] pairs of every offset.
+// map[k][row - row_base] = partner row, for the first indice_num[k] pairs of every offset
+// whose row lies in [row_base, row_base + n_rows): the map of one chunk of result rows.
 // row_col / src_col select which pair column owns the result row (1 for
-// forward, 0 for backward data).  Indices outside their tensor are ignored.
-// Such pairs are counted: *ignored, which the map's fill left at -1, goes down by one each.
+// forward, 0 for backward data).  Pairs that name a row outside their tensors are ignored.
+// Every workgroup leaves the number of pairs it put into the map in accepted[its index]
+// (unless accepted is null).
 // A map slot holds one partner.  Rulebooks built from distinct coordinates name a
 // result row once per offset at most; when coordinates repeat (or the pairs are
 // made up, as in test case files) several pairs of one offset can name the same
 // row, and the reference adds them all.  Plain stores keep whichever of them was
 // written last; every workgroup of a gather kernel records how many slots of its
 // tile it found filled, and repairLostPairs adds what the other pairs would have
-// contributed when those counts fall short of the number of pairs.
+// contributed when those counts fall short of the number of accepted pairs.
 __global__ __launch_bounds__(256) void scatterRowMap(const int32_t *pairs, int L,
                                                      OffsetCounts inl, const int32_t *dev_counts,
-                                                     int row_col, int src_col, int n_rows,
-                                                     int n_src, int32_t *map, int32_t *ignored) {
+                                                     int row_col, int src_col, int row_base,
+                                                     int n_rows, int n_src, int32_t *map,
+                                                     int32_t *accepted) {
   const int k = blockIdx.y;
   const int n = offsetCount(inl, dev_counts, k);
   const int32_t *base = pairs + (size_t)k * 2 * L;
+  int mine = 0;
   for (int p = blockIdx.x * 256 + threadIdx.x; p < n; p += gridDim.x * 256) {
-    const int r = base[(size_t)row_col * L + p];
+    const int r = base[(size_t)row_col * L + p] - row_base;
     const int s = base[(size_t)src_col * L + p];
-    if ((unsigned)r < (unsigned)n_rows && (unsigned)s < (unsigned)n_src)
+    if ((unsigned)r < (unsigned)n_rows && (unsigned)s < (unsigned)n_src) {
       map[(size_t)k * n_rows + r] = s;
-    else
-      atomicSub(ignored, 1);  // rare: a pair outside its tensors; *ignored starts at -1
+      ++mine;
+    }
   }
+  __shared__ int s_accepted;
+  if (threadIdx.x == 0) s_accepted = 0;
+  __syncthreads();
+  mine = waveInclusiveScan(mine);
+  if ((threadIdx.x & 63) == 63 && mine != 0) atomicAdd(&s_accepted, mine);
+  __syncthreads();
+  if (threadIdx.x == 0 && accepted != nullptr) accepted[blockIdx.y * gridDim.x + blockIdx.x] = s_accepted;
 }
 
 // The same on a flat grid: an offset gets the workgroups its pairs need and no
@@ -153,8 +164,8 @@ struct OffsetBlocks {
 __global__ __launch_bounds__(256) void scatterRowMapFlat(const int32_t *pairs, int L,
                                                          OffsetCounts inl, OffsetBlocks blocks,
                                                          int K, int row_col, int src_col,
-                                                         int n_rows, int n_src, int32_t *map,
-                                                         int32_t *ignored) {
+                                                         int row_base, int n_rows, int n_src,
+                                                         int32_t *map, int32_t *accepted) {
   // last offset whose first workgroup is not behind this one (an offset without
   // pairs shares its prefix with the next one and is never chosen)
   int lo = 0, hi = K - 1;
@@ -164,14 +175,16 @@ __global__ __launch_bounds__(256) void scatterRowMapFlat(const int32_t *pairs, i
   }
   const int k = lo;
   const int p = ((int)blockIdx.x - blocks.first[k]) * 256 + threadIdx.x;
-  if (p >= inl.n[k]) return;
-  const int32_t *base = pairs + (size_t)k * 2 * L;
-  const int r = base[(size_t)row_col * L + p];
-  const int s = base[(size_t)src_col * L + p];
-  if ((unsigned)r < (unsigned)n_rows && (unsigned)s < (unsigned)n_src)
-    map[(size_t)k * n_rows + r] = s;
-  else
-    atomicSub(ignored, 1);
+  bool ok = false;
+  if (p < inl.n[k]) {
+    const int32_t *base = pairs + (size_t)k * 2 * L;
+    const int r = base[(size_t)row_col * L + p] - row_base;
+    const int s = base[(size_t)src_col * L + p];
+    ok = (unsigned)r < (unsigned)n_rows && (unsigned)s < (unsigned)n_src;
+    if (ok) map[(size_t)k * n_rows + r] = s;
+  }
+  const int total = __syncthreads_count(ok);
+  if (threadIdx.x == 0 && accepted != nullptr) accepted[blockIdx.x] = total;
 }
 
 // ---- SIMT gather convolution -------------------------------------------------
@@ -1364,22 +1377,23 @@ template <typename E>
 __global__ __launch_bounds__(256) void repairLostPairs(
     const typename E::storage *A, int Q, const typename E::storage *W, int64_t sK, int64_t sQ,
     int64_t sC, const int32_t *pairs, int L, int row_col, int src_col, int R, int n_src, int K,
-    OffsetCounts inl, const int32_t *dev_counts, int32_t *map, const int32_t *filled,
-    int n_filled, int listed, const int32_t *ignored, int C, RepairScratch scratch,
-    typename E::storage *result) {
+    int row_base, OffsetCounts inl, const int32_t *dev_counts, int32_t *map,
+    const int32_t *filled, int n_filled, const int32_t *accepted, int n_accepted, int C,
+    RepairScratch scratch, typename E::storage *result) {
   __shared__ int s_found;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   if (tid == 0) s_found = 0;
   __syncthreads();
+  // filled slots the gather kernel met, less the pairs the scatter put into the map
   int mine = 0;
   for (int i = tid; i < n_filled; i += 256) mine += filled[i];
+  for (int i = tid; i < n_accepted; i += 256) mine -= accepted[i];
   mine = waveInclusiveScan(mine);
-  if (lane == 63) atomicAdd(&s_found, mine);
+  if (lane == 63 && mine != 0) atomicAdd(&s_found, mine);
   __syncthreads();
-  // pairs the map could hold: all that are listed but those outside their tensors
-  if (s_found == listed - (-1 - *ignored)) return;
+  if (s_found == 0) return;
 
   __shared__ int s_row[256];
   __shared__ int s_src[256];
@@ -1439,7 +1453,7 @@ __global__ __launch_bounds__(256) void repairLostPairs(
         int r = -1, src = -1;
         bool lost = false;
         if (p < n) {
-          r = base[(size_t)row_col * L + p];
+          r = base[(size_t)row_col * L + p] - row_base;
           if (r >= r_lo && r < r_hi) {
             src = base[(size_t)src_col * L + p];
             if ((unsigned)src < (unsigned)n_src) {
@@ -2003,6 +2017,8 @@ struct GatherWorkspace {
   unsigned long long *verdict = nullptr;
   int32_t *dev_counts = nullptr;
   int32_t *filled = nullptr;  // map slots the gather kernel's workgroups found filled
+  int32_t *accepted = nullptr;  // pairs the map scatter's workgroups put into the map
+  int map_rows = 0;           // result rows one map holds: the rows of a chunk
   int32_t *shadow = nullptr;  // repairLostPairs' scratch, touched only when pairs collide
   int32_t *pool_row = nullptr;
   float *pool = nullptr;
@@ -2017,8 +2033,27 @@ int repairBlocks(int R) {
   return windows < 1 ? 1 : (windows > kRepairBlocks ? kRepairBlocks : windows);
 }
 
+// Entries of the `accepted` array the scatter kernels may write for K offsets of up to L pairs.
+size_t scatterBlocksBound(int K, int L) {
+  const size_t flat = (size_t)K * ((size_t)L / 256 + 1);
+  const size_t grid = (size_t)K * 1024;
+  return flat > grid ? flat : grid;
+}
+
+// The row map is built and used for a chunk of result rows at a time, so that it stays
+// below kMapChunkBytes however many offsets and rows there are (a multiple of the repair
+// window, hence of every tile height).
+constexpr size_t kMapChunkBytes = 64u << 20;
+int mapChunkRows(int K, int R) {
+  size_t rows = kMapChunkBytes / ((size_t)K * 4);
+  rows = rows / kRepairPoolRows * kRepairPoolRows;
+  if (rows < (size_t)kRepairPoolRows) rows = kRepairPoolRows;
+  return rows < (size_t)R ? (int)rows : R;
+}
+
 GatherWorkspace carveGather(const ConvProblem &p, const GatherDims &d, void *base) {
   GatherWorkspace ws;
+  ws.map_rows = mapChunkRows(p.K, d.R);
   char *ptr = alignPtr(base);
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -2033,12 +2068,12 @@ GatherWorkspace carveGather(const ConvProblem &p, const GatherDims &d, void *bas
     ws.verdict = reinterpret_cast<unsigned long long *>(take(8));
   }
   ws.filled = reinterpret_cast<int32_t *>(take(((size_t)d.R / 32 + 16) * 4));
-  ws.shadow = reinterpret_cast<int32_t *>(take((size_t)d.R * 4));
-  const size_t repair_blocks = (size_t)repairBlocks(d.R);
+  ws.accepted = reinterpret_cast<int32_t *>(take(scatterBlocksBound(p.K, p.L) * 4));
+  ws.shadow = reinterpret_cast<int32_t *>(take((size_t)ws.map_rows * 4));
+  const size_t repair_blocks = (size_t)repairBlocks(ws.map_rows);
   ws.pool_row = reinterpret_cast<int32_t *>(take(repair_blocks * kRepairPoolRows * 4));
   ws.pool = reinterpret_cast<float *>(take(repair_blocks * kRepairPoolRows * d.C * 4));
-  // one word behind the map counts the pairs that lie outside their tensors
-  ws.map = reinterpret_cast<int32_t *>(take((size_t)p.K * d.R * 4 + 16));
+  ws.map = reinterpret_cast<int32_t *>(take((size_t)p.K * ws.map_rows * 4));
   if (mfmaShapeOk(p.dtype, d.Q, d.C)) {
     // reduction channels are padded to whole 16-byte fragments (32 for the 2-byte types)
     const size_t chunk = 64 / elemSize(p.dtype);
@@ -2239,11 +2274,12 @@ void launchDense(const LaunchCtx &lc, int Q, int C, const void *A, const void *p
 constexpr int kFlatScatterFromBlocks = 16384;
 
 // Caller brackets this with its timing marks.  dev_counts != nullptr: more offsets
-// than the inline tables hold, counts in device memory, grid kernel only.
-void enqueueScatterRowMap(const LaunchCtx &lc, const int32_t *pairs, int L, int K,
-                          const OffsetCounts &inl, const int32_t *dev_counts, int max_count,
-                          int row_col, int src_col, int n_rows, int n_src, int32_t *map,
-                          int32_t *ignored) {
+// than the inline tables hold, counts in device memory, grid kernel only.  Returns the
+// number of workgroups, each of which writes one entry of `accepted`.
+int enqueueScatterRowMap(const LaunchCtx &lc, const int32_t *pairs, int L, int K,
+                         const OffsetCounts &inl, const int32_t *dev_counts, int max_count,
+                         int row_col, int src_col, int row_base, int n_rows, int n_src,
+                         int32_t *map, int32_t *accepted) {
   const int gx = (max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256;
   if (dev_counts == nullptr && K <= kMaxInlineK &&
       (lc.choices.flat_scatter == 1 ||
@@ -2255,21 +2291,25 @@ void enqueueScatterRowMap(const LaunchCtx &lc, const int32_t *pairs, int L, int 
       blocks += inl.n[k] > 0 ? (inl.n[k] + 255) / 256 : 0;
     }
     if (blocks > 0)
-      scatterRowMapFlat<<<blocks, 256, 0, lc.stream>>>(pairs, L, inl, ob, K, row_col, src_col, n_rows,
-                                                   n_src, map, ignored);
-    return;
+      scatterRowMapFlat<<<blocks, 256, 0, lc.stream>>>(pairs, L, inl, ob, K, row_col, src_col,
+                                                   row_base, n_rows, n_src, map, accepted);
+    return blocks;
   }
   scatterRowMap<<<dim3(gx, K), 256, 0, lc.stream>>>(pairs, L, inl, dev_counts, row_col, src_col,
-                                                 n_rows, n_src, map, ignored);
+                                                 row_base, n_rows, n_src, map, accepted);
+  return gx * K;
 }
 
-void launchScatterRowMap(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d,
-                         const GatherWorkspace &ws, const OffsetCounts &inl, int max_count) {
-  if (max_count <= 0) return;
+// The map of result rows [row_base, row_base + n_rows); returns the entries of ws.accepted written.
+int launchScatterRowMap(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d,
+                        const GatherWorkspace &ws, const OffsetCounts &inl, int max_count,
+                        int row_base, int n_rows) {
+  if (max_count <= 0) return 0;
   lc.begin("scatterRowMap");
-  enqueueScatterRowMap(lc, p.indice_pairs, p.L, p.K, inl, ws.dev_counts, max_count, d.row_col,
-                       d.src_col, d.R, d.n_src, ws.map, ws.map + (size_t)p.K * d.R);
+  const int n = enqueueScatterRowMap(lc, p.indice_pairs, p.L, p.K, inl, ws.dev_counts, max_count,
+                                     d.row_col, d.src_col, row_base, n_rows, d.n_src, ws.map, ws.accepted);
   lc.end();
+  return n;
 }
 
 template <typename E>
@@ -2326,61 +2366,67 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
       launchMfma<E, SegmentSource>(lc, d.Q, d.C, tile_cols, gathered, ws.packed, src, d.R, p.K, result);
     return;
   }
-  const size_t map_elems = (size_t)p.K * d.R;
   const bool own_map = p.row_map == nullptr;  // else: built ahead, nothing to clear or fill
-  const int32_t *entries = own_map ? ws.map : p.row_map;
-  int n_filled = 0;  // workgroups along x of the gather kernel = slot counts it leaves
-  if (use_mfma) {
-    const size_t frags = (size_t)p.K * (d.C / 16) * ((d.Q + E::kChunk - 1) / E::kChunk) * 64;
-    const int fill_blocks = own_map ? gridFor(map_elems / 4 + 1, 2048) : 0;
-    const int pack_blocks = gridFor(frags, 512);
-    lc.begin("fillMapPackFilter");
-    fillMapPackFilter<E><<<fill_blocks + pack_blocks, 256, 0, lc.stream>>>(
-        ws.map, map_elems + 4 /* and the word that counts ignored pairs */, fill_blocks,
-        static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K,
-        d.Q, d.C, static_cast<S *>(ws.packed));
-    lc.end();
-    if (own_map) launchScatterRowMap(lc, p, d, ws, inl, max_count);
-    const MapSource map = {entries, ws.filled};
-    if (useDenseKernel(lc, p, d)) {
-      n_filled = denseGridX(d.R);
-      launchDense<E, MapSource>(lc, d.Q, d.C, gathered, ws.packed, map, d.R, p.K, result);
+  // A map of the library's own covers a chunk of result rows at a time: filled, used by the
+  // gather kernel for those rows, checked for lost pairs, and filled again for the next rows.
+  int chunk_rows = own_map ? ws.map_rows : d.R;
+  if (own_map && lc.choices.small_map_chunks == 1 && chunk_rows > kRepairPoolRows) chunk_rows = kRepairPoolRows;
+  const bool dense = use_mfma && useDenseKernel(lc, p, d);
+  const int tile_cols = use_mfma && !dense ? mfmaTileCols(p, d) : d.C;
+  for (int row_base = 0; row_base < d.R; row_base += chunk_rows) {
+    const int rows = d.R - row_base < chunk_rows ? d.R - row_base : chunk_rows;
+    const size_t map_elems = (size_t)p.K * rows;
+    const int32_t *entries = own_map ? ws.map : p.row_map;
+    S *result_rows = static_cast<S *>(result) + (size_t)row_base * d.C;
+    int n_filled = 0;    // workgroups along x of the gather kernel = slot counts it leaves
+    int n_accepted = 0;  // workgroups of the map scatter = counts of pairs it leaves
+    if (use_mfma) {
+      // the filter is repacked with the first chunk's map fill
+      const size_t frags = (size_t)p.K * (d.C / 16) * ((d.Q + E::kChunk - 1) / E::kChunk) * 64;
+      const int fill_blocks = own_map ? gridFor(map_elems / 4 + 1, 2048) : 0;
+      const int pack_blocks = row_base == 0 ? gridFor(frags, 512) : 0;
+      if (fill_blocks + pack_blocks > 0) {
+        lc.begin("fillMapPackFilter");
+        fillMapPackFilter<E><<<fill_blocks + pack_blocks, 256, 0, lc.stream>>>(
+            ws.map, map_elems, fill_blocks, static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K,
+            d.Q, d.C, static_cast<S *>(ws.packed));
+        lc.end();
+      }
+      if (own_map) n_accepted = launchScatterRowMap(lc, p, d, ws, inl, max_count, row_base, rows);
+      const MapSource map = {entries, ws.filled};
+      if (dense) {
+        n_filled = denseGridX(rows);
+        launchDense<E, MapSource>(lc, d.Q, d.C, gathered, ws.packed, map, rows, p.K, result_rows);
+      } else {
+        n_filled = mfmaGridX(rows, tile_cols);
+        launchMfma<E, MapSource>(lc, d.Q, d.C, tile_cols, gathered, ws.packed, map, rows, p.K, result_rows);
+      }
     } else {
-      const int tile_cols = mfmaTileCols(p, d);
-      n_filled = mfmaGridX(d.R, tile_cols);
-      launchMfma<E, MapSource>(lc, d.Q, d.C, tile_cols, gathered, ws.packed, map, d.R, p.K, result);
-    }
-  } else {
-    if (own_map) {
-      lc.begin("fillInt32");
-      fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems + 4, -1);
+      if (own_map) {
+        lc.begin("fillInt32");
+        fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems, -1);
+        lc.end();
+        n_accepted = launchScatterRowMap(lc, p, d, ws, inl, max_count, row_base, rows);
+      }
+      dim3 grid((rows + 31) / 32, (d.C + 63) / 64);
+      n_filled = (int)grid.x;
+      lc.begin("gatherConvSimt");
+      gatherConvSimt<E><<<grid, 256, 0, lc.stream>>>(static_cast<const S *>(gathered), d.Q,
+                                                  static_cast<const S *>(f.base), f.stride_k, sQ, sC,
+                                                  entries, rows, p.K, inl, ws.dev_counts, d.C,
+                                                  ws.filled, result_rows);
       lc.end();
-      launchScatterRowMap(lc, p, d, ws, inl, max_count);
     }
-    dim3 grid((d.R + 31) / 32, (d.C + 63) / 64);
-    n_filled = (int)grid.x;
-    lc.begin("gatherConvSimt");
-    gatherConvSimt<E><<<grid, 256, 0, lc.stream>>>(static_cast<const S *>(gathered), d.Q,
-                                                static_cast<const S *>(f.base), f.stride_k, sQ, sC,
-                                                entries, d.R, p.K, inl, ws.dev_counts, d.C,
-                                                ws.filled, static_cast<S *>(result));
+    if (p.distinct_pairs || !own_map) continue;  // a map built ahead was checked when it was built
+    // returns at once unless pairs of one offset share a result row
+    lc.begin("repairLostPairs");
+    repairLostPairs<E><<<repairBlocks(rows), 256, 0, lc.stream>>>(
+        static_cast<const S *>(gathered), d.Q, static_cast<const S *>(f.base), f.stride_k, sQ, sC,
+        p.indice_pairs, p.L, d.row_col, d.src_col, rows, d.n_src, p.K, row_base, inl, ws.dev_counts,
+        ws.map, ws.filled, n_filled, ws.accepted, n_accepted, d.C,
+        RepairScratch{ws.shadow, ws.pool_row, ws.pool}, result_rows);
     lc.end();
   }
-  if (p.distinct_pairs || !own_map) return;  // a map built ahead was checked when it was built
-  // returns at once unless pairs of one offset share a result row
-  long long expected = 0;
-  for (int k = 0; k < p.K; ++k) {
-    const int64_t n = p.indice_num[k];
-    expected += n < 0 ? 0 : (n > p.L ? p.L : n);
-  }
-  lc.begin("repairLostPairs");
-  repairLostPairs<E><<<repairBlocks(d.R), 256, 0, lc.stream>>>(
-      static_cast<const S *>(gathered), d.Q, static_cast<const S *>(f.base), f.stride_k, sQ, sC,
-      p.indice_pairs, p.L, d.row_col, d.src_col, d.R, d.n_src, p.K, inl, ws.dev_counts, ws.map,
-      ws.filled, n_filled, (int)expected, ws.map + map_elems, d.C,
-      RepairScratch{ws.shadow, ws.pool_row, ws.pool},
-      static_cast<S *>(result));
-  lc.end();
 }
 
 struct FilterGradWorkspace {
@@ -2611,8 +2657,7 @@ hipError_t buildRowMap(const LaunchCtx &lc, const int32_t *indice_pairs, const i
     lc.begin("scatterRowMap");
     enqueueScatterRowMap(lc, indice_pairs, shape.L, shape.K, inl,
                          shape.K > kMaxInlineK ? dev_counts : nullptr, max_count, shape.row_column,
-                         1 - shape.row_column, shape.rows, shape.source_rows, map,
-                         counter + 1);  // nobody reads this count: the block behind `counter` is spare
+                         1 - shape.row_column, 0, shape.rows, shape.source_rows, map, nullptr);
     lc.end();
   }
   if (filled_host == nullptr) return hipGetLastError();

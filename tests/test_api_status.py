@@ -747,9 +747,30 @@ def test_row_map_entry_points(handle):
 def test_kernel_choice_setter_checks_its_arguments(handle):
     ok, bad = STATUS["MLUOP_STATUS_SUCCESS"], STATUS["MLUOP_STATUS_BAD_PARAM"]
     f = m.lib().mluOpExtSetKernelChoice
-    for which in range(5):
+    for which in range(6):
         for value in (-1, 0, 1, -1):
             assert f(handle.ptr, which, value) == ok
     assert f(None, 0, 1) == bad
-    assert f(handle.ptr, 5, 1) == bad and f(handle.ptr, -1, 1) == bad
+    assert f(handle.ptr, 6, 1) == bad and f(handle.ptr, -1, 1) == bad
     assert f(handle.ptr, 0, 2) == bad and f(handle.ptr, 0, -2) == bad
+
+
+def test_gather_workspaces_do_not_grow_with_offsets_times_rows(handle):
+    """The row map of forward and backward data covers a chunk of result rows at a time (64 MiB at
+    most), so the workspace of a 5x5x5 filter over 400 000 or 1 000 000 rows stays far below the
+    K x rows x 4 bytes (200 MB, 500 MB) a whole map would take."""
+    lib = m.lib()
+    for rows, bound in ((400000, 128 << 20), (1000000, 160 << 20)):
+        K, c = 125, 128
+        descs = [_d([rows, c]), _d([5, 5, 5, c, c]), _d([K, 2, rows], "MLUOP_DTYPE_INT32"), _d([rows, c])]
+        try:
+            size = ctypes.c_size_t(0)
+            num = [rows] * K
+            assert lib.mluOpGetIndiceConvolutionForwardWorkspaceSize(
+                handle.ptr, descs[0], descs[1], descs[2], descs[3], i64(num), rows, 0, 1, ctypes.byref(size)) == 0
+            assert 0 < size.value < bound < K * rows * 4, size.value
+            assert lib.mluOpGetIndiceConvolutionBackwardDataWorkspaceSize(
+                handle.ptr, descs[0], descs[1], descs[2], descs[3], i64(num), 0, ctypes.byref(size)) == 0
+            assert 0 < size.value < bound, size.value
+        finally:
+            free_descs(*descs)

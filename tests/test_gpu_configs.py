@@ -159,6 +159,33 @@ def test_config5a_subm_5x5x5_rulebook_and_forward(gpu_handle, config5_voxels):
         grade_sample(dw_np[k], ref_k, "float16", "config5a backward filter, offset %d" % k)
 
 
+def test_config5a_rows_out_of_order_take_the_row_map_in_chunks(gpu_handle, config5_voxels):
+    """The same 400 000 voxels in shuffled row order: forward cannot read the pair lists by result
+    row and builds row maps, 64 MiB (131 072 rows of 125 offsets) at a time: four chunks."""
+    import torch
+    import mluop_hip
+    rng = np.random.default_rng(55)
+    idx = np.ascontiguousarray(config5_voxels[rng.permutation(config5_voxels.shape[0])])
+    space, ks, pad = (64, 1024, 1024), (5, 5, 5), [2, 2, 2]
+    pairs, out_idx, num, n_out, ospace = gpu_rulebook(gpu_handle, idx, 1, space, ks, pad, [1, 1, 1], [1, 1, 1],
+                                                      True)
+    num_host = num.cpu().tolist()
+    feats = round_to(rng.standard_normal((idx.shape[0], 128)).astype(np.float32), "float16")
+    w = round_to(mluop_hip.datagen.kaiming_uniform_filters(ks, 128, 128, seed=5), "float16")
+    gpu_handle.set_kernel_timing(True)
+    try:
+        out = mluop_hip.indice_conv_forward(gpu_handle, to_torch(feats, "float16", "cuda"),
+                                            to_torch(w, "float16", "cuda"), mluop_hip.LAYOUT_ARRAY, pairs, num_host,
+                                            n_out, True)
+        names = [n for n, _ in gpu_handle.kernel_timings()]
+    finally:
+        gpu_handle.set_kernel_timing(False)
+    assert names.count("scatterRowMap") == 4 and names.count("repairLostPairs") == 4, names
+    rows = np.sort(rng.choice(n_out, size=3000, replace=False))
+    ref = sampled_rows_reference(feats, w.reshape(125, 128, 128), pairs.cpu().numpy(), num_host, rows)
+    grade_sample(from_torch(out[torch.from_numpy(rows).cuda()]), ref, "float16", "config5a, shuffled rows")
+
+
 def test_config5b_regular_2x2x2_stride2_on_5a_outputs(gpu_handle, config5_voxels):
     """Config 5b: regular 2x2x2 stride 2 pad 0 over the rows 5a leaves (a submanifold layer keeps
     its input coordinates), out 1x32x512x512, Ci=Co=128, fp16 and fp32."""
