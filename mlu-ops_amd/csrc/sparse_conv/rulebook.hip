@@ -557,11 +557,41 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
       const uint32_t sb = hashCell(c0 + (uint32_t)(16 - r)) & mask;
       const bool load_a = want_a != 0 && sa + kWindow <= mask + 1u;
       const bool load_b = want_b != 0 && sb + kWindow <= mask + 1u;
-      KeyWindow win_a, win_b;
+      // A window is looked at once for all KW cells: where[d] becomes the place of the key
+      // c0 + d (0..7 in window A, 8..15 in window B, -1 if it is in neither), empty_x gets
+      // bit i set when slot i of the window is empty.  A cell whose key is in a window is a
+      // hit wherever it sits (keys are unique in the table, and a key lies at or behind its
+      // home slot); a cell without one is a miss for sure when its window has an empty slot
+      // at or behind the cell's home slot, and goes on slot by slot behind the window
+      // otherwise.
+      int where[KW];
 #pragma unroll
-      for (int i = 0; i < kWindow; ++i) win_a.k[i] = win_b.k[i] = kEmptyKey;
+      for (int d = 0; d < KW; ++d) where[d] = -1;
+      uint32_t empty_a = 0, empty_b = 0;
+      KeyWindow win_a;
+#pragma unroll
+      for (int i = 0; i < kWindow; ++i) win_a.k[i] = kEmptyKey;
       if (load_a) win_a = *reinterpret_cast<const KeyWindow *>(keys + sa);
-      if (load_b) win_b = *reinterpret_cast<const KeyWindow *>(keys + sb);
+      if (__any(load_b)) {  // few waves have a lane whose cells cross a run boundary
+        KeyWindow win_b;
+#pragma unroll
+        for (int i = 0; i < kWindow; ++i) win_b.k[i] = kEmptyKey;
+        if (load_b) win_b = *reinterpret_cast<const KeyWindow *>(keys + sb);
+#pragma unroll
+        for (int i = 0; i < kWindow; ++i) {
+          const uint32_t rel = win_b.k[i] - c0;
+          if (win_b.k[i] == kEmptyKey) empty_b |= 1u << i;
+#pragma unroll
+          for (int d = 0; d < KW; ++d) where[d] = rel == (uint32_t)d ? kWindow + i : where[d];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < kWindow; ++i) {
+        const uint32_t rel = win_a.k[i] - c0;
+        if (win_a.k[i] == kEmptyKey) empty_a |= 1u << i;
+#pragma unroll
+        for (int d = 0; d < KW; ++d) where[d] = rel == (uint32_t)d ? i : where[d];
+      }
 #pragma unroll
       for (int d = 0; d < KW; ++d) {
         const int u = KW * a + (KW - 1 - d);
@@ -571,25 +601,11 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
         if (!loaded) {  // window would leave the table: slot by slot from the home slot
           slot[u] = hashCell(cell[u]) & mask;
           pending |= 1u << u;
-          continue;
-        }
-        // walk the window from the cell's home slot
-        const uint32_t base = beyond ? sb : sa;
-        const int first = beyond ? r + d - 16 : d;
-        bool open = true;
-#pragma unroll
-        for (int i = 0; i < kWindow; ++i) {
-          const uint32_t key = beyond ? win_b.k[i] : win_a.k[i];
-          if (open && i >= first && key == cell[u]) {
-            hit |= 1u << u;
-            slot[u] = base + (uint32_t)i;
-            open = false;
-          } else if (open && i >= first && key == kEmptyKey) {
-            open = false;
-          }
-        }
-        if (open) {
-          slot[u] = (base + (uint32_t)kWindow) & mask;
+        } else if (where[d] >= 0) {
+          hit |= 1u << u;
+          slot[u] = (where[d] >= kWindow ? sb : sa) + (uint32_t)(where[d] & (kWindow - 1));
+        } else if (((beyond ? empty_b : empty_a) >> (beyond ? r + d - 16 : d)) == 0) {
+          slot[u] = ((beyond ? sb : sa) + (uint32_t)kWindow) & mask;
           pending |= 1u << u;
         }
       }
