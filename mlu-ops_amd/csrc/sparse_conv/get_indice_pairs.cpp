@@ -7,6 +7,7 @@
 #include <string>
 
 #include "core/core.h"
+#include "core/gen_case.h"
 #include "sparse_conv/rulebook.h"
 #include "sparse_conv/rulebook_notes.h"
 
@@ -199,6 +200,26 @@ mluOpStatus_t MLUOP_WIN_API mluOpGetIndicePairs(
     MLUOP_LOG(ERROR) << api << " workspace of " << workspace_size << " bytes is smaller than the "
                      << need << " bytes mluOpGetIndicePairsWorkspaceSize reports.";
     return MLUOP_STATUS_BAD_PARAM;
+  }
+  if (mluop::gen_case::mode() != 0) {
+    // (reference get_indice_pairs.cpp:47-75)
+    mluop::gen_case::CaseWriter c(handle, "get_indice_pairs", "get_indice_pairs_param");
+    c.input("indices", indices_desc, indices);
+    c.output("out_indices", out_indices_desc);
+    c.output("indice_pairs", indice_pairs_desc);
+    c.output("indice_num", indice_num_desc);
+    c.param("dimnb", sparse_conv_desc->dimNb);
+    c.param("batch", sparse_conv_desc->batch);
+    c.params("pad", sparse_conv_desc->pad, 3);
+    c.params("stride", sparse_conv_desc->stride, 3);
+    c.params("dilation", sparse_conv_desc->dilation, 3);
+    c.params("input_space", sparse_conv_desc->input_space, 3);
+    c.params("filter_space", sparse_conv_desc->filter_space, 3);
+    c.params("output_space", sparse_conv_desc->output_space, 3);
+    c.param("sub_m", sparse_conv_desc->sub_m);
+    c.param("transpose", sparse_conv_desc->transpose);
+    c.param("inverse", sparse_conv_desc->inverse);
+    c.finish(0.0);
   }
   DEVICE_HANDLE_CHECK(api, handle);
 

@@ -6,6 +6,7 @@
 #include <string>
 
 #include "core/core.h"
+#include "core/gen_case.h"
 #include "sparse_conv/indice_conv.h"
 #include "sparse_conv/row_map.h"
 #include "sparse_conv/rulebook_notes.h"
@@ -309,6 +310,19 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardData(
                      << " bytes is smaller than the " << need
                      << " bytes mluOpGetIndiceConvolutionBackwardDataWorkspaceSize reports.";
     return MLUOP_STATUS_BAD_PARAM;
+  }
+  if (mluop::gen_case::mode() != 0) {
+    // (reference indice_convolution_backward_data.cpp:316-332)
+    mluop::gen_case::CaseWriter c(handle, "indice_convolution_backward_data",
+                                  "indice_convolution_backward_data_param");
+    c.input("output_grad", output_grad_desc, output_grad);
+    c.input("filters", filters_desc, filters);
+    c.input("indice_pairs", indice_pairs_desc, indice_pairs);
+    c.output("input_grad", input_grad_desc);
+    c.params("indice_num", indice_num, p.K);
+    c.param("sub_m", sub_m);
+    c.param("inverse", inverse);
+    c.finish(0.003);
   }
   DEVICE_HANDLE_CHECK(api, handle);
   const FilterView f = filterView(filters_desc, filters, p);

@@ -9,6 +9,7 @@
 #include <string>
 
 #include "core/core.h"
+#include "core/gen_case.h"
 #include "mlu_op_ext.h"
 #include "sparse_conv/indice_conv.h"
 #include "sparse_conv/no_alloc_scratch.h"
@@ -276,6 +277,19 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardFilter(
                      << " bytes is smaller than the " << need
                      << " bytes mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize reports.";
     return MLUOP_STATUS_BAD_PARAM;
+  }
+  if (mluop::gen_case::mode() != 0) {
+    // (reference indice_convolution_backward_filter.cpp:82-97)
+    mluop::gen_case::CaseWriter c(handle, "indice_convolution_backward_filter",
+                                  "indice_convolution_backward_param");
+    c.input("features", features_desc, features);
+    c.input("output_grad", output_grad_desc, output_grad);
+    c.input("indice_pairs", indice_pairs_desc, indice_pairs);
+    c.output("filters_grad", filters_grad_desc);
+    c.params("indice_num", indice_num, p.K);
+    c.param("sub_m", subm);
+    c.param("inverse", inverse);
+    c.finish(0.003);
   }
   DEVICE_HANDLE_CHECK(api, handle);
   HIP_CHECK_RETURN(api, mluop::sparse_conv::launchBackwardFilter(handle->launchCtx(), p, features,

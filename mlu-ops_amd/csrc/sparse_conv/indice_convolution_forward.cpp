@@ -5,6 +5,7 @@
 #include <string>
 
 #include "core/core.h"
+#include "core/gen_case.h"
 #include "sparse_conv/indice_conv.h"
 #include "sparse_conv/row_map.h"
 #include "sparse_conv/rulebook_notes.h"
@@ -251,6 +252,19 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionForward(
                      << " bytes is smaller than the " << need
                      << " bytes mluOpGetIndiceConvolutionForwardWorkspaceSize reports.";
     return MLUOP_STATUS_BAD_PARAM;
+  }
+  if (mluop::gen_case::mode() != 0) {
+    // (reference indice_convolution_forward.cpp:657-675; tensor ids as the test runner's executor reads them)
+    mluop::gen_case::CaseWriter c(handle, "indice_convolution_forward", "indice_convolution_forward_param");
+    c.input("features", features_desc, features);
+    c.input("filters", filters_desc, filters);
+    c.input("indice_pairs", indice_pairs_desc, indice_pairs);
+    c.output("features_out", features_out_desc);
+    c.params("indice_num", indice_num, p.K);
+    c.param("num_active_out", num_act_out);
+    c.param("sub_m", sub_m);
+    c.param("inverse", inverse);
+    c.finish(0.003);
   }
   DEVICE_HANDLE_CHECK(api, handle);
   const FilterView f = forwardFilterView(filters_desc, filters, p);

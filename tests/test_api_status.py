@@ -1,7 +1,8 @@
 """Status-code behaviour of the C ABI, checked without a GPU.
 
-The library is loaded with MLUOP_HOST_ONLY_HANDLE=1, which lets mluOpCreate succeed on a machine
-with no HIP device; every parameter check and zero-element early return runs before any kernel
+Handles are created with MLUOP_HOST_ONLY_HANDLE=1 in the environment (for the moment of the
+call only: GPU tests collected into the same process need real handles), which gives a handle
+without a device on any machine; every parameter check and zero-element early return runs before any kernel
 would be launched, so the reference's api_gtest expectations can be replayed here:
 
 * tests/golden/api_status_tables.json -- the value-parameterised tables of
@@ -19,7 +20,6 @@ import re
 
 import pytest
 
-os.environ.setdefault("MLUOP_HOST_ONLY_HANDLE", "1")
 os.environ.setdefault("MLUOP_LOG_PRINT", "0")
 
 import mluop_hip as m  # noqa: E402
@@ -42,9 +42,22 @@ DTYPE = {"MLUOP_DTYPE_INVALID": 0, "MLUOP_DTYPE_HALF": 1, "MLUOP_DTYPE_FLOAT": 2
 FAKE = ctypes.c_void_p(0x1000)  # a non-NULL "device pointer"; never dereferenced on these paths
 
 
+def host_only_handle():
+    """A handle that never launches anything: the made-up pointers below must not reach a kernel."""
+    old = os.environ.get("MLUOP_HOST_ONLY_HANDLE")
+    os.environ["MLUOP_HOST_ONLY_HANDLE"] = "1"
+    try:
+        return m.Handle()
+    finally:
+        if old is None:
+            del os.environ["MLUOP_HOST_ONLY_HANDLE"]
+        else:
+            os.environ["MLUOP_HOST_ONLY_HANDLE"] = old
+
+
 @pytest.fixture(scope="module")
 def handle():
-    h = m.Handle()
+    h = host_only_handle()
     yield h
     h.close()
 
@@ -483,7 +496,7 @@ def test_large_inputs_are_not_supported(handle):
 def test_handle_queue_and_modes():
     lib = m.lib()
     assert lib.mluOpCreate(None) == STATUS["MLUOP_STATUS_BAD_PARAM"]
-    h = m.Handle()
+    h = host_only_handle()
     q = ctypes.c_void_p(123)
     assert lib.mluOpGetQueue(h.ptr, ctypes.byref(q)) == 0 and q.value is None  # starts on the NULL stream
     assert lib.mluOpSetQueue(h.ptr, ctypes.c_void_p(0x40)) == 0
