@@ -2222,12 +2222,14 @@ bool denseShapeOk(ElemType t, int Q, int C) {
 bool useDenseKernel(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d) {
   if (!denseShapeOk(p.dtype, d.Q, d.C)) return false;
   if (lc.choices.dense_tiles >= 0) return lc.choices.dense_tiles == 1;
-  // measured: 128 result columns gain (128 -> 128 at 0.73 pairs per slot: 250 us against
-  // 305 us), 64 result columns tie with the pair-list kernel
-  if (d.C != 128) return false;
+  // Measured on scene-like voxels (filled sheets and walls), 3x3x3: at 64 result columns the
+  // kernel wins from a quarter of the slots filled (0.24: 78 us against 82 us, 0.35: 79
+  // against 93, 0.42: 108 against 156), at 128 columns from a third (0.29: 60.5 us against
+  // 55.5 us, 0.35: a tie, 0.42: 272 against 317).
   double pairs = 0;
   for (int k = 0; k < p.K; ++k) pairs += (double)p.indice_num[k];
-  return pairs >= 0.25 * (double)d.R * p.K;
+  const double fill = pairs / ((double)d.R * p.K);
+  return d.C == 64 ? fill >= 0.25 : fill >= 0.33;
 }
 
 template <typename E, int Q, int C, typename SRC>
