@@ -42,6 +42,22 @@ typedef unsigned short u16;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
+
+// A workgroup barrier for LDS traffic only: what the wave wrote to or read from LDS is done,
+// loads from global memory stay in flight across it (__syncthreads() would wait for them).
+__device__ __forceinline__ void ldsBarrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// 16 bytes per lane from global memory straight into LDS: lane l of the wave writes bytes
+// [16 l, 16 l + 16) behind `lds_address` (the same in all lanes).  Written as the instruction
+// itself: the compiler then does not know of an LDS write in flight, and does not hold every
+// later LDS read of the wave back until all loads have returned; the caller waits (vmcnt)
+// before anybody reads what was requested.
+__device__ __forceinline__ void requestToLds(const void *global, uint32_t lds_address) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :: "s"(lds_address), "v"(global) : "memory", "m0");
+}
 constexpr int kMaxInlineK = 128;
 
 // Pair counts per offset, passed by value for the common small kernel volumes.
@@ -1100,54 +1116,53 @@ __global__ __launch_bounds__(64) void gatherConvWave(
 // When most rows of a tile have a partner at most offsets, compacting pairs buys
 // little and the fp32 accumulate in LDS (a 16-byte read-modify-write per lane and
 // 16 result columns, on arbitrary rows: bank conflicts) is what the kernel above
-// spends its time on.  Here a tile is 64 result rows = four groups of 16, the
-// partner rows of one offset are staged at their result-row position, and a wave
-// accumulates 32 result columns of two row groups in registers over all offsets:
-// no accumulator traffic at all.  A lane whose row has no partner at the
-// offset multiplies zeros; a row group none of whose rows has one is skipped.
-//
-// The partner rows travel from global memory straight into LDS (16-byte
-// `global_load_lds`: lane l of a wave-load writes bytes [16 l, 16 l + 16) of a
-// 1 KiB block, no registers involved), requested kDenseDepth - 1 offsets ahead by
-// the multiplying waves themselves: there are no fetching waves and one barrier
-// per offset.  Because those blocks are unpadded, a row's 16-byte pieces are
-// stored permuted (piece ^ f(row)) so that the 16 rows an operand read touches
-// fall into 16 different bank groups.
-constexpr int kDenseTileRows = 64;
-constexpr int kDenseChunk = 32;  // offsets whose row-map slice is resident in LDS at once
-constexpr int kDenseDepth = 4;   // stage buffers: offsets i .. i+3 are resident or in flight
-constexpr int kDenseRowSplit = 2;  // waves along the rows of a tile
-constexpr int denseThreads(int C) { return 64 * (C / 32) * kDenseRowSplit; }
+// spends its time on.  Here a wave owns G groups of 16 result rows and all result
+// columns, and accumulates them in registers over all offsets: no accumulator traffic
+// at all.  The partner rows of an offset come from global memory straight into the
+// operand registers of the lane that multiplies them (lane (row, quarter) loads 16
+// bytes of its row per reduction chunk, one offset ahead), so no wave waits for
+// another one's rows.  What the waves of a workgroup share is the offset's filter: its
+// fragments travel from global memory into one of two LDS buffers (16 bytes per lane
+// straight into LDS, one offset ahead, every wave a share of them) and every wave reads
+// all of them from there, once per offset for all its row groups.  One barrier per
+// offset hands the buffers over; it waits for LDS traffic only, and each wave waits for
+// its own loads itself (__syncthreads() would make every wave wait for all loads in
+// flight, the requests for the offset after included).  A lane whose row has no
+// partner at the offset reads a row of zeros; a row group none of whose rows has one
+// is skipped, and a wave without any skips the offset.
+__device__ __attribute__((aligned(256))) unsigned char kZeroRow[512];  // never written
+constexpr int kDenseChunk = 27;      // offsets whose row-map slice is resident in LDS at once
+constexpr int kDenseMapBatch = 14;   // loads in flight per thread while a tile's row map is read
+constexpr int kDenseWaves = 4;
+// row groups per wave: as many as leave room for two sets of partner rows in the registers
+constexpr int denseGroups(int Q, int C) { return (C >= 128 || Q >= 128) ? 2 : 4; }
+constexpr int denseTileRows(int Q, int C) { return kDenseWaves * denseGroups(Q, C) * 16; }
 
 template <typename E, int Q, int C, typename SRC>
-__global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
+__global__ __launch_bounds__(64 * kDenseWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void gatherConvDense(
     const typename E::storage *A, const typename E::storage *packedW, SRC source, int R,
     int K, int ldc, typename E::storage *result) {
   typedef typename E::vec8 vec8;
   typedef typename E::storage S;
-  constexpr int NB = 2;                      // 16-column blocks per wave
-  constexpr int CW = C / 32;                 // waves along the columns
-  constexpr int RS = kDenseRowSplit;         // waves along the rows
-  constexpr int WAVES = CW * RS;
-  constexpr int GPW = kDenseTileRows / 16 / RS;  // row groups per wave
-  constexpr int TR = kDenseTileRows;
+  constexpr int WAVES = kDenseWaves;
+  constexpr int G = denseGroups(Q, C);
+  constexpr int TR = denseTileRows(Q, C);
+  constexpr int NB = C / 16;                 // 16-column blocks, all of them in every wave
   constexpr int KC = kDenseChunk;
-  constexpr int D = kDenseDepth;
   constexpr int KB = Q / E::kChunk;
   constexpr int ROW_BYTES = Q * (int)sizeof(S);
-  constexpr int PPR = ROW_BYTES / 16;        // 16-byte pieces per row
-  constexpr int RP256 = 256 / ROW_BYTES;     // rows per 256 bytes (one pass over all banks)
-  constexpr int LOADS = TR * PPR / 64;       // wave-loads per offset
-  constexpr int LPW = LOADS / WAVES;         // every wave issues at least this many of them
-  constexpr int LPW_MAX = (LOADS + WAVES - 1) / WAVES;
-  static_assert(Q % E::kChunk == 0 && C % 32 == 0, "whole fragments and column pairs");
-  static_assert(ROW_BYTES <= 256 && 256 % ROW_BYTES == 0, "rows of 32 to 256 bytes");
-  static_assert((D - 2) * (LPW + KB * NB) <= 63, "fits the load counter");
+  constexpr int FRAGS = NB * KB;             // 1 KiB filter fragments per offset
+  constexpr int W_BYTES = FRAGS * 1024;
+  constexpr int FPW = (FRAGS + WAVES - 1) / WAVES;
+  constexpr int POOL = 2 * W_BYTES;
+  static_assert(Q % E::kChunk == 0 && C % 16 == 0, "whole fragments");
+  static_assert(G >= 1 && G <= 4, "one code path per set of row groups");
 
-  __shared__ __attribute__((aligned(1024))) char s_stage[D][TR * ROW_BYTES];
+  __shared__ __attribute__((aligned(1024))) char s_w[POOL];
   __shared__ int s_map[KC][TR];   // partner row of (offset in chunk, tile row) or -1
   __shared__ int s_list[KC];      // offsets of the chunk that have a pair in this tile
   __shared__ int s_has[KC];
+  __shared__ int s_first[KC];
   __shared__ int s_count;
 
   const int tid = threadIdx.x;
@@ -1165,11 +1180,11 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
   const int col_group = blockIdx.y;
   if constexpr (SRC::kSegments) {
     if (*source.verdict == source.ticket) {
-      // pair lists out of order: fp32 rows in the stage memory, as many columns at a
-      // time as fit, every pair looked at by every workgroup
-      float *acc = reinterpret_cast<float *>(&s_stage[0][0]);
-      constexpr int CP = D * ROW_BYTES / 4 >= C ? C : 64;  // columns per pass
-      static_assert(D * ROW_BYTES / 4 >= 64, "a pass of 64 columns fits the stage");
+      // pair lists out of order: fp32 rows where the row map would be, 16 columns at a
+      // time, every pair looked at by every workgroup
+      float *acc = reinterpret_cast<float *>(&s_map[0][0]);
+      constexpr int CP = 16;  // columns per pass
+      static_assert(CP <= KC && C % CP == 0, "a pass of columns fits the row map");
       const int r_end = r0 + TR < R ? r0 + TR : R;
       for (int c0 = 0; c0 < C; c0 += CP) {
         for (int i = tid; i < TR * CP; i += WAVES * 64) acc[i] = 0.f;
@@ -1186,49 +1201,85 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
   }
   const int pair = lane & 15;
   const int quad = lane >> 4;
-  const char *a_bytes = reinterpret_cast<const char *>(A);
-  const int cw = wave % CW;                  // this wave's column pair
-  const int g0 = (wave / CW) * GPW;          // and its first row group
-  const char *b_base = reinterpret_cast<const char *>(packedW) +
-                       ((size_t)(col_group * (C / 16) + cw * NB) * KB * 64 + lane) * 16;
-  const uint32_t kBytesPerOffset = (uint32_t)(ldc / 16) * KB * 64 * 16;
+  const char *a_lane = reinterpret_cast<const char *>(A) + quad * 16;
+  const char *zero_lane = reinterpret_cast<const char *>(kZeroRow) + quad * 16;
+  const char *w_base = reinterpret_cast<const char *>(packedW) +
+                       (size_t)col_group * FRAGS * 1024 + lane * 16;
+  const size_t kBytesPerOffset = (size_t)(ldc / 16) * KB * 1024;
+  const uint32_t w_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)s_w;
+  const int row_first = wave * (G * 16) + pair;  // this lane's row in its wave's first group
 
-  float4v acc[GPW][NB];
+  float4v acc[G][NB];
 #pragma unroll
-  for (int g = 0; g < GPW; ++g)
+  for (int g = 0; g < G; ++g)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[g][nb] = float4v{0.f, 0.f, 0.f, 0.f};
-  int slots = 0;  // filled map slots this wave staged
+  int slots = 0;  // filled map slots this thread staged
+  constexpr int NT = WAVES * 64;
 
   for (int kc = 0; kc < K; kc += KC) {
     const int kn = (K - kc) < KC ? (K - kc) : KC;
-    __syncthreads();  // the chunk before is finished with s_map and the stage
-    for (int kk = wave; kk < kn; kk += WAVES) {
-      if constexpr (SRC::kSegments) {
-        // the offset's pairs of this tile are one piece of its list: lane l of the
-        // piece writes its partner at the result row's position (same wave, in order
-        // behind the clearing store)
-        s_map[kk][lane] = -1;
-        int cut = 0;
-        if (lane < 2) cut = source.cuts[(size_t)(kc + kk) * source.cut_stride + tile + lane];
-        const int first = __shfl(cut, 0, kWave);
-        int count = __shfl(cut, 1, kWave) - first;
+    __syncthreads();  // the chunk before is finished with s_map and the filter buffers
+    if constexpr (SRC::kSegments) {
+      // The pairs of an offset that fall into this tile are one piece of its list, between
+      // two neighbouring entries of the cut table.
+      if (tid < kn) {
+        const int32_t *cut = source.cuts + (size_t)(kc + tid) * source.cut_stride + tile;
+        const int first = cut[0];
+        int count = cut[1] - first;
         count = count < 0 ? 0 : (count > TR ? TR : count);
-        if (lane < count) {
-          int p = first + lane;
-          p = p < 0 ? 0 : (p < source.L ? p : source.L - 1);
-          const int32_t *list = source.pairs + (size_t)(kc + kk) * 2 * source.L;
-          const int own = (list[(size_t)source.row_col * source.L + p] - r0) & (TR - 1);
-          s_map[kk][own] = list[(size_t)source.src_col * source.L + p];
+        s_first[tid] = first;
+        s_has[tid] = count;
+      }
+      for (int i = tid; i < kn * TR; i += NT) (&s_map[0][0])[i] = -1;
+      __syncthreads();
+      // a thread per (offset, pair of the piece): the partner goes to the result row's
+      // position.  A thread's loads of one batch are all requested before the first is
+      // used (a slot without a pair reads pair 0 of its offset and drops it).
+      if (source.L > 0) {
+        for (int base = tid; base < kn * TR; base += NT * kDenseMapBatch) {
+          int own[kDenseMapBatch], partner[kDenseMapBatch], at[kDenseMapBatch];
+#pragma unroll
+          for (int u = 0; u < kDenseMapBatch; ++u) {
+            const int slot = base + u * NT;
+            int kk = slot / TR;
+            const int q = slot % TR;
+            kk = kk < kn ? kk : kn - 1;
+            const bool live = slot < kn * TR && q < s_has[kk];
+            int p = live ? s_first[kk] + q : 0;
+            p = p < 0 ? 0 : (p < source.L ? p : source.L - 1);
+            const int32_t *list = source.pairs + (size_t)(kc + kk) * 2 * source.L;
+            own[u] = list[(size_t)source.row_col * source.L + p];
+            partner[u] = list[(size_t)source.src_col * source.L + p];
+            at[u] = live ? kk : -1;
+          }
+#pragma unroll
+          for (int u = 0; u < kDenseMapBatch; ++u)
+            if (at[u] >= 0) s_map[at[u]][(own[u] - r0) & (TR - 1)] = partner[u];
         }
-        if (lane == 0) s_has[kk] = count > 0;
-      } else {
-        const int r = r0 + lane;
-        const int v = r < R ? source.map[(size_t)(kc + kk) * R + r] : -1;
-        s_map[kk][lane] = v;
-        const unsigned long long any = __ballot(v >= 0);
-        if (lane == 0) s_has[kk] = any != 0ull;
-        slots += __popcll(any);
+      }
+    } else {
+      if (tid < kn) s_has[tid] = 0;
+      __syncthreads();
+      for (int base = tid; base < kn * TR; base += NT * kDenseMapBatch) {
+        int v[kDenseMapBatch];
+#pragma unroll
+        for (int u = 0; u < kDenseMapBatch; ++u) {
+          const int slot = base + u * NT;
+          int kk = slot / TR;
+          kk = kk < kn ? kk : kn - 1;
+          const int r = r0 + slot % TR;
+          v[u] = source.map[(size_t)(kc + kk) * R + (r < R ? r : R - 1)];
+          if (slot >= kn * TR || r >= R) v[u] = -1;
+        }
+#pragma unroll
+        for (int u = 0; u < kDenseMapBatch; ++u) {
+          const int slot = base + u * NT;  // (a wave stays inside one offset)
+          if (slot < kn * TR) s_map[slot / TR][slot % TR] = v[u];
+          const unsigned long long m = __ballot(v[u] >= 0);
+          if (m != 0ull && lane == 0) s_has[slot / TR] = 1;
+          slots += v[u] >= 0;
+        }
       }
     }
     __syncthreads();
@@ -1242,91 +1293,111 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
     const int items = s_count;
     if (items == 0) continue;
 
-    // Requests the rows of one offset into its stage buffer.  Position p (in 16-byte
-    // units) of the buffer holds piece (p % PPR) ^ f(row) of row p / PPR; a row
-    // without a partner fetches row 0, which nobody reads.
-    auto request = [&](int item) {
+    // The partner rows of one offset, into the registers of the lanes that multiply them
+    // (a lane without a partner reads zeros); returns which of the wave's row groups have
+    // a partner at all.
+    auto load_rows = [&](int item, vec8 (&rows)[G][KB]) -> int {
       const int kk = s_list[item];
-      char *buf = s_stage[item & (D - 1)];
+      int present = 0;
 #pragma unroll
-      for (int t = 0; t < LPW_MAX; ++t) {
-        const int wl = wave + t * WAVES;
-        if (wl >= LOADS) break;
-        const int p = wl * 64 + lane;
-        const int row = p / PPR;
-        const int piece = (p % PPR) ^ ((row / RP256) & (PPR - 1));
-        const int src = s_map[kk][row];
-        const char *g = a_bytes + (size_t)(src < 0 ? 0 : src) * ROW_BYTES + piece * 16;
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void *)g,
-            (__attribute__((address_space(3))) void *)(buf + wl * 1024), 16, 0, 0);
+      for (int g = 0; g < G; ++g) {
+        const int src = s_map[kk][row_first + g * 16];
+        const bool mine = src >= 0;
+        const char *row = mine ? a_lane + (size_t)src * ROW_BYTES : zero_lane;
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+          rows[g][kb] = *reinterpret_cast<const vec8 *>(row + kb * 64);
+        if (__ballot(mine) != 0ull) present |= 1 << g;
+      }
+      return present;
+    };
+    // The filter fragments of one offset into a buffer: fragment f by wave f % WAVES.
+    auto request_filter = [&](int item, int buffer) {
+      const char *wk = w_base + (size_t)(kc + s_list[item]) * kBytesPerOffset;
+      const uint32_t buf = w_lds + buffer * W_BYTES;
+#pragma unroll
+      for (int t = 0; t < FPW; ++t) {
+        const int f = wave + t * WAVES;
+        if (FRAGS % WAVES != 0 && f >= FRAGS) break;
+        requestToLds(wk + f * 1024, buf + f * 1024);
       }
     };
-    vec8 wnext[KB][NB];
-    auto fetch_w = [&](int item) {
-      const char *bk = b_base + (size_t)(kc + s_list[item]) * kBytesPerOffset;
+    // acc[g] += rows[g] x filter for the two row groups from G0 on that MASK names
+    auto multiply = [&](auto g0_tag, auto mask_tag, const vec8 (&rows)[G][KB], const char *wbuf) {
+      constexpr int G0 = decltype(g0_tag)::value;
+      constexpr int MASK = decltype(mask_tag)::value;
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-          wnext[kb][nb] = *reinterpret_cast<const vec8 *>(bk + (nb * KB + kb) * 1024);
-    };
-#pragma unroll
-    for (int j = 0; j < D - 1; ++j)
-      if (j < items) request(j);
-    fetch_w(0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();  // item 0 (and whatever else has arrived) is staged
-
-    for (int i = 0; i < items; ++i) {
-      vec8 wcur[KB][NB];
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) wcur[kb][nb] = wnext[kb][nb];
-      if (i + 1 < items) fetch_w(i + 1);
-      // buffer (i + D - 1) % D held item i - 1, which every wave left at the last barrier
-      const bool more = i + D - 1 < items;
-      if (more) request(i + D - 1);
-
-      const int kk = s_list[i];
-      const char *stage = s_stage[i & (D - 1)];
-#pragma unroll
-      for (int g = 0; g < GPW; ++g) {
-        const int row = (g0 + g) * 16 + pair;
-        const bool mine = s_map[kk][row] >= 0;
-        if (__ballot(mine) == 0ull) continue;  // no row of the group has a partner here
-        const char *arow = stage + row * ROW_BYTES;
-        const int swz = (row / RP256) & (PPR - 1);
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-          vec8 afr = *reinterpret_cast<const vec8 *>(arow + (((kb * 4 + quad) ^ swz) * 16));
-          if (!mine) afr = vec8{};
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) acc[g][nb] = E::mfma(wcur[kb][nb], afr, acc[g][nb]);
+        for (int nb = 0; nb < NB; ++nb) {
+          const vec8 wf = *reinterpret_cast<const vec8 *>(wbuf + (nb * KB + kb) * 1024 + lane * 16);
+          if (MASK & 1) acc[G0][nb] = E::mfma(wf, rows[G0][kb], acc[G0][nb]);
+          if (MASK & 2) acc[G0 + 1][nb] = E::mfma(wf, rows[G0 + 1][kb], acc[G0 + 1][nb]);
         }
+    };
+    auto multiply_present = [&](int present, const vec8 (&rows)[G][KB], const char *wbuf) {
+      typedef std::integral_constant<int, 1> one;
+      typedef std::integral_constant<int, 2> two;
+      typedef std::integral_constant<int, 3> both;
+      {
+        typedef std::integral_constant<int, 0> first;
+        const int bits = present & 3;
+        if (bits == 3) multiply(first(), both(), rows, wbuf);
+        else if (bits == 1) multiply(first(), one(), rows, wbuf);
+        else if (bits == 2) multiply(first(), two(), rows, wbuf);
       }
-      // Item i + 1 must have landed before anybody reads it.  Loads complete in order, and
-      // the last D - 2 iterations (this one included) each issued at least LPW row requests
-      // and KB * NB filter fragments, all of them after the requests of item i + 1 (nothing
-      // moves across the barrier below), so that many loads may stay in flight.  Waiting for
-      // fewer would also wait for the filter fragments of item i + 1, requested a moment ago.
-      // Near the end of the list nothing newer is in flight and everything is awaited.
-      if (more)
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((D - 2) * (LPW + KB * NB)) : "memory");
-      else
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
+      if constexpr (G == 4) {
+        typedef std::integral_constant<int, 2> first;
+        const int bits = (present >> 2) & 3;
+        if (bits == 3) multiply(first(), both(), rows, wbuf);
+        else if (bits == 1) multiply(first(), one(), rows, wbuf);
+        else if (bits == 2) multiply(first(), two(), rows, wbuf);
+      }
+    };
+    // Waits for everything this wave has requested.  The rows pass through an empty
+    // statement that the compiler must take for their last writer: it then places its own
+    // wait for their loads here, where it costs nothing, and not in front of their first
+    // use, behind the requests for the offset after, which it would wait for as well.
+    auto landed = [&](vec8 (&rows)[G][KB]) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) asm volatile("" : "+v"(rows[g][kb]));
+    };
+    // Offset `item` with the rows in `cur`, while the rows and the filter of the next one
+    // travel.  Everything requested here has landed when the barrier is passed, and every
+    // wave has left the buffer that the offset after the next will be written to.
+    auto phase = [&](int item, int present, const vec8 (&cur)[G][KB], vec8 (&nxt)[G][KB]) -> int {
+      int present_next = 0;
+      if (item + 1 < items) {
+        present_next = load_rows(item + 1, nxt);
+        request_filter(item + 1, (item + 1) & 1);
+      }
+      multiply_present(present, cur, s_w + (item & 1) * W_BYTES);
+      landed(nxt);
+      ldsBarrier();
+      return present_next;
+    };
+
+    vec8 rows_a[G][KB], rows_b[G][KB];
+    int present = load_rows(0, rows_a);
+    request_filter(0, 0);
+    landed(rows_a);
+    ldsBarrier();
+    for (int i = 0; i < items; i += 2) {
+      present = phase(i, present, rows_a, rows_b);
+      if (i + 1 < items) present = phase(i + 1, present, rows_b, rows_a);
     }
   }
-  // lane holds result columns 16*nb + 4*quad + (0..3) of row 16*g + pair
+  // lane holds result columns 16*nb + 4*quad + (0..3) of row 16*g + pair of its wave's rows
 #pragma unroll
-  for (int g = 0; g < GPW; ++g) {
-    const int r = r0 + (g0 + g) * 16 + pair;
+  for (int g = 0; g < G; ++g) {
+    const int r = r0 + row_first + g * 16;
     if (r >= R) continue;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-      S *dst = result + (size_t)r * ldc + col_group * C + cw * 32 + nb * 16 + quad * 4;
+      S *dst = result + (size_t)r * ldc + col_group * C + nb * 16 + quad * 4;
       S tmp[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) E::store(&tmp[e], acc[g][nb][e]);
@@ -1339,7 +1410,10 @@ __global__ __launch_bounds__(denseThreads(C)) void gatherConvDense(
   if constexpr (!SRC::kSegments) {
     // s_has is free again: the waves' slot counts meet there
     __syncthreads();
-    if (lane == 0) s_has[wave] = slots;
+    int wave_slots = slots;
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) wave_slots += __shfl_xor(wave_slots, d, kWave);
+    if (lane == 0) s_has[wave] = wave_slots;
     __syncthreads();
     if (tid == 0 && blockIdx.y == 0) {
       int all = 0;
@@ -2132,7 +2206,10 @@ int mfmaGridX(int R, int tile_cols) {
   const int tr = mfmaTileRows(tile_cols);
   return ((R + tr - 1) / tr + 7) / 8 * 8;
 }
-int denseGridX(int R) { return ((R + kDenseTileRows - 1) / kDenseTileRows + 7) / 8 * 8; }
+int denseGridX(int R, int Q, int C) {
+  const int rows = denseTileRows(Q, C);
+  return ((R + rows - 1) / rows + 7) / 8 * 8;
+}
 
 template <typename E, int Q, int C, typename SRC>
 void launchMfmaInstance(const LaunchCtx &lc, const void *A, const void *packed,
@@ -2222,22 +2299,40 @@ bool denseShapeOk(ElemType t, int Q, int C) {
 bool useDenseKernel(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d) {
   if (!denseShapeOk(p.dtype, d.Q, d.C)) return false;
   if (lc.choices.dense_tiles >= 0) return lc.choices.dense_tiles == 1;
-  // Measured on scene-like voxels (filled sheets and walls), 3x3x3: at 64 result columns the
-  // kernel wins from a quarter of the slots filled (0.24: 78 us against 82 us, 0.35: 79
-  // against 93, 0.42: 108 against 156), at 128 columns from a third (0.29: 60.5 us against
-  // 55.5 us, 0.35: a tie, 0.42: 272 against 317).
-  double pairs = 0;
-  for (int k = 0; k < p.K; ++k) pairs += (double)p.indice_num[k];
+  // What the kernel costs goes with the (tile, offset) pieces that hold a pair at all, what
+  // the pair-list kernel costs with the pairs.  On voxels strewn uniformly every piece holds
+  // a few, and the kernel wins from 0.25 of all (row, offset) slots filled at 128 result
+  // columns (175 us against 183 us, 150000 rows, 3x3x3) and 0.4 at 64 columns (0.27: 86
+  // against 77, 0.51: 104 against 119).  On scenes (filled sheets and walls) the pairs of an
+  // offset sit in few pieces, and it wins at 128 columns from 0.05 (88 against 98) and at 64
+  // columns from 0.15 (67 against 73; 0.35: 75 against 93).  The host only knows the pair
+  // counts: sheets and walls show there as offsets with far more pairs than the average
+  // offset (in-plane neighbours), which uniform voxels never have.
+  double pairs = 0, largest = 0, second = 0;
+  for (int k = 0; k < p.K; ++k) {
+    const double n = (double)p.indice_num[k];
+    pairs += n;
+    if (n > largest) {
+      second = largest;
+      largest = n;
+    } else if (n > second) {
+      second = n;
+    }
+  }
   const double fill = pairs / ((double)d.R * p.K);
-  return d.C == 64 ? fill >= 0.25 : fill >= 0.33;
+  // (the largest count is the centre offset of a submanifold convolution: left out)
+  const double mean_rest = p.K > 1 ? (pairs - largest) / (p.K - 1) : 0.0;
+  const bool sheets = mean_rest > 0 && second >= 1.5 * mean_rest;
+  if (d.C == 64) return fill >= (sheets ? 0.15 : 0.38);
+  return fill >= (sheets ? 0.04 : 0.25);
 }
 
 template <typename E, int Q, int C, typename SRC>
 void launchDenseInstance(const LaunchCtx &lc, const void *A, const void *packed, const SRC &source,
                          int R, int K, void *result) {
-  const dim3 grid(denseGridX(R), 1);
+  const dim3 grid(denseGridX(R, Q, C), 1);
   lc.begin("gatherConvDense");
-  gatherConvDense<E, Q, C, SRC><<<grid, denseThreads(C), 0, lc.stream>>>(
+  gatherConvDense<E, Q, C, SRC><<<grid, 64 * kDenseWaves, 0, lc.stream>>>(
       static_cast<const typename E::storage *>(A), static_cast<const typename E::storage *>(packed),
       source, R, K, C, static_cast<typename E::storage *>(result));
   lc.end();
@@ -2327,7 +2422,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
     // gather kernel reads them cut by tile, no row map.
     const bool dense = useDenseKernel(lc, p, d);
     const int tile_cols = dense ? d.C : mfmaTileCols(p, d);
-    const int tile_rows = dense ? kDenseTileRows : mfmaTileRows(tile_cols);
+    const int tile_rows = dense ? denseTileRows(d.Q, d.C) : mfmaTileRows(tile_cols);
     int tile_shift = 0;
     while ((1 << tile_shift) < tile_rows) ++tile_shift;
     const int n_tiles = (d.R + tile_rows - 1) / tile_rows;
@@ -2397,7 +2492,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
       if (own_map) n_accepted = launchScatterRowMap(lc, p, d, ws, inl, max_count, row_base, rows);
       const MapSource map = {entries, ws.filled};
       if (dense) {
-        n_filled = denseGridX(rows);
+        n_filled = denseGridX(rows, d.Q, d.C);
         launchDense<E, MapSource>(lc, d.Q, d.C, gathered, ws.packed, map, rows, p.K, result_rows);
       } else {
         n_filled = mfmaGridX(rows, tile_cols);

@@ -82,8 +82,15 @@ def test_map_kernels_and_collision_check_are_not_launched(gpu_handle):
         gpu_handle.set_kernel_timing(False)
         return names
 
-    assert kernels(None) == ["fillMapPackFilter", "scatterRowMap", "gatherConvMfma", "repairLostPairs"]
-    assert kernels(rm) == ["fillMapPackFilter", "gatherConvMfma"]     # the first one only packs the filter here
+    # (four cells in five are occupied: left to itself the library takes the kernel for dense rulebooks)
+    gpu_handle.set_kernel_choice("dense_tiles", False)
+    try:
+        assert kernels(None) == ["fillMapPackFilter", "scatterRowMap", "gatherConvMfma", "repairLostPairs"]
+        assert kernels(rm) == ["fillMapPackFilter", "gatherConvMfma"]     # the first one only packs the filter here
+    finally:
+        gpu_handle.set_kernel_choice("dense_tiles", None)
+    assert kernels(None) == ["fillMapPackFilter", "scatterRowMap", "gatherConvDense", "repairLostPairs"]
+    assert kernels(rm) == ["fillMapPackFilter", "gatherConvDense"]
     rm.close()
 
 
