@@ -1149,13 +1149,16 @@ __global__ __launch_bounds__(64 * kDenseWaves) __attribute__((amdgpu_waves_per_e
   constexpr int TR = denseTileRows(Q, C);
   constexpr int NB = C / 16;                 // 16-column blocks, all of them in every wave
   constexpr int KC = kDenseChunk;
-  constexpr int KB = Q / E::kChunk;
+  constexpr int KB = (Q + E::kChunk - 1) / E::kChunk;
+  // 16 channels of a 2-byte type: half a fragment, the lanes of the other half read zeros
+  constexpr bool kHalfFragment = Q % E::kChunk != 0;
   constexpr int ROW_BYTES = Q * (int)sizeof(S);
   constexpr int FRAGS = NB * KB;             // 1 KiB filter fragments per offset
   constexpr int W_BYTES = FRAGS * 1024;
   constexpr int FPW = (FRAGS + WAVES - 1) / WAVES;
   constexpr int POOL = 2 * W_BYTES;
-  static_assert(Q % E::kChunk == 0 && C % 16 == 0, "whole fragments");
+  static_assert((Q % E::kChunk == 0 || (KB == 1 && Q % E::kVec == 0)) && C % 16 == 0,
+                "whole fragments, or part of a single one");
   static_assert(G >= 1 && G <= 4, "one code path per set of row groups");
 
   __shared__ __attribute__((aligned(1024))) char s_w[POOL];
@@ -1303,7 +1306,8 @@ __global__ __launch_bounds__(64 * kDenseWaves) __attribute__((amdgpu_waves_per_e
       for (int g = 0; g < G; ++g) {
         const int src = s_map[kk][row_first + g * 16];
         const bool mine = src >= 0;
-        const char *row = mine ? a_lane + (size_t)src * ROW_BYTES : zero_lane;
+        const bool read = mine && (!kHalfFragment || quad * E::kVec < Q);
+        const char *row = read ? a_lane + (size_t)src * ROW_BYTES : zero_lane;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
           rows[g][kb] = *reinterpret_cast<const vec8 *>(row + kb * 64);
@@ -2286,28 +2290,28 @@ bool useWaveKernel(const LaunchCtx &lc, ElemType t, int Q, int C) {
   return waveKernelShape((int)elemSize(t), Q, C);
 }
 
-// The register-accumulating kernel pays when a quarter or more of all (row, offset)
-// slots hold a pair (below that, most of its multiplies are zeros); it takes 64
-// or 128 result columns and reduction channels of whole fragments.
+// The register-accumulating kernel takes 16 to 128 result columns and 16 to 128 reduction
+// channels (16 channels of a 2-byte type as half a fragment).
 bool denseShapeOk(ElemType t, int Q, int C) {
-  const int chunk = t == ElemType::kFloat ? 16 : 32;
-  // fp32 rows of 128 channels leave no room for the double-buffered stage and the fragments
+  // fp32 rows of 128 channels leave no room for two sets of partner rows and the fragments
   if (t == ElemType::kFloat && Q > 64) return false;
-  return (C == 64 || C == 128) && Q % chunk == 0 && (Q == 16 || Q == 32 || Q == 64 || Q == 128);
+  return (C == 16 || C == 32 || C == 64 || C == 128) && (Q == 16 || Q == 32 || Q == 64 || Q == 128);
 }
 
 bool useDenseKernel(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d) {
   if (!denseShapeOk(p.dtype, d.Q, d.C)) return false;
   if (lc.choices.dense_tiles >= 0) return lc.choices.dense_tiles == 1;
   // What the kernel costs goes with the (tile, offset) pieces that hold a pair at all, what
-  // the pair-list kernel costs with the pairs.  On voxels strewn uniformly every piece holds
-  // a few, and the kernel wins from 0.25 of all (row, offset) slots filled at 128 result
-  // columns (175 us against 183 us, 150000 rows, 3x3x3) and 0.4 at 64 columns (0.27: 86
-  // against 77, 0.51: 104 against 119).  On scenes (filled sheets and walls) the pairs of an
-  // offset sit in few pieces, and it wins at 128 columns from 0.05 (88 against 98) and at 64
-  // columns from 0.15 (67 against 73; 0.35: 75 against 93).  The host only knows the pair
-  // counts: sheets and walls show there as offsets with far more pairs than the average
-  // offset (in-plane neighbours), which uniform voxels never have.
+  // the pair-list kernels cost with the pairs.  Measured on 150000 rows, 3x3x3, fp16, as the
+  // share of all (row, offset) slots that hold a pair from which the kernel wins:
+  //   result columns   voxels strewn uniformly   scenes (filled sheets and walls)
+  //   16, 32           0.4  (0.27: 53 us against 45 us, 0.51: 57 against 67)   0.07 (38 against 49)
+  //   64               0.38 (0.27: 86 against 77, 0.51: 104 against 119)      0.15 (67 against 73)
+  //   128              0.25 (175 against 183)                                  0.04 (88 against 98)
+  // On strewn voxels every piece holds a few pairs; in a scene the pairs of an offset sit in
+  // few pieces.  The host only knows the pair counts: sheets and walls show there as offsets
+  // with far more pairs than the average offset (in-plane neighbours), which strewn voxels
+  // never have.
   double pairs = 0, largest = 0, second = 0;
   for (int k = 0; k < p.K; ++k) {
     const double n = (double)p.indice_num[k];
@@ -2323,6 +2327,7 @@ bool useDenseKernel(const LaunchCtx &lc, const ConvProblem &p, const GatherDims 
   // (the largest count is the centre offset of a submanifold convolution: left out)
   const double mean_rest = p.K > 1 ? (pairs - largest) / (p.K - 1) : 0.0;
   const bool sheets = mean_rest > 0 && second >= 1.5 * mean_rest;
+  if (d.C <= 32) return fill >= (sheets ? 0.07 : 0.4);
   if (d.C == 64) return fill >= (sheets ? 0.15 : 0.38);
   return fill >= (sheets ? 0.04 : 0.25);
 }
@@ -2342,29 +2347,21 @@ template <typename E, typename SRC>
 void launchDense(const LaunchCtx &lc, int Q, int C, const void *A, const void *packed,
                  const SRC &source, int R, int K, void *result) {
   constexpr bool is_float = std::is_same<E, FloatElem>::value;
-#define DENSE_CASE(q)                                                                           \
-  case q:                                                                                       \
-    if (C == 64) launchDenseInstance<E, q, 64, SRC>(lc, A, packed, source, R, K, result);       \
-    else launchDenseInstance<E, q, 128, SRC>(lc, A, packed, source, R, K, result);              \
-    break;
+#define DENSE_BY_C(q)                                                                           \
+  if (C == 16) launchDenseInstance<E, q, 16, SRC>(lc, A, packed, source, R, K, result);         \
+  else if (C == 32) launchDenseInstance<E, q, 32, SRC>(lc, A, packed, source, R, K, result);    \
+  else if (C == 64) launchDenseInstance<E, q, 64, SRC>(lc, A, packed, source, R, K, result);    \
+  else launchDenseInstance<E, q, 128, SRC>(lc, A, packed, source, R, K, result);
   switch (Q) {
-    case 16:
-      if constexpr (is_float) {
-        if (C == 64) launchDenseInstance<E, 16, 64, SRC>(lc, A, packed, source, R, K, result);
-        else launchDenseInstance<E, 16, 128, SRC>(lc, A, packed, source, R, K, result);
-      }
-      break;
-    DENSE_CASE(32)
-    DENSE_CASE(64)
+    case 16: DENSE_BY_C(16) break;
+    case 32: DENSE_BY_C(32) break;
+    case 64: DENSE_BY_C(64) break;
     case 128:
-      if constexpr (!is_float) {
-        if (C == 64) launchDenseInstance<E, 128, 64, SRC>(lc, A, packed, source, R, K, result);
-        else launchDenseInstance<E, 128, 128, SRC>(lc, A, packed, source, R, K, result);
-      }
+      if constexpr (!is_float) { DENSE_BY_C(128) }
       break;
     default: break;
   }
-#undef DENSE_CASE
+#undef DENSE_BY_C
 }
 
 // Row maps are built on the flat grid from this many workgroups of the per-offset grid on.

@@ -109,7 +109,12 @@ def test_simt_path_matches_oracle_on_mfma_shapes(gpu_handle, dtype_name):
 
 
 DENSE_SHAPES = [
-    # the register-accumulating kernel takes 64 or 128 result columns; (8, 8, 8) with 300 voxels is dense
+    # the register-accumulating kernel takes 16 to 128 result columns; (8, 8, 8) with 300 voxels is dense
+    (1, (8, 8, 8), 300, (3, 3, 3), 16, 16, True, (1, 1, 1)),      # half a reduction fragment in fp16
+    (2, (8, 8, 8), 500, (3, 3, 3), 16, 32, True, (1, 1, 1)),
+    (1, (8, 8, 8), 300, (3, 3, 3), 32, 16, False, (1, 1, 1)),
+    (1, (10, 10, 10), 700, (3, 3, 3), 32, 32, True, (1, 1, 1)),   # 700 rows: three tiles of 256
+    (1, (9, 9, 9), 500, (3, 3, 3), 16, 128, False, (2, 2, 2)),
     (1, (8, 8, 8), 300, (3, 3, 3), 64, 64, True, (1, 1, 1)),
     (1, (8, 8, 8), 300, (3, 3, 3), 128, 128, True, (1, 1, 1)),
     (2, (8, 8, 8), 500, (3, 3, 3), 32, 128, True, (1, 1, 1)),
