@@ -31,8 +31,11 @@ typedef enum {
   MLUOP_EXT_KERNEL_WAVE_PER_TILE = 2,  /* one-wavefront-per-tile gather kernel */
   MLUOP_EXT_KERNEL_FLAT_SLICE_SUM = 3, /* backward filter: partial tiles summed on a flat grid */
   MLUOP_EXT_KERNEL_FLAT_SCATTER = 4,   /* row maps built on a flat grid */
-  MLUOP_EXT_KERNEL_SMALL_MAP_CHUNKS = 5 /* 1: row maps cover 2048 result rows at a time instead of
-                                           as many as 64 MiB hold (runs the chunked path on small inputs) */
+  MLUOP_EXT_KERNEL_SMALL_MAP_CHUNKS = 5, /* 1: row maps cover 2048 result rows at a time instead of
+                                            as many as 64 MiB hold (runs the chunked path on small inputs) */
+  MLUOP_EXT_KERNEL_FILTER_STORES = 6    /* 1: backward filter transposes its operands with element-sized
+                                           LDS stores also for 2-byte types of 32 to 128 channels, where
+                                           transposing LDS reads are the default */
 } mluOpExtKernelChoice_t;
 
 mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelChoice(mluOpHandle_t handle,

@@ -176,6 +176,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelChoice(mluOpHandle_t handle,
     case MLUOP_EXT_KERNEL_FLAT_SLICE_SUM: c.flat_slice_sum = value; break;
     case MLUOP_EXT_KERNEL_FLAT_SCATTER: c.flat_scatter = value; break;
     case MLUOP_EXT_KERNEL_SMALL_MAP_CHUNKS: c.small_map_chunks = value; break;
+    case MLUOP_EXT_KERNEL_FILTER_STORES: c.filter_stores = value; break;
     default:
       MLUOP_LOG(ERROR) << "[mluOpExtSetKernelChoice] unknown kernel choice " << as_int;
       return MLUOP_STATUS_BAD_PARAM;

@@ -56,6 +56,7 @@ struct KernelChoices {
   int flat_slice_sum = -1;  // backward filter: partial tiles summed on the flat grid
   int flat_scatter = -1;    // 1: row maps built on the flat grid
   int small_map_chunks = -1;  // 1: row maps cover 2048 result rows at a time (the chunked path, on small inputs)
+  int filter_stores = -1;   // 1: backward filter transposes with element-sized LDS stores also where transposing reads serve
 };
 
 class LaunchCtx {

@@ -1728,6 +1728,46 @@ constexpr int kFilterStepPairs = 64;     // pairs multiplied per barrier
 constexpr int kFilterIndexChunk = 1024;  // pair indices resident in LDS at once
 constexpr int kFilterMaxSlices = 768;    // about three workgroups per CU
 
+// The order in which the workgroups take the slices: by the share of its offset's list that
+// lies in front of a slice, so that the workgroups running at one time are at about the same
+// rows of the feature and gradient tensors in all offsets (the lists ascend by row), and a
+// row fetched for one offset is still in the L2 cache when the others want it.  Entry j names
+// the offset of the j-th slice in that order; it is that offset's s-th slice when s earlier
+// entries name the same offset.  Workgroup b takes entry (b % 8) * (grid / 8) + b / 8:
+// neighbouring entries on one XCD, behind one L2.
+struct SliceOrder {
+  uint8_t offset[kFilterMaxSlices + kMaxInlineK];
+};
+
+struct SlicePlace {
+  int k, slice;
+};
+
+// For all threads of a workgroup (one barrier inside).  k < 0: no slice for this workgroup.
+__device__ __forceinline__ SlicePlace sliceOfWorkgroup(const SliceOrder &order, int total) {
+  __shared__ int s_place[2];
+  const int per_xcd = gridDim.x >> 3;
+  const int j = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  if (threadIdx.x < 64) {
+    int k = -1, earlier = 0;
+    if (j < total) {
+      k = order.offset[j];
+      for (int i = threadIdx.x; i < j; i += 64) earlier += order.offset[i] == k;
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) earlier += __shfl_xor(earlier, d, kWave);
+    if (threadIdx.x == 0) {
+      s_place[0] = k;
+      s_place[1] = earlier;
+    }
+  }
+  __syncthreads();
+  SlicePlace at;
+  at.k = s_place[0];
+  at.slice = s_place[1];
+  return at;
+}
+
 // Both operands are needed with the pair index running along the MFMA's K
 // dimension, i.e. transposed relative to the row-major tensors: rows are
 // gathered with 16-byte loads and written to LDS transposed ([channel][pair],
@@ -1741,7 +1781,8 @@ constexpr int kFilterMaxSlices = 768;    // about three workgroups per CU
 template <typename E, int CI, int CO>
 __global__ __launch_bounds__(256) void backwardFilterMfma(
     const typename E::storage *X, const typename E::storage *dY, const int32_t *pairs, int L,
-    int x_col, int n_in, int n_out, int K, SliceTable tab, int slice_len, float *partial) {
+    int x_col, int n_in, int n_out, int K, SliceTable tab, SliceOrder order, int total_slices,
+    int slice_len, float *partial) {
   typedef typename E::vec8 vec8;
   typedef typename E::storage S;
   constexpr int SP = kFilterStepPairs;
@@ -1764,11 +1805,11 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
   __shared__ int s_in[kFilterIndexChunk];
   __shared__ int s_out[kFilterIndexChunk];
 
-  // blockIdx.x numbers the slices of all offsets; offset = last one starting at or before it
-  int k = K - 1;
-  while (k > 0 && tab.first[k] > (int)blockIdx.x) --k;
+  const SlicePlace at = sliceOfWorkgroup(order, total_slices);
+  if (at.k < 0) return;
+  const int k = at.k;
   const int n = tab.n[k];
-  const int p_begin = ((int)blockIdx.x - tab.first[k]) * slice_len;
+  const int p_begin = at.slice * slice_len;
   if (p_begin >= n) return;
   const int p_end = p_begin + slice_len < n ? p_begin + slice_len : n;
   const int tid = threadIdx.x;
@@ -1883,7 +1924,7 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
     }
   }
   // lane holds rows 4*(lane/16)+v, column lane%16 of every 16 x 16 block
-  float *tile = partial + (size_t)blockIdx.x * CI * CO;
+  float *tile = partial + (size_t)(tab.first[k] + at.slice) * CI * CO;
 #pragma unroll
   for (int a = 0; a < CBW; ++a) {
     const int cb = wave + a * 4;
@@ -1895,6 +1936,205 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
           tile[(size_t)(cb * 16 + 4 * (lane >> 4) + v) * CO + b * 16 + (lane & 15)] = acc[a][b][v];
     }
   }
+}
+
+// The same product for 2-byte elements and 32 to 128 channels on both sides, with the
+// transposition done by the LDS read itself.  The gathered rows go from global memory
+// straight into LDS as they are ([pair][channel], 16 bytes per lane, a pair without a
+// valid row reads a row of zeros), one step of 64 pairs ahead into the other of two
+// buffers, and `ds_read_b64_tr_b16` hands a lane four consecutive pairs of one channel:
+// within 16 lanes, lane i supplies the address of 4 channels of pair i / 4 and lane j
+// receives channel j of the four pairs.  Two such reads are one operand fragment.  No
+// element-sized stores, no registers for staging, one barrier per step.
+//
+// A row's 16-byte pieces are stored permuted (piece ^ f(pair)), since rows lie a
+// multiple of the bank width apart: f spreads the eight pairs that half a wavefront
+// reads at once over all 64 banks.  Waves are laid out 2 x 2 over the blocks of dW[k].
+constexpr int filterRowSwizzle(int row_bytes, int pair) {
+  return row_bytes == 256 ? (((pair & 1) << 1) | ((pair & 2) << 1) | (pair & 8))
+       : row_bytes == 128 ? ((pair & 2) | ((pair & 8) >> 1))
+       : row_bytes == 64  ? ((pair & 8) >> 2)
+                          : 0;
+}
+
+template <typename E, int CI, int CO>
+__global__ __launch_bounds__(256) void backwardFilterMfmaTr(
+    const typename E::storage *X, const typename E::storage *dY, const int32_t *pairs, int L,
+    int x_col, int n_in, int n_out, int K, SliceTable tab, SliceOrder order, int total_slices,
+    int slice_len, float *partial) {
+  typedef typename E::vec8 vec8;
+  typedef typename E::storage S;
+  typedef short v4i16 __attribute__((ext_vector_type(4)));
+  typedef short v8i16 __attribute__((ext_vector_type(8)));
+  static_assert(sizeof(S) == 2 && E::kChunk == 32, "2-byte elements, 32 pairs per fragment");
+  static_assert(CI % 32 == 0 && CO % 32 == 0 && CI <= 128 && CO <= 128, "two row and column blocks per wave pair");
+  constexpr int SP = kFilterStepPairs;
+  // two chunks of row indices: with 128 channels on both sides the buffers leave 16 KiB of
+  // half a CU's LDS
+  constexpr int kIndexChunk = 512;
+  constexpr int kChunkSteps = kIndexChunk / SP;
+  constexpr int RBX = CI * 2, RBY = CO * 2;     // bytes per row
+  constexpr int XN = SP * RBX / 1024;           // 1 KiB wave-loads per step
+  constexpr int YN = SP * RBY / 1024;
+  constexpr int AB = CI / 32, BB = CO / 32;     // 16-row / 16-column blocks per wave
+  static_assert(SP == 64, "two fragments per step");
+
+  __shared__ __attribute__((aligned(1024))) char s_x[2][SP * RBX];
+  __shared__ __attribute__((aligned(1024))) char s_y[2][SP * RBY];
+  __shared__ int s_in[2][kIndexChunk];   // row indices of a chunk of pairs, and of the chunk after
+  __shared__ int s_out[2][kIndexChunk];
+
+  const SlicePlace at = sliceOfWorkgroup(order, total_slices);
+  if (at.k < 0) return;
+  const int k = at.k;
+  const int n = tab.n[k];
+  const int p_begin = at.slice * slice_len;
+  if (p_begin >= n) return;
+  const int p_end = p_begin + slice_len < n ? p_begin + slice_len : n;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wa = wave >> 1, wb = wave & 1;
+  const int32_t *in_col = pairs + ((size_t)k * 2 + x_col) * L;
+  const int32_t *out_col = pairs + ((size_t)k * 2 + 1 - x_col) * L;
+  const uint32_t x_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)&s_x[0][0];
+  const uint32_t y_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)&s_y[0][0];
+  const char *zero_row = reinterpret_cast<const char *>(kZeroRow);
+
+  float4v acc[AB][BB];
+#pragma unroll
+  for (int a = 0; a < AB; ++a)
+#pragma unroll
+    for (int b = 0; b < BB; ++b) acc[a][b] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  // One step's rows into a buffer: wave-load t of an operand covers 1 KiB of the buffer, lane
+  // l its bytes [16 l, 16 l + 16), i.e. a fixed (pair, place) of the step.  Wave w issues
+  // loads w, w + 4, ...: `locate` reads all row indices first and forms the addresses (one
+  // LDS latency a step, not one a load), `request` issues load u of the wave's XM + YM.
+  constexpr int XM = (XN + 3) / 4, YM = (YN + 3) / 4;
+  struct StepLoads {
+    const char *from[XM + YM];
+  };
+  // (live == false: a step that is not there; every lane then reads the row of zeros, so
+  // that the requests need no branch around them)
+  auto locate = [&](int step, bool live, StepLoads &loads) {
+    const int *in = s_in[(step / kChunkSteps) & 1] + (step % kChunkSteps) * SP;
+    const int *out = s_out[(step / kChunkSteps) & 1] + (step % kChunkSteps) * SP;
+    int row[XM + YM];
+#pragma unroll
+    for (int u = 0; u < XM; ++u) row[u] = in[((wave + u * 4) * 1024 + lane * 16) / RBX];
+#pragma unroll
+    for (int u = 0; u < YM; ++u) row[XM + u] = out[((wave + u * 4) * 1024 + lane * 16) / RBY];
+#pragma unroll
+    for (int u = 0; u < XM + YM; ++u) {
+      const bool is_x = u < XM;
+      const int row_bytes = is_x ? RBX : RBY;
+      const int byte = (wave + (is_x ? u : u - XM) * 4) * 1024 + lane * 16;
+      const int piece = ((byte % row_bytes) / 16) ^ filterRowSwizzle(row_bytes, byte / row_bytes);
+      const char *rows = reinterpret_cast<const char *>(is_x ? (const void *)X : (const void *)dY);
+      loads.from[u] = (live && row[u] >= 0 ? rows + (size_t)row[u] * row_bytes : zero_row) + piece * 16;
+    }
+  };
+  auto request = [&](const StepLoads &loads, int u, int buffer) {
+    if (u < XM) {
+      const int t = wave + u * 4;
+      if (XN % 4 == 0 || t < XN) requestToLds(loads.from[u], x_lds + buffer * (SP * RBX) + t * 1024);
+    } else if (u < XM + YM) {
+      const int t = wave + (u - XM) * 4;
+      if (YN % 4 == 0 || t < YN) requestToLds(loads.from[u], y_lds + buffer * (SP * RBY) + t * 1024);
+    }
+  };
+  // fragment of block `block` (16 channels) for the 32 pairs from `pair0` on: lane (c, kq)
+  // receives pairs pair0 + 8 kq + (0..7) of channel 16 block + c
+  const int sub = lane & 15, kq = lane >> 4;
+  auto fragment = [&](const char *buffer, int row_bytes, int block, int pair0) -> vec8 {
+    const int pair = pair0 + 8 * kq + (sub >> 2);  // the four pairs after it have the same swizzle
+    const int place = (block * 2 + ((sub & 3) >> 1)) ^ filterRowSwizzle(row_bytes, pair);
+    const char *at = buffer + pair * row_bytes + place * 16 + (sub & 1) * 8;
+    const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) v4i16 *)(at));
+    const v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) v4i16 *)(at + 4 * row_bytes));
+    const v8i16 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(vec8, both);
+  };
+
+  // Row indices of chunk c: four pairs a thread, checked; -1 marks a pair that is not there.
+  constexpr int IPT = kIndexChunk / 256;
+  int idx_in[IPT], idx_out[IPT];
+  auto fetch_indices = [&](int chunk) {
+#pragma unroll
+    for (int u = 0; u < IPT; ++u) {
+      const int at = p_begin + chunk * kIndexChunk + u * 256 + tid;
+      int i = -1, o = -1;
+      if (at < p_end) {
+        i = in_col[at];
+        o = out_col[at];
+      }
+      idx_in[u] = i;
+      idx_out[u] = o;
+    }
+  };
+  auto store_indices = [&](int chunk) {
+#pragma unroll
+    for (int u = 0; u < IPT; ++u) {
+      int i = idx_in[u], o = idx_out[u];
+      if ((unsigned)i >= (unsigned)n_in || (unsigned)o >= (unsigned)n_out) i = o = -1;
+      s_in[chunk & 1][u * 256 + tid] = i;
+      s_out[chunk & 1][u * 256 + tid] = o;
+    }
+  };
+
+  const int steps = (p_end - p_begin + SP - 1) / SP;
+  fetch_indices(0);
+  store_indices(0);
+  __syncthreads();
+  StepLoads next_rows;
+  locate(0, true, next_rows);
+#pragma unroll
+  for (int u = 0; u < XM + YM; ++u) request(next_rows, u, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  ldsBarrier();
+  for (int step = 0; step < steps; ++step) {
+    const int cur = step & 1;
+    const int in_chunk = step % kChunkSteps, chunk = step / kChunkSteps;
+    // the chunk after this one: its indices are requested at the chunk's first step and are
+    // in LDS one barrier before the chunk's last step asks for the next chunk's first rows
+    const bool chunk_follows = (chunk + 1) * kChunkSteps < steps;
+    if (in_chunk == 0 && chunk_follows) fetch_indices(chunk + 1);
+    const bool ahead = step + 1 < steps;
+    locate(ahead ? step + 1 : step, ahead, next_rows);
+    const char *bx = s_x[cur], *by = s_y[cur];
+    // (all requests first: they have one step's multiplies to land)
+#pragma unroll
+    for (int u = 0; u < XM + YM; ++u) request(next_rows, u, cur ^ 1);
+#pragma unroll
+    for (int kb = 0; kb < SP / 32; ++kb) {
+      vec8 bfr[BB];
+#pragma unroll
+      for (int b = 0; b < BB; ++b) bfr[b] = fragment(by, RBY, wb * BB + b, kb * 32);
+#pragma unroll
+      for (int a = 0; a < AB; ++a) {
+        const vec8 afr = fragment(bx, RBX, wa * AB + a, kb * 32);
+#pragma unroll
+        for (int b = 0; b < BB; ++b) acc[a][b] = E::mfma(afr, bfr[b], acc[a][b]);
+      }
+    }
+    if (in_chunk == kChunkSteps - 2 && chunk_follows) store_indices(chunk + 1);
+    // the next step's rows have landed, and every wave has left this step's buffers
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    ldsBarrier();
+  }
+  // lane holds rows 4*(lane/16)+v, column lane%16 of every 16 x 16 block
+  float *tile = partial + (size_t)(tab.first[k] + at.slice) * CI * CO;
+#pragma unroll
+  for (int a = 0; a < AB; ++a)
+#pragma unroll
+    for (int b = 0; b < BB; ++b)
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        tile[(size_t)((wa * AB + a) * 16 + 4 * (lane >> 4) + v) * CO + (wb * BB + b) * 16 + (lane & 15)] =
+            acc[a][b][v];
 }
 
 // dW[k] = sum of the offset's partial tiles, rounded once.  A block adds 256
@@ -2577,15 +2817,32 @@ GradLayout gradLayout(const ConvProblem &p) {
 
 template <typename E, int CI, int CO>
 void launchFilterMfmaInstance(const LaunchCtx &lc, const ConvProblem &p, const SliceTable &tab,
-                              int slice_len, int total_slices, float *partial, const void *features,
+                              const SliceOrder &order, int slice_len, int total_slices, float *partial, const void *features,
                               const void *output_grad, void *filters_grad) {
   typedef typename E::storage S;
-  lc.begin("backwardFilterMfma");
-  if (total_slices > 0)
-    backwardFilterMfma<E, CI, CO><<<total_slices, 256, 0, lc.stream>>>(
-        static_cast<const S *>(features), static_cast<const S *>(output_grad), p.indice_pairs,
-        p.L, p.inverse ? 1 : 0, p.inverse ? p.num_out : p.L, p.inverse ? p.L : p.num_out, p.K,
-        tab, slice_len, partial);
+  constexpr bool kTransposingReads = sizeof(S) == 2 && CI >= 32 && CO >= 32;
+  const int grid = (total_slices + 7) / 8 * 8;
+  lc.begin(kTransposingReads && lc.choices.filter_stores != 1 ? "backwardFilterMfmaTr" : "backwardFilterMfma");
+  if (total_slices > 0) {
+    if constexpr (kTransposingReads) {
+      if (lc.choices.filter_stores != 1) {
+        backwardFilterMfmaTr<E, CI, CO><<<grid, 256, 0, lc.stream>>>(
+            static_cast<const S *>(features), static_cast<const S *>(output_grad), p.indice_pairs,
+            p.L, p.inverse ? 1 : 0, p.inverse ? p.num_out : p.L, p.inverse ? p.L : p.num_out, p.K,
+            tab, order, total_slices, slice_len, partial);
+      } else {
+        backwardFilterMfma<E, CI, CO><<<grid, 256, 0, lc.stream>>>(
+            static_cast<const S *>(features), static_cast<const S *>(output_grad), p.indice_pairs,
+            p.L, p.inverse ? 1 : 0, p.inverse ? p.num_out : p.L, p.inverse ? p.L : p.num_out, p.K,
+            tab, order, total_slices, slice_len, partial);
+      }
+    } else {
+      backwardFilterMfma<E, CI, CO><<<grid, 256, 0, lc.stream>>>(
+          static_cast<const S *>(features), static_cast<const S *>(output_grad), p.indice_pairs,
+          p.L, p.inverse ? 1 : 0, p.inverse ? p.num_out : p.L, p.inverse ? p.L : p.num_out, p.K,
+          tab, order, total_slices, slice_len, partial);
+    }
+  }
   lc.end();
   // Many offsets of few slices each: the flat grid, on which such an offset takes a
   // sixteenth of the workgroups (same bits).
@@ -2611,13 +2868,13 @@ void launchFilterMfmaInstance(const LaunchCtx &lc, const ConvProblem &p, const S
 
 template <typename E, int CI>
 void launchFilterMfmaByCo(const LaunchCtx &lc, const ConvProblem &p, const SliceTable &tab,
-                          int slice_len, int total_slices, float *partial, const void *features,
+                          const SliceOrder &order, int slice_len, int total_slices, float *partial, const void *features,
                           const void *output_grad, void *filters_grad) {
   switch (p.Co) {
-    case 16: launchFilterMfmaInstance<E, CI, 16>(lc, p, tab, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
-    case 32: launchFilterMfmaInstance<E, CI, 32>(lc, p, tab, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
-    case 64: launchFilterMfmaInstance<E, CI, 64>(lc, p, tab, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
-    case 128: launchFilterMfmaInstance<E, CI, 128>(lc, p, tab, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
+    case 16: launchFilterMfmaInstance<E, CI, 16>(lc, p, tab, order, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
+    case 32: launchFilterMfmaInstance<E, CI, 32>(lc, p, tab, order, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
+    case 64: launchFilterMfmaInstance<E, CI, 64>(lc, p, tab, order, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
+    case 128: launchFilterMfmaInstance<E, CI, 128>(lc, p, tab, order, slice_len, total_slices, partial, features, output_grad, filters_grad); break;
     default: break;
   }
 }
@@ -2643,11 +2900,27 @@ void launchFilterMfma(const LaunchCtx &lc, const ConvProblem &p, const FilterGra
       tab.first[k] = first;
       first += slices;
     }
+    // slices in the order of the share of their offset's list in front of them, in `steps`
+    // steps of that share (as many as the longest list has slices)
+    SliceOrder order;
+    int steps = 1, next[kMaxInlineK], count[kMaxInlineK];
+    for (int k = 0; k < p.K; ++k) {
+      next[k] = 0;
+      count[k] = (tab.n[k] + slice_len - 1) / slice_len;
+      if (count[k] > steps) steps = count[k];
+    }
+    int placed = 0;
+    for (int t = 0; t < steps; ++t)
+      for (int k = 0; k < p.K; ++k)
+        while (next[k] < count[k] && (long long)next[k] * steps < (long long)(t + 1) * count[k]) {
+          order.offset[placed++] = (uint8_t)k;
+          ++next[k];
+        }
     switch (p.Ci) {
-      case 16: launchFilterMfmaByCo<E, 16>(lc, p, tab, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
-      case 32: launchFilterMfmaByCo<E, 32>(lc, p, tab, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
-      case 64: launchFilterMfmaByCo<E, 64>(lc, p, tab, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
-      case 128: launchFilterMfmaByCo<E, 128>(lc, p, tab, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
+      case 16: launchFilterMfmaByCo<E, 16>(lc, p, tab, order, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
+      case 32: launchFilterMfmaByCo<E, 32>(lc, p, tab, order, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
+      case 64: launchFilterMfmaByCo<E, 64>(lc, p, tab, order, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
+      case 128: launchFilterMfmaByCo<E, 128>(lc, p, tab, order, slice_len, first, ws.partial, features, output_grad, filters_grad); break;
       default: break;
     }
   }

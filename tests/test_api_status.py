@@ -760,11 +760,11 @@ def test_row_map_entry_points(handle):
 def test_kernel_choice_setter_checks_its_arguments(handle):
     ok, bad = STATUS["MLUOP_STATUS_SUCCESS"], STATUS["MLUOP_STATUS_BAD_PARAM"]
     f = m.lib().mluOpExtSetKernelChoice
-    for which in range(6):
+    for which in range(7):
         for value in (-1, 0, 1, -1):
             assert f(handle.ptr, which, value) == ok
     assert f(None, 0, 1) == bad
-    assert f(handle.ptr, 6, 1) == bad and f(handle.ptr, -1, 1) == bad
+    assert f(handle.ptr, 7, 1) == bad and f(handle.ptr, -1, 1) == bad
     assert f(handle.ptr, 0, 2) == bad and f(handle.ptr, 0, -2) == bad
 
 
