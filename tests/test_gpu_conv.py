@@ -139,6 +139,46 @@ def test_dense_kernel_matches_oracle(gpu_handle, shape, dtype_name):
             gpu_handle.set_kernel_choice("dense_tiles", None)
 
 
+@pytest.mark.parametrize("shape", [
+    # (space, L, ks, ci, co, sub_m, stride): slices of several chunks of row indices, ragged ends
+    ((14, 20, 20), 4000, (3, 3, 3), 128, 128, True, (1, 1, 1)),
+    ((14, 20, 20), 3100, (3, 3, 3), 64, 32, True, (1, 1, 1)),
+    ((12, 30, 30), 5000, (3, 3, 3), 32, 128, False, (2, 2, 2)),
+    ((6, 6, 6), 150, (5, 5, 5), 64, 64, True, (1, 1, 1)),      # 125 offsets, short lists
+])
+@pytest.mark.parametrize("dtype_name", ["float16", "bfloat16"])
+def test_backward_filter_kernels_agree(gpu_handle, shape, dtype_name):
+    """2-byte types of 32 to 128 channels: the kernel that reads its operand fragments with the
+    transposing LDS read against the oracle, and bit for bit against the kernel that transposes with
+    element-sized stores (same products, same order of sums)."""
+    import torch
+    import mluop_hip
+    space, L, ks, ci, co, sub_m, stride = shape
+    print("backward filter case", shape, dtype_name, flush=True)
+    c = conv_case(14, 1, space, L, ks, ci, co, sub_m, stride)
+    feats_t = to_torch(round_to(c["feats"], dtype_name), dtype_name, "cuda")
+    dy_t = to_torch(round_to(c["dy"], dtype_name), dtype_name, "cuda")
+    pairs_t = torch.from_numpy(c["pairs"]).cuda()
+    num_host = [int(v) for v in c["num"]]
+    got = {}
+    for stores in (False, True):
+        gpu_handle.set_kernel_choice("filter_stores", True if stores else None)
+        try:
+            gpu_handle.set_kernel_timing(True)
+            dw = mluop_hip.indice_conv_backward_filter(gpu_handle, feats_t, dy_t, pairs_t, num_host, c["ks"], sub_m)
+            torch.cuda.synchronize()
+            names = [k for k, _ in gpu_handle.kernel_timings()]
+            gpu_handle.set_kernel_timing(False)
+        finally:
+            gpu_handle.set_kernel_choice("filter_stores", None)
+        assert names[0] == ("backwardFilterMfma" if stores else "backwardFilterMfmaTr")
+        got[stores] = dw
+    ref = oracle.backward_filter(round_to(c["feats"], dtype_name), round_to(c["dy"], dtype_name), c["pairs"],
+                                 c["num"], fast=True)
+    check_close(from_torch(got[False]).reshape(ref.shape), ref, dtype_name, "backward_filter")
+    assert torch.equal(got[False], got[True])
+
+
 @pytest.mark.parametrize("layout_name", ["NDHWC", "NCDHW", "ARRAY"])
 @pytest.mark.parametrize("dtype_name", ["float32", "float16"])
 def test_forward_filter_layouts(gpu_handle, layout_name, dtype_name):
