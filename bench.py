@@ -382,16 +382,14 @@ def run_backbone(args, torch, m):
         layers.append(spnn.SparseConv3d(c, co, 3, stride=2, padding=1))
         layers += [spnn.SubMConv3d(co, co, 3, indice_key="s%d" % stage) for _ in range(2)]
         c = co
-    net = torch.nn.ModuleList(layers).cuda().half()
+    # (a ReLU behind every layer; the container builds all rulebooks before the first layer runs)
+    net = spnn.SparseSequential(*[m for layer in layers for m in (layer, torch.nn.ReLU())]).cuda().half()
     # MLUOP_BENCH_SHARE_ROW_MAPS=1: layers of a stage share their rulebook's row maps
     spnn.share_row_maps(os.environ.get("MLUOP_BENCH_SHARE_ROW_MAPS", "0") == "1")
 
     def step():
         # the voxels are distinct, as a voxelizer's output is: the layers skip the collision check
-        x = spnn.SparseTensor(feats.clone().requires_grad_(True), indices, grid[1:], grid[0], distinct=True)
-        for layer in net:
-            x = layer(x)
-            x = x.replace_features(torch.relu(x.features))
+        x = net(spnn.SparseTensor(feats.clone().requires_grad_(True), indices, grid[1:], grid[0], distinct=True))
         x.features.float().square().mean().backward()
         return x
 
@@ -406,7 +404,7 @@ def run_backbone(args, torch, m):
     rows = [int(idx.shape[0])]
     x = spnn.SparseTensor(feats, indices, grid[1:], grid[0], distinct=True)
     with torch.no_grad():
-        for layer in net:
+        for layer in layers:
             x = layer(x)
             if not layer.sub_m:
                 rows.append(int(x.features.shape[0]))

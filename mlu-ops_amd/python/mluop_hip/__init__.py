@@ -256,6 +256,22 @@ class TensorDescriptor:
             pass
 
 
+_descriptors = {}
+
+
+def _descriptor(layout, dtype, dims, onchip_dtype=None):
+    """A tensor descriptor for the operator wrappers below, shared by every call of the same
+    (layout, dtype, dims): a layer's calls repeat their shapes, and creating and setting a
+    descriptor through ctypes costs more host time than the operator's own launch code."""
+    key = (layout, dtype, tuple(int(d) for d in dims), onchip_dtype)
+    d = _descriptors.get(key)
+    if d is None:
+        if len(_descriptors) >= 1024:
+            _descriptors.clear()   # (descriptors in use are kept alive by their callers)
+        d = _descriptors[key] = TensorDescriptor(layout, dtype, list(key[2]), onchip_dtype)
+    return d
+
+
 class SparseConvDescriptor:
     def __init__(self, batch, pad, stride, dilation, input_space, filter_space, output_space,
                  sub_m, transpose=0, inverse=0, dim_nb=5):
@@ -424,10 +440,10 @@ def get_indice_pairs(handle, indices, batch, input_space, filter_space, output_s
     indice_num = _output((K,), torch.int32, dev, "indice_num")
     desc = SparseConvDescriptor(batch, pad, stride, dilation, input_space, filter_space,
                                 output_space, sub_m)
-    d_in = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [L, 4])
-    d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
-    d_out = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [out_rows, 4])
-    d_num = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K])
+    d_in = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [L, 4])
+    d_pairs = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+    d_out = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [out_rows, 4])
+    d_num = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [K])
     size = ctypes.c_size_t(0)
     check(lib().mluOpGetIndicePairsWorkspaceSize(handle.ptr, desc.ptr, d_in.ptr, d_pairs.ptr,
                                                  d_out.ptr, d_num.ptr, ctypes.byref(size)),
@@ -457,7 +473,7 @@ class RowMap:
         the wait for the queue that reads it."""
         torch = _torch()
         K, _, L = indice_pairs.shape
-        d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+        d_pairs = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
         size = ctypes.c_size_t(0)
         check(lib().mluOpExtGetRowMapSize(d_pairs.ptr, int(rows), ctypes.byref(size)), "mluOpExtGetRowMapSize")
         self.handle = handle
@@ -501,10 +517,10 @@ def indice_conv_forward(handle, features, filters, filters_layout, indice_pairs,
     else:
         co = filters.shape[0]
     out = _output((num_act_out, co), features.dtype, features.device, "features_out")
-    d_feat = TensorDescriptor(LAYOUT_ARRAY, code, list(features.shape))
-    d_filt = TensorDescriptor(filters_layout, code, list(filters.shape))
-    d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
-    d_out = TensorDescriptor(LAYOUT_ARRAY, code, [num_act_out, co])
+    d_feat = _descriptor(LAYOUT_ARRAY, code, list(features.shape))
+    d_filt = _descriptor(filters_layout, code, list(filters.shape))
+    d_pairs = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+    d_out = _descriptor(LAYOUT_ARRAY, code, [num_act_out, co])
     counts = _host_counts(indice_num_host)
     size = ctypes.c_size_t(0)
     check(lib().mluOpGetIndiceConvolutionForwardWorkspaceSize(
@@ -529,10 +545,10 @@ def indice_conv_backward_data(handle, output_grad, filters, filters_layout, indi
     K, _, L = indice_pairs.shape
     rows = L if rows is None else int(rows)
     dx = _output((rows, ci), output_grad.dtype, output_grad.device, "input_grad")
-    d_dy = TensorDescriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
-    d_filt = TensorDescriptor(filters_layout, code, list(filters.shape))
-    d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
-    d_dx = TensorDescriptor(LAYOUT_ARRAY, code, [rows, ci])
+    d_dy = _descriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
+    d_filt = _descriptor(filters_layout, code, list(filters.shape))
+    d_pairs = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+    d_dx = _descriptor(LAYOUT_ARRAY, code, [rows, ci])
     counts = _host_counts(indice_num_host)
     size = ctypes.c_size_t(0)
     check(lib().mluOpGetIndiceConvolutionBackwardDataWorkspaceSize(
@@ -565,10 +581,10 @@ def indice_conv_backward_filter(handle, features, output_grad, indice_pairs, ind
     else:
         shape = tuple(filter_space) + (ci, co)
     dw = _output(shape, features.dtype, features.device, "filters_grad")
-    d_x = TensorDescriptor(LAYOUT_ARRAY, code, list(features.shape))
-    d_dy = TensorDescriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
-    d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
-    d_dw = TensorDescriptor(grad_layout, code, list(dw.shape),
+    d_x = _descriptor(LAYOUT_ARRAY, code, list(features.shape))
+    d_dy = _descriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
+    d_pairs = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+    d_dw = _descriptor(grad_layout, code, list(dw.shape),
                             onchip_dtype=DTYPE_FLOAT if onchip_float else None)
     counts = _host_counts(indice_num_host)
     size = ctypes.c_size_t(0)
@@ -594,10 +610,10 @@ def indice_conv_backward_filter_no_alloc(handle, features, output_grad, indice_p
     ([kd, kh, kw, Ci, Co]): no workspace, the library's own scratch array instead."""
     code = torch_dtype_code(features.dtype)
     K, _, L = indice_pairs.shape
-    d_x = TensorDescriptor(LAYOUT_ARRAY, code, list(features.shape))
-    d_dy = TensorDescriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
-    d_pairs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
-    d_dw = TensorDescriptor(LAYOUT_ARRAY, code, list(filters_grad.shape),
+    d_x = _descriptor(LAYOUT_ARRAY, code, list(features.shape))
+    d_dy = _descriptor(LAYOUT_ARRAY, code, list(output_grad.shape))
+    d_pairs = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [K, 2, L])
+    d_dw = _descriptor(LAYOUT_ARRAY, code, list(filters_grad.shape),
                             onchip_dtype=DTYPE_FLOAT if onchip_float else None)
     check(lib().mluOpExtIndiceConvolutionBackwardFilterNoAlloc(
         handle.ptr, d_x.ptr, features.data_ptr(), d_dy.ptr, output_grad.data_ptr(), d_pairs.ptr,
@@ -620,13 +636,13 @@ def voxelization(handle, points, voxel_size, coors_range, max_points, max_voxels
     coors = _output((max_voxels, 3), torch.int32, dev, "coors")
     npv = _output((max_voxels,), torch.int32, dev, "num_points_per_voxel")
     voxel_num = torch.zeros((1,), dtype=torch.int32, device=dev)
-    d_points = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, f])
-    d_vs = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [3])
-    d_cr = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [6])
-    d_voxels = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [max_voxels, max_points, f])
-    d_coors = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [max_voxels, 3])
-    d_npv = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [max_voxels])
-    d_num = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [1])
+    d_points = _descriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, f])
+    d_vs = _descriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [3])
+    d_cr = _descriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [6])
+    d_voxels = _descriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [max_voxels, max_points, f])
+    d_coors = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [max_voxels, 3])
+    d_npv = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [max_voxels])
+    d_num = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [1])
     size = ctypes.c_size_t(0)
     check(lib().mluOpGetVoxelizationWorkspaceSize(
         handle.ptr, d_points.ptr, d_vs.ptr, d_cr.ptr, max_points, max_voxels, 3, bool(deterministic),
@@ -658,13 +674,13 @@ def dynamic_point_to_voxel_forward(handle, feats, coors, reduce_type="max", rows
     count = _output((m,), torch.int32, dev, "voxel_points_count")
     voxel_num = torch.zeros((1,), dtype=torch.int32, device=dev)
     mode = {"max": REDUCE_DMAX, "mean": REDUCE_DMEAN, "sum": REDUCE_DSUM}[reduce_type]
-    d_feats = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
-    d_coors = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [n, 3])
-    d_vf = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [m, c])
-    d_vc = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [m, 3])
-    d_p2v = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [n])
-    d_cnt = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [m])
-    d_num = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [1])
+    d_feats = _descriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
+    d_coors = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [n, 3])
+    d_vf = _descriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [m, c])
+    d_vc = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [m, 3])
+    d_p2v = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [n])
+    d_cnt = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [m])
+    d_num = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [1])
     size = ctypes.c_size_t(0)
     check(lib().mluOpGetDynamicPointToVoxelForwardWorkspaceSize(handle.ptr, d_feats.ptr, d_coors.ptr,
                                                                 ctypes.byref(size)),
@@ -687,13 +703,13 @@ def dynamic_point_to_voxel_backward(handle, grad_voxel_feats, feats, voxel_feats
     m = grad_voxel_feats.shape[0]
     grad_feats = _output((n, c), torch.float32, feats.device, "grad_feats")
     mode = {"max": REDUCE_DMAX, "mean": REDUCE_DMEAN, "sum": REDUCE_DSUM}[reduce_type]
-    d_g = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [m, c])
-    d_feats = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
-    d_vf = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [m, c])
-    d_p2v = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [n])
-    d_cnt = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [m])
-    d_num = TensorDescriptor(LAYOUT_ARRAY, DTYPE_INT32, [1])
-    d_out = TensorDescriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
+    d_g = _descriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [m, c])
+    d_feats = _descriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
+    d_vf = _descriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [m, c])
+    d_p2v = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [n])
+    d_cnt = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [m])
+    d_num = _descriptor(LAYOUT_ARRAY, DTYPE_INT32, [1])
+    d_out = _descriptor(LAYOUT_ARRAY, DTYPE_FLOAT, [n, c])
     size = ctypes.c_size_t(0)
     check(lib().mluOpGetDynamicPointToVoxelBackwardWorkspaceSize(
         handle.ptr, mode, d_g.ptr, d_feats.ptr, d_vf.ptr, d_p2v.ptr, d_cnt.ptr, d_num.ptr, ctypes.byref(size)),

@@ -187,6 +187,10 @@ class _ConvBase(torch.nn.Module):
             rb = x.rulebooks[self.indice_key]
             assert rb.filter_space == tuple(self.kernel_size) and rb.sub_m == self.sub_m
             return rb
+        # a rulebook planned for this layer and these very coordinates (SparseSequential)
+        planned = x.rulebooks.get(("planned", id(self)))
+        if planned is not None and planned.in_indices is x.indices and planned.in_space == x.spatial_shape:
+            return planned
         if self.sub_m:
             out_space = list(x.spatial_shape)
         else:
@@ -200,7 +204,17 @@ class _ConvBase(torch.nn.Module):
                       out_space, in_indices=x.indices, in_space=x.spatial_shape, distinct=x.distinct)
         if self.indice_key is not None:
             x.rulebooks[self.indice_key] = rb
+        else:
+            x.rulebooks[("planned", id(self))] = rb
         return rb
+
+    def _cells_after(self, x, rb):
+        """(indices, spatial shape, distinct) of this layer's result on `x`, from the rulebook alone."""
+        if self.sub_m:
+            return x.indices, x.spatial_shape, x.distinct
+        if self.inverse:
+            return rb.in_indices, rb.in_space, rb.distinct
+        return rb.out_indices.contiguous(), rb.out_space, True
 
     def _result(self, x, rb, feats):
         if self.sub_m:
@@ -267,6 +281,40 @@ class SparseInverseConv3d(_ConvBase):
 
     def _result(self, x, rb, feats):
         return SparseTensor(feats, rb.in_indices, rb.in_space, x.batch_size, x.rulebooks, distinct=rb.distinct)
+
+
+class SparseSequential(torch.nn.Sequential):
+    """Layers applied in order to a SparseTensor (spconv's SparseSequential): sparse convolutions
+    take and return the tensor, any other module is applied to its features.
+
+    Before the first layer runs, the rulebooks of all its convolutions are built, one after the
+    other: a rulebook needs coordinates only, and each ends in a wait for its pair counts (the
+    operators take `indice_num` on the host).  Built layer by layer inside the network, every such
+    wait drains the queue in front of the convolutions that follow; built up front, the host
+    runs ahead through all convolutions and the device stays busy."""
+
+    def plan(self, x):
+        cells = x
+        for m in self:
+            if isinstance(m, SparseSequential):
+                cells = m.plan(cells)
+            elif isinstance(m, _ConvBase):
+                rb = m._rulebook(cells)
+                indices, space, distinct = m._cells_after(cells, rb)
+                if indices is not cells.indices:
+                    # (features are not looked at while planning: a view of the right height)
+                    cells = SparseTensor(indices.new_empty((indices.shape[0], 0)), indices, space,
+                                         cells.batch_size, cells.rulebooks, distinct)
+        return cells
+
+    def forward(self, x):
+        self.plan(x)
+        for m in self:
+            if isinstance(m, (_ConvBase, SparseSequential)):
+                x = m(x)
+            else:
+                x = x.replace_features(m(x.features))
+        return x
 
 
 class Voxelization(torch.nn.Module):

@@ -77,6 +77,56 @@ def test_layers_match_dense_autograd(gpu_handle):
         close(layer.weight.grad.cpu().numpy(), rw.grad.numpy(), "grad " + name)
 
 
+def test_sequential_plans_all_rulebooks_first_and_matches_the_layers_one_by_one(gpu_handle, monkeypatch):
+    """SparseSequential builds the rulebooks of all its convolutions before the first layer runs (keyed
+    layers share one, keyless strided layers get theirs planned, the inverse layer finds its partner's)
+    and gives the bits of the same layers applied one by one."""
+    import torch
+    from mluop_hip import nn as spnn
+    rng = np.random.default_rng(23)
+    batch, space, L = 2, (8, 10, 12), 400
+    idx = random_voxels(rng, batch, space, L)
+    feats = torch.from_numpy(rng.standard_normal((L, 16)).astype(np.float32)).cuda()
+    torch.manual_seed(5)
+    layers = [spnn.SubMConv3d(16, 16, 3, indice_key="a"), torch.nn.ReLU(),
+              spnn.SubMConv3d(16, 32, 3, indice_key="a"), torch.nn.ReLU(),
+              spnn.SparseConv3d(32, 32, 3, stride=2, padding=1, indice_key="down"),
+              spnn.SparseSequential(spnn.SubMConv3d(32, 32, 3), torch.nn.ReLU(),
+                                    spnn.SparseConv3d(32, 64, 3, stride=2, padding=1)),
+              spnn.SubMConv3d(64, 64, 3)]
+    net = spnn.SparseSequential(*layers).cuda()
+    indices = torch.from_numpy(idx).cuda()
+
+    built, order = [], []
+    real = spnn.get_indice_pairs
+    monkeypatch.setattr(spnn, "get_indice_pairs", lambda *a, **k: (built.append(1), real(*a, **k))[1])
+    real_apply = spnn._IndiceConv.apply
+    x1 = feats.clone().requires_grad_(True)
+    hooks = [m.register_forward_pre_hook(lambda mod, inp: order.append(len(built)))
+             for m in net.modules() if isinstance(m, spnn._ConvBase)]
+    y = net(spnn.SparseTensor(x1, indices, space, batch))
+    for h in hooks:
+        h.remove()
+    # six convolutions, five rulebooks (two layers share "a"), all of them there before the first layer ran
+    assert len(built) == 5 and order == [5] * 6
+    y.features.square().sum().backward()
+
+    x2 = feats.clone().requires_grad_(True)
+    grads1 = [p.grad.clone() for p in net.parameters()]
+    for p in net.parameters():
+        p.grad = None
+    t = spnn.SparseTensor(x2, indices, space, batch)
+    flat = layers[:5] + list(layers[5]) + layers[6:]
+    for m in flat:
+        t = m(t) if isinstance(m, spnn._ConvBase) else t.replace_features(m(t.features))
+    t.features.square().sum().backward()
+    torch.cuda.synchronize()
+    assert torch.equal(y.indices, t.indices) and torch.equal(y.features, t.features)
+    assert torch.equal(x1.grad, x2.grad)
+    for g1, p in zip(grads1, net.parameters()):
+        assert torch.equal(g1, p.grad)
+
+
 def test_half_precision_layer_runs_mfma_path(gpu_handle):
     """fp16 features through SubMConv3d(64, 64): graded at the fp16 threshold against float64."""
     import torch
