@@ -876,6 +876,9 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   }
 }
 
+// What a lane without a row of its own loads: a row of zeros in device memory.
+__device__ __attribute__((aligned(256))) unsigned char kZeroRow[512];  // never written
+
 // ---- MFMA gather convolution, one free-running wavefront per tile ---------------------
 //
 // The kernel above spends a tile's life waiting: cut positions, then pairs, then
@@ -1019,6 +1022,10 @@ __global__ __launch_bounds__(64) void gatherConvWave(
   char *acc_lane = reinterpret_cast<char *>(s_acc) + 4 * quad * 4;
   char *stage = s_stage;
 
+  // Rows of up to 64 bytes are loaded by the lane that multiplies them, 16 bytes of its own
+  // pair's row (the 16 rows of a unit are 16 cache lines either way); longer rows are
+  // fetched row by row, half as many lines a load, and turned into fragments by the LDS slot.
+  constexpr bool kDirectRows = ROW_BYTES <= 64;
   int pair_row[NE], pair_src[NE];
   u32x4 rows[NR][RL];
   vec8 w[NR][KB][NB];
@@ -1040,12 +1047,22 @@ __global__ __launch_bounds__(64) void gatherConvWave(
   auto request_rows = [&](int pslot, int rslot) {
     const int n = unit_n[pslot];
     const int k = unit_k[pslot] < K ? unit_k[pslot] : 0;
+    if constexpr (kDirectRows) {
+      static_assert(!kDirectRows || (RL == 1 && KB == 1), "one fragment a row");
+      int g = pair_src[pslot];
+      if (pair >= n || (unsigned)g >= (unsigned)source.n_src) g = 0;
+      // (a lane beyond the row's channels reads the row of zeros)
+      const char *from = quad * 16 < ROW_BYTES ? a_bytes + (size_t)g * ROW_BYTES + quad * 16
+                                               : reinterpret_cast<const char *>(kZeroRow);
+      rows[rslot][0] = *reinterpret_cast<const u32x4 *>(from);
+    } else {
 #pragma unroll
-    for (int h = 0; h < RL; ++h) {
-      const int e = lane / PPR + EPL * h;  // which pair's row this lane fetches a piece of
-      int g = __shfl(pair_src[pslot], e & 15, kWave);
-      if (e >= n || (unsigned)g >= (unsigned)source.n_src) g = 0;
-      rows[rslot][h] = *reinterpret_cast<const u32x4 *>(a_bytes + (size_t)g * ROW_BYTES + (lane % PPR) * 16);
+      for (int h = 0; h < RL; ++h) {
+        const int e = lane / PPR + EPL * h;  // which pair's row this lane fetches a piece of
+        int g = __shfl(pair_src[pslot], e & 15, kWave);
+        if (e >= n || (unsigned)g >= (unsigned)source.n_src) g = 0;
+        rows[rslot][h] = *reinterpret_cast<const u32x4 *>(a_bytes + (size_t)g * ROW_BYTES + (lane % PPR) * 16);
+      }
     }
     const char *bk = b_base + (size_t)k * kBytesPerOffset;
 #pragma unroll
@@ -1067,18 +1084,22 @@ __global__ __launch_bounds__(64) void gatherConvWave(
       acc[nb] = *reinterpret_cast<float4v *>(dst + nb * 64);
       prod[nb] = float4v{0.f, 0.f, 0.f, 0.f};
     }
-#pragma unroll
-    for (int h = 0; h < RL; ++h) {
-      const int e = lane / PPR + EPL * h;
-      if (16 * PPR >= 64 || lane < 16 * PPR)
-        *reinterpret_cast<u32x4 *>(stage + e * STAGE_STRIDE + (lane % PPR) * 16) = rows[rslot][h];
-    }
     vec8 afr[KB];
+    if constexpr (kDirectRows) {
+      afr[0] = __builtin_bit_cast(vec8, rows[rslot][0]);
+    } else {
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-      afr[kb] = *reinterpret_cast<const vec8 *>(stage + pair * STAGE_STRIDE + kb * 64 + quad * 16);
-    if constexpr (kPartialFragment) {
-      if (quad * E::kVec >= Q) afr[0] = vec8{};
+      for (int h = 0; h < RL; ++h) {
+        const int e = lane / PPR + EPL * h;
+        if (16 * PPR >= 64 || lane < 16 * PPR)
+          *reinterpret_cast<u32x4 *>(stage + e * STAGE_STRIDE + (lane % PPR) * 16) = rows[rslot][h];
+      }
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+        afr[kb] = *reinterpret_cast<const vec8 *>(stage + pair * STAGE_STRIDE + kb * 64 + quad * 16);
+      if constexpr (kPartialFragment) {
+        if (quad * E::kVec >= Q) afr[0] = vec8{};
+      }
     }
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
@@ -1130,7 +1151,6 @@ __global__ __launch_bounds__(64) void gatherConvWave(
 // flight, the requests for the offset after included).  A lane whose row has no
 // partner at the offset reads a row of zeros; a row group none of whose rows has one
 // is skipped, and a wave without any skips the offset.
-__device__ __attribute__((aligned(256))) unsigned char kZeroRow[512];  // never written
 constexpr int kDenseChunk = 27;      // offsets whose row-map slice is resident in LDS at once
 constexpr int kDenseMapBatch = 14;   // loads in flight per thread while a tile's row map is read
 constexpr int kDenseWaves = 4;
