@@ -1961,7 +1961,7 @@ __global__ __launch_bounds__(256) void backwardFilterMfma(
 // The same product for 2-byte elements and 32 to 128 channels on both sides, with the
 // transposition done by the LDS read itself.  The gathered rows go from global memory
 // straight into LDS as they are ([pair][channel], 16 bytes per lane, a pair without a
-// valid row reads a row of zeros), one step of 64 pairs ahead into the other of two
+// valid row reads a row of zeros), one step of 64 (or 32) pairs ahead into the other of two
 // buffers, and `ds_read_b64_tr_b16` hands a lane four consecutive pairs of one channel:
 // within 16 lanes, lane i supplies the address of 4 channels of pair i / 4 and lane j
 // receives channel j of the four pairs.  Two such reads are one operand fragment.  No
@@ -1977,7 +1977,7 @@ constexpr int filterRowSwizzle(int row_bytes, int pair) {
                           : 0;
 }
 
-template <typename E, int CI, int CO>
+template <typename E, int CI, int CO, int SP>
 __global__ __launch_bounds__(256) void backwardFilterMfmaTr(
     const typename E::storage *X, const typename E::storage *dY, const int32_t *pairs, int L,
     int x_col, int n_in, int n_out, int K, SliceTable tab, SliceOrder order, int total_slices,
@@ -1988,7 +1988,6 @@ __global__ __launch_bounds__(256) void backwardFilterMfmaTr(
   typedef short v8i16 __attribute__((ext_vector_type(8)));
   static_assert(sizeof(S) == 2 && E::kChunk == 32, "2-byte elements, 32 pairs per fragment");
   static_assert(CI % 32 == 0 && CO % 32 == 0 && CI <= 128 && CO <= 128, "two row and column blocks per wave pair");
-  constexpr int SP = kFilterStepPairs;
   // two chunks of row indices: with 128 channels on both sides the buffers leave 16 KiB of
   // half a CU's LDS
   constexpr int kIndexChunk = 512;
@@ -1997,7 +1996,7 @@ __global__ __launch_bounds__(256) void backwardFilterMfmaTr(
   constexpr int XN = SP * RBX / 1024;           // 1 KiB wave-loads per step
   constexpr int YN = SP * RBY / 1024;
   constexpr int AB = CI / 32, BB = CO / 32;     // 16-row / 16-column blocks per wave
-  static_assert(SP == 64, "two fragments per step");
+  static_assert(SP == 32 || SP == 64, "one or two fragments per step");
 
   __shared__ __attribute__((aligned(1024))) char s_x[2][SP * RBX];
   __shared__ __attribute__((aligned(1024))) char s_y[2][SP * RBY];
@@ -2846,7 +2845,12 @@ void launchFilterMfmaInstance(const LaunchCtx &lc, const ConvProblem &p, const S
   if (total_slices > 0) {
     if constexpr (kTransposingReads) {
       if (lc.choices.filter_stores != 1) {
-        backwardFilterMfmaTr<E, CI, CO><<<grid, 256, 0, lc.stream>>>(
+        // Steps of 32 pairs halve the row buffers: below 128 x 128 channels more workgroups
+        // share a CU then, which pays when the slices are long (network 64 x 64: 101 -> 88 us;
+        // on slices of a few steps the shorter steps only add barriers: config 4 23.7 -> 25.3 us).
+        const bool short_steps = CI + CO < 256 && slice_len >= 2048;
+        auto kernel = short_steps ? backwardFilterMfmaTr<E, CI, CO, 32> : backwardFilterMfmaTr<E, CI, CO, 64>;
+        kernel<<<grid, 256, 0, lc.stream>>>(
             static_cast<const S *>(features), static_cast<const S *>(output_grad), p.indice_pairs,
             p.L, p.inverse ? 1 : 0, p.inverse ? p.num_out : p.L, p.inverse ? p.L : p.num_out, p.K,
             tab, order, total_slices, slice_len, partial);

@@ -179,6 +179,41 @@ def test_backward_filter_kernels_agree(gpu_handle, shape, dtype_name):
     assert torch.equal(got[False], got[True])
 
 
+def test_backward_filter_short_steps_on_long_slices(gpu_handle):
+    """Below 128 x 128 channels, slices of 2048 pairs and more are multiplied in steps of 32 pairs
+    (another instance of the transposing-read kernel).  3.4 million pairs of a nearly full grid: bit
+    for bit against the storing kernel, and a sample of offsets against a float64 product on the host."""
+    import torch
+    import mluop_hip
+    from spconv_cases import random_voxels, to_torch
+    rng = np.random.default_rng(61)
+    space, ks, ci, co = (32, 64, 64), (3, 3, 3), 64, 32
+    idx = random_voxels(rng, 1, space, 125000, shuffle=False)
+    pairs, _, num, n_out = mluop_hip.get_indice_pairs(gpu_handle, torch.from_numpy(idx).cuda(), 1, space, ks, space,
+                                                      [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+    num_host = [int(v) for v in num.cpu()]
+    assert sum(num_host) >= 768 * 2048
+    feats = torch.from_numpy(rng.standard_normal((idx.shape[0], ci)).astype(np.float32)).cuda().half()
+    dy = torch.from_numpy((rng.standard_normal((n_out, co)) * 0.1).astype(np.float32)).cuda().half()
+    got = {}
+    for stores in (False, True):
+        gpu_handle.set_kernel_choice("filter_stores", True if stores else None)
+        try:
+            got[stores] = mluop_hip.indice_conv_backward_filter(gpu_handle, feats, dy, pairs, num_host, ks, True)
+            torch.cuda.synchronize()
+        finally:
+            gpu_handle.set_kernel_choice("filter_stores", None)
+    assert torch.equal(got[False], got[True])
+    dw = got[False].float().reshape(27, ci, co)
+    for k in (0, 13, 26):
+        n = num_host[k]
+        x_k = feats[pairs[k, 0, :n].long()].double()
+        dy_k = dy[pairs[k, 1, :n].long()].double()
+        ref = x_k.t() @ dy_k
+        err = (dw[k].double() - ref).abs().sum() / ref.abs().sum()
+        assert float(err) <= 3e-3, (k, float(err))
+
+
 @pytest.mark.parametrize("layout_name", ["NDHWC", "NCDHW", "ARRAY"])
 @pytest.mark.parametrize("dtype_name", ["float32", "float16"])
 def test_forward_filter_layouts(gpu_handle, layout_name, dtype_name):
