@@ -1137,9 +1137,9 @@ __global__ __launch_bounds__(64) void gatherConvWave(
 // When most rows of a tile have a partner at most offsets, compacting pairs buys
 // little and the fp32 accumulate in LDS (a 16-byte read-modify-write per lane and
 // 16 result columns, on arbitrary rows: bank conflicts) is what the kernel above
-// spends its time on.  Here a wave owns G groups of 16 result rows and all result
-// columns, and accumulates them in registers over all offsets: no accumulator traffic
-// at all.  The partner rows of an offset come from global memory straight into the
+// spends its time on.  Here a tile is 128 result rows (256 below 128 channels), a wave
+// of eight owns G = 1 (2) groups of 16 of them and all result columns, and accumulates
+// them in registers over all offsets: no accumulator traffic at all.  The partner rows of an offset come from global memory straight into the
 // operand registers of the lane that multiplies them (lane (row, quarter) loads 16
 // bytes of its row per reduction chunk, one offset ahead), so no wave waits for
 // another one's rows.  What the waves of a workgroup share is the offset's filter: its
@@ -1153,13 +1153,15 @@ __global__ __launch_bounds__(64) void gatherConvWave(
 // is skipped, and a wave without any skips the offset.
 constexpr int kDenseChunk = 27;      // offsets whose row-map slice is resident in LDS at once
 constexpr int kDenseMapBatch = 14;   // loads in flight per thread while a tile's row map is read
-constexpr int kDenseWaves = 4;
-// row groups per wave: as many as leave room for two sets of partner rows in the registers
-constexpr int denseGroups(int Q, int C) { return (C >= 128 || Q >= 128) ? 2 : 4; }
+constexpr int kDenseWaves = 8;
+// Row groups per wave: with two sets of partner rows a wave stays within 128 registers, four
+// waves a SIMD.  (Four waves of twice the groups measured the same at 64 and 128 columns and
+// 12 % slower at 16 and 32, where a wave has little to multiply between two barriers.)
+constexpr int denseGroups(int Q, int C) { return (C >= 128 || Q >= 128) ? 1 : 2; }
 constexpr int denseTileRows(int Q, int C) { return kDenseWaves * denseGroups(Q, C) * 16; }
 
 template <typename E, int Q, int C, typename SRC>
-__global__ __launch_bounds__(64 * kDenseWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void gatherConvDense(
+__global__ __launch_bounds__(64 * kDenseWaves) __attribute__((amdgpu_waves_per_eu(4, 4))) void gatherConvDense(
     const typename E::storage *A, const typename E::storage *packedW, SRC source, int R,
     int K, int ldc, typename E::storage *result) {
   typedef typename E::vec8 vec8;
@@ -1355,8 +1357,9 @@ __global__ __launch_bounds__(64 * kDenseWaves) __attribute__((amdgpu_waves_per_e
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           const vec8 wf = *reinterpret_cast<const vec8 *>(wbuf + (nb * KB + kb) * 1024 + lane * 16);
-          if (MASK & 1) acc[G0][nb] = E::mfma(wf, rows[G0][kb], acc[G0][nb]);
-          if (MASK & 2) acc[G0 + 1][nb] = E::mfma(wf, rows[G0 + 1][kb], acc[G0 + 1][nb]);
+          if constexpr ((MASK & 1) != 0) acc[G0][nb] = E::mfma(wf, rows[G0][kb], acc[G0][nb]);
+          if constexpr ((MASK & 2) != 0 && G0 + 1 < G)
+            acc[G0 + 1][nb] = E::mfma(wf, rows[G0 + 1][kb], acc[G0 + 1][nb]);
         }
     };
     auto multiply_present = [&](int present, const vec8 (&rows)[G][KB], const char *wbuf) {
