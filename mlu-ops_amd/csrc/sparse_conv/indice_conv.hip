@@ -2567,7 +2567,7 @@ bool useDenseKernel(const LaunchCtx &lc, const ConvProblem &p, const GatherDims 
   // the pair-list kernels cost with the pairs.  Measured on 150000 rows, 3x3x3, fp16, as the
   // share of all (row, offset) slots that hold a pair from which the kernel wins:
   //   result columns   voxels strewn uniformly   scenes (filled sheets and walls)
-  //   16, 32           0.4  (0.27: 53 us against 45 us, 0.51: 57 against 67)   0.07 (38 against 49)
+  //   16, 32           0.35 (0.27: 45 us against 40 us, 0.51: 50 against 60)   0.04 (30 against 32)
   //   64               0.38 (0.27: 86 against 77, 0.51: 104 against 119)      0.15 (67 against 73)
   //   128              0.25 (175 against 183)                                  0.04 (88 against 98)
   // On strewn voxels every piece holds a few pairs; in a scene the pairs of an offset sit in
@@ -2589,7 +2589,7 @@ bool useDenseKernel(const LaunchCtx &lc, const ConvProblem &p, const GatherDims 
   // (the largest count is the centre offset of a submanifold convolution: left out)
   const double mean_rest = p.K > 1 ? (pairs - largest) / (p.K - 1) : 0.0;
   const bool sheets = mean_rest > 0 && second >= 1.5 * mean_rest;
-  if (d.C <= 32) return fill >= (sheets ? 0.07 : 0.4);
+  if (d.C <= 32) return fill >= (sheets ? 0.04 : 0.35);
   if (d.C == 64) return fill >= (sheets ? 0.15 : 0.38);
   return fill >= (sheets ? 0.04 : 0.25);
 }
