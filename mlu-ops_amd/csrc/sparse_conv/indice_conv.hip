@@ -405,6 +405,8 @@ __device__ __forceinline__ void scanAllPairsForTile(const typename E::storage *A
 //    remaining tiles with the pair count (an offset without pairs gets one workgroup
 //    that closes all its tiles with 0).  A lane with more than a few tiles to close
 //    hands them to the whole wave.
+constexpr int kCutPairsPerThread = 4;
+
 template <typename E>
 __global__ __launch_bounds__(256) void packFilterCutPairLists(
     const typename E::storage *W, int64_t sK, int64_t sQ, int64_t sC, int K, int Q, int C,
@@ -440,45 +442,58 @@ __global__ __launch_bounds__(256) void packFilterCutPairLists(
   }
   const int k = lo;
   const int n = inl.n[k];
-  const int p = (b - blocks.first[k]) * 256 + (int)threadIdx.x;
   const int lane = threadIdx.x & 63;
-  const bool live = p < n;
   const int32_t *row_list = pairs + ((size_t)k * 2 + row_col) * L;
   const int32_t *src_list = pairs + ((size_t)k * 2 + src_col) * L;
-  int r = 0, prev = -1, s = 0;
-  if (live) {
-    r = row_list[p];
-    s = src_list[p];
-    if (p > 0) prev = row_list[p - 1];
-  }
-  const bool ok = (unsigned)r < (unsigned)R && (unsigned)s < (unsigned)n_src && r > prev;
-  if (live && !ok) *verdict = ticket;
-  // tiles (t_lo .. t_mid] open at p, tiles (t_mid .. n_tiles] close with n; clamped so
-  // that a list out of order, whose table nobody reads, still writes inside the table
-  int t_mid = r >> tile_shift;
-  t_mid = t_mid < 0 ? 0 : (t_mid > n_tiles - 1 ? n_tiles - 1 : t_mid);
-  int t_lo = p == 0 ? -1 : (prev >> tile_shift);
-  t_lo = t_lo < -1 ? -1 : (t_lo > t_mid ? t_mid : t_lo);
   int32_t *row_cuts = cuts + (size_t)k * (n_tiles + 1);
-  // job 0: value p over (t_lo, t_mid]; job 1 (last pair only): value n over (t_mid, n_tiles]
+  // kCutPairsPerThread pairs a thread, 256 apart: all their loads are requested first
+  const int p0 = (b - blocks.first[k]) * (256 * kCutPairsPerThread) + (int)threadIdx.x;
+  int rs[kCutPairsPerThread], prevs[kCutPairsPerThread], ss[kCutPairsPerThread];
 #pragma unroll
-  for (int job = 0; job < 2; ++job) {
-    // (an offset without pairs has one workgroup, whose first lane closes all tiles with 0)
-    const bool empty_offset = n == 0 && threadIdx.x == 0;
-    const int first = empty_offset ? 0 : (job == 0 ? t_lo + 1 : t_mid + 1);
-    const int last = job == 0 ? t_mid : n_tiles;
-    const int value = job == 0 ? p : n;
-    const bool mine = ((live && (job == 0 || p == n - 1)) || (empty_offset && job == 1)) && first <= last;
-    const bool wide = mine && last - first >= 4;
-    if (mine && !wide)
-      for (int t = first; t <= last; ++t) row_cuts[t] = value;
-    unsigned long long m = __ballot(wide);
-    while (m) {
-      const int from = __ffsll((long long)m) - 1;
-      m &= m - 1;
-      const int f = __shfl(first, from, kWave), l = __shfl(last, from, kWave);
-      const int v = __shfl(value, from, kWave);
-      for (int t = f + lane; t <= l; t += kWave) row_cuts[t] = v;
+  for (int j = 0; j < kCutPairsPerThread; ++j) {
+    const int p = p0 + j * 256;
+    rs[j] = 0;
+    prevs[j] = -1;
+    ss[j] = 0;
+    if (p < n) {
+      rs[j] = row_list[p];
+      ss[j] = src_list[p];
+      if (p > 0) prevs[j] = row_list[p - 1];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kCutPairsPerThread; ++j) {
+    const int p = p0 + j * 256;
+    const bool live = p < n;
+    const int r = rs[j], prev = prevs[j], s = ss[j];
+    const bool ok = (unsigned)r < (unsigned)R && (unsigned)s < (unsigned)n_src && r > prev;
+    if (live && !ok) *verdict = ticket;
+    // tiles (t_lo .. t_mid] open at p, tiles (t_mid .. n_tiles] close with n; clamped so
+    // that a list out of order, whose table nobody reads, still writes inside the table
+    int t_mid = r >> tile_shift;
+    t_mid = t_mid < 0 ? 0 : (t_mid > n_tiles - 1 ? n_tiles - 1 : t_mid);
+    int t_lo = p == 0 ? -1 : (prev >> tile_shift);
+    t_lo = t_lo < -1 ? -1 : (t_lo > t_mid ? t_mid : t_lo);
+    // job 0: value p over (t_lo, t_mid]; job 1 (last pair only): value n over (t_mid, n_tiles]
+#pragma unroll
+    for (int job = 0; job < 2; ++job) {
+      // (an offset without pairs has one workgroup, whose first lane closes all tiles with 0)
+      const bool empty_offset = n == 0 && threadIdx.x == 0 && j == 0;
+      const int first = empty_offset ? 0 : (job == 0 ? t_lo + 1 : t_mid + 1);
+      const int last = job == 0 ? t_mid : n_tiles;
+      const int value = job == 0 ? p : n;
+      const bool mine = ((live && (job == 0 || p == n - 1)) || (empty_offset && job == 1)) && first <= last;
+      const bool wide = mine && last - first >= 4;
+      if (mine && !wide)
+        for (int t = first; t <= last; ++t) row_cuts[t] = value;
+      unsigned long long m = __ballot(wide);
+      while (m) {
+        const int from = __ffsll((long long)m) - 1;
+        m &= m - 1;
+        const int f = __shfl(first, from, kWave), l = __shfl(last, from, kWave);
+        const int v = __shfl(value, from, kWave);
+        for (int t = f + lane; t <= l; t += kWave) row_cuts[t] = v;
+      }
     }
   }
 }
@@ -2689,7 +2704,8 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
     int list_blocks = 0;
     for (int k = 0; k < kMaxInlineK; ++k) {
       ob.first[k] = list_blocks;
-      if (k < p.K) list_blocks += inl.n[k] > 0 ? (inl.n[k] + 255) / 256 : 1;
+      const int per_block = 256 * kCutPairsPerThread;
+      if (k < p.K) list_blocks += inl.n[k] > 0 ? (inl.n[k] + per_block - 1) / per_block : 1;
     }
     const size_t frags = (size_t)p.K * (d.C / 16) * ((d.Q + E::kChunk - 1) / E::kChunk) * 64;
     const int pack_blocks = gridFor(frags, 512);
