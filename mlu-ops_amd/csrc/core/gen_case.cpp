@@ -136,6 +136,11 @@ void CaseWriter::param(const char *name, int64_t value) {
   params_ += std::string("  ") + name + ": " + std::to_string(value) + "\n";
 }
 
+void CaseWriter::paramName(const char *name, const char *enumerator) {
+  if (mode_ == 0) return;
+  params_ += std::string("  ") + name + ": " + enumerator + "\n";
+}
+
 void CaseWriter::params(const char *name, const int *values, int n) {
   for (int i = 0; i < n; ++i) param(name, values[i]);
 }

@@ -31,6 +31,7 @@ class CaseWriter {
   void input(const char *id, const mluOpTensorDescriptor_t desc, const void *device_values);
   void output(const char *id, const mluOpTensorDescriptor_t desc);
   void param(const char *name, int64_t value);
+  void paramName(const char *name, const char *enumerator);  // an enumeration written by name
   void params(const char *name, const int *values, int n);
   void params(const char *name, const int64_t *values, int n);
   // error functions DIFF1 and DIFF2 at `threshold`, CPU baseline; writes the file

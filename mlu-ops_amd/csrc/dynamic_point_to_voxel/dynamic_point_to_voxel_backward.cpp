@@ -6,6 +6,7 @@
 // exceeds one core's on-chip memory (5 N + 20 C + 4 bytes, :118-136); there is no
 // such limit here.
 #include "core/core.h"
+#include "core/gen_case.h"
 #include "dynamic_point_to_voxel/scatter_points.h"
 
 namespace {
@@ -117,6 +118,20 @@ mluOpStatus_t MLUOP_WIN_API mluOpDynamicPointToVoxelBackward(
   PARAM_CHECK(api, grad_feats != NULL);
   if (workspace_size != 0) {
     PARAM_CHECK(api, workspace != NULL);
+  }
+  if (mluop::gen_case::mode() != 0) {
+    // (reference kernels/dynamic_point_to_voxel/dynamic_point_to_voxel_backward/
+    // dynamic_point_to_voxel_backward.cpp:254-270)
+    mluop::gen_case::CaseWriter c(handle, "dynamic_point_to_voxel_backward", "dynamic_point_to_voxel_backward_param");
+    c.input("grad_voxel_feats", grad_voxel_feats_desc, grad_voxel_feats);
+    c.input("feats", feats_desc, feats);
+    c.input("voxel_feats", voxel_feats_desc, voxel_feats);
+    c.input("point2voxel_map", point2voxel_map_desc, point2voxel_map);
+    c.input("voxel_points_count", voxel_points_count_desc, voxel_points_count);
+    c.input("voxel_num", voxel_num_desc, voxel_num);
+    c.output("grad_feats", grad_feats_desc);
+    c.paramName("reduce_type", reduce_type == MLUOP_REDUCE_DMAX ? "REDUCE_MODE_MAX" : "REDUCE_MODE_MEAN");
+    c.finish(0.003);
   }
   DEVICE_HANDLE_CHECK(api, handle);
   HIP_CHECK_RETURN(api, hipSetDevice(handle->device));

@@ -6,6 +6,7 @@
 #include <string>
 
 #include "core/core.h"
+#include "core/gen_case.h"
 #include "dynamic_point_to_voxel/scatter_points.h"
 
 namespace {
@@ -139,6 +140,20 @@ mluOpStatus_t MLUOP_WIN_API mluOpDynamicPointToVoxelForward(
     return ret;
   }
   if (zero_element) return MLUOP_STATUS_SUCCESS;
+  if (mluop::gen_case::mode() != 0) {
+    // (reference kernels/dynamic_point_to_voxel/dynamic_point_to_voxel_forward/
+    // dynamic_point_to_voxel_forward.cpp:264-279)
+    mluop::gen_case::CaseWriter c(handle, "dynamic_point_to_voxel_forward", "dynamic_point_to_voxel_forward_param");
+    c.input("feats", feats_desc, feats);
+    c.input("coors", coors_desc, coors);
+    c.output("voxel_feats", voxel_feats_desc);
+    c.output("voxel_coors", voxel_coors_desc);
+    c.output("point2voxel_map", point2voxel_map_desc);
+    c.output("voxel_points_count", voxel_points_count_desc);
+    c.output("voxel_num", voxel_num_desc);
+    c.paramName("reduce_type", reduce_type == MLUOP_REDUCE_DMAX ? "REDUCE_MODE_MAX" : "REDUCE_MODE_MEAN");
+    c.finish(0.003);
+  }
   DEVICE_HANDLE_CHECK(api, handle);
   HIP_CHECK_RETURN(api, hipSetDevice(handle->device));
 

@@ -2,6 +2,7 @@
 // reference's status conventions (kernels/voxelization/voxelization.cpp:55-172),
 // then the kernel set of voxelize.hip.
 #include "core/core.h"
+#include "core/gen_case.h"
 #include "voxelization/voxelize.h"
 
 namespace {
@@ -181,6 +182,22 @@ mluOpStatus_t MLUOP_WIN_API mluOpVoxelization(
   PARAM_CHECK(api, coors != NULL);
   PARAM_CHECK(api, num_points_per_voxel != NULL);
   PARAM_CHECK(api, voxel_num != NULL);
+  if (mluop::gen_case::mode() != 0) {
+    // as the reference's call site lists them (kernels/voxelization/voxelization.cpp:269-284)
+    mluop::gen_case::CaseWriter c(handle, "voxelization", "voxelization_param");
+    c.input("points", points_desc, points);
+    c.input("voxel_size", voxel_size_desc, voxel_size);
+    c.input("coors_range", coors_range_desc, coors_range);
+    c.output("voxels", voxels_desc);
+    c.output("coors", coors_desc);
+    c.output("num_points_per_voxel", num_points_per_voxel_desc);
+    c.output("voxel_num", voxel_num_desc);
+    c.param("max_points", max_points);
+    c.param("max_voxels", max_voxels);
+    c.param("ndim", NDim);
+    c.param("deterministic", deterministic ? 1 : 0);
+    c.finish(0.0);
+  }
   DEVICE_HANDLE_CHECK(api, handle);
   HIP_CHECK_RETURN(api, hipSetDevice(handle->device));
 

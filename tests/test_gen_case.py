@@ -105,6 +105,13 @@ WITH_DATA = textwrap.dedent("""
     m.indice_conv_forward(h, x, w, m.LAYOUT_ARRAY, pairs, num_host, n_out, True)
     m.indice_conv_backward_data(h, dy, w, m.LAYOUT_ARRAY, pairs, num_host, True, 16)
     m.indice_conv_backward_filter(h, x, dy, pairs, num_host, (3, 3, 3), True)
+    pts = torch.rand(500, 4, device="cuda") * torch.tensor([4.0, 4.0, 2.0, 1.0], device="cuda")
+    m.voxelization(h, pts, torch.tensor([0.5, 0.5, 0.5], device="cuda"),
+                   torch.tensor([0.0, 0.0, 0.0, 4.0, 4.0, 2.0], device="cuda"), 6, 100)
+    feats = torch.randn(400, 5, device="cuda")
+    coors = torch.randint(0, 6, (400, 3), device="cuda", dtype=torch.int32)
+    vf, vc, p2v, cnt, vn = m.dynamic_point_to_voxel_forward(h, feats, coors, "max")
+    m.dynamic_point_to_voxel_backward(h, torch.randn_like(vf), feats, vf, p2v, cnt, vn, reduce_type="max")
     torch.cuda.synchronize()
 """)
 
@@ -117,10 +124,12 @@ def test_dumped_cases_with_values_replay_through_the_library(tmp_path, gpu_handl
     assert r.returncode == 0, r.stderr
     files = sorted(glob.glob(str(tmp_path / "*" / "*.prototxt")))
     ops = [os.path.basename(os.path.dirname(f)) for f in files]
-    assert ops == ["get_indice_pairs", "indice_convolution_backward_data", "indice_convolution_backward_filter",
-                   "indice_convolution_forward"]
+    assert ops == ["dynamic_point_to_voxel_backward", "dynamic_point_to_voxel_forward", "get_indice_pairs",
+                   "indice_convolution_backward_data", "indice_convolution_backward_filter",
+                   "indice_convolution_forward", "voxelization"]
     for f in files:
         node, _ = casefile.load(f)
-        assert node.all("input")[0].has("value_i") or node.all("input")[0].has("value_h")
+        first = node.all("input")[0]
+        assert first.has("value_i") or first.has("value_h")
         res = casefile.replay(f, gpu_handle)      # inputs from the file, outputs graded against the CPU oracle
         assert res.passed, (f, res.errors)
