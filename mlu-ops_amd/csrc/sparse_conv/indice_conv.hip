@@ -1193,7 +1193,11 @@ __global__ __launch_bounds__(64 * kDenseWaves) __attribute__((amdgpu_waves_per_e
   constexpr int FRAGS = NB * KB;             // 1 KiB filter fragments per offset
   constexpr int W_BYTES = FRAGS * 1024;
   constexpr int FPW = (FRAGS + WAVES - 1) / WAVES;
-  constexpr int POOL = 2 * W_BYTES;
+  // Offsets multiplied between two barriers: two where a filter is 4 KiB at most (a wave then
+  // has little to multiply per offset, and the second set of rows fits the registers): 16 and
+  // 32 column layers 7 % faster; at 64 x 64 the rows of two offsets spill.
+  constexpr int OPP = W_BYTES <= 4096 ? 2 : 1;
+  constexpr int POOL = 2 * OPP * W_BYTES;
   static_assert((Q % E::kChunk == 0 || (KB == 1 && Q % E::kVec == 0)) && C % 16 == 0,
                 "whole fragments, or part of a single one");
   static_assert(G >= 1 && G <= 4, "one code path per set of row groups");
@@ -1399,37 +1403,50 @@ __global__ __launch_bounds__(64 * kDenseWaves) __attribute__((amdgpu_waves_per_e
     // Waits for everything this wave has requested.  The rows pass through an empty
     // statement that the compiler must take for their last writer: it then places its own
     // wait for their loads here, where it costs nothing, and not in front of their first
-    // use, behind the requests for the offset after, which it would wait for as well.
-    auto landed = [&](vec8 (&rows)[G][KB]) {
+    // use, behind the requests for the offsets after, which it would wait for as well.
+    auto landed = [&](vec8 (&rows)[OPP][G][KB]) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-      for (int g = 0; g < G; ++g)
+      for (int o = 0; o < OPP; ++o)
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) asm volatile("" : "+v"(rows[g][kb]));
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) asm volatile("" : "+v"(rows[o][g][kb]));
     };
-    // Offset `item` with the rows in `cur`, while the rows and the filter of the next one
-    // travel.  Everything requested here has landed when the barrier is passed, and every
-    // wave has left the buffer that the offset after the next will be written to.
-    auto phase = [&](int item, int present, const vec8 (&cur)[G][KB], vec8 (&nxt)[G][KB]) -> int {
-      int present_next = 0;
-      if (item + 1 < items) {
-        present_next = load_rows(item + 1, nxt);
-        request_filter(item + 1, (item + 1) & 1);
+    // requests rows and filters of the OPP offsets from `item` on into `rows` and LDS buffer
+    // `buffer`; an offset past the last one repeats the last (its rows are not multiplied)
+    auto request_phase = [&](int item, int buffer, vec8 (&rows)[OPP][G][KB], int (&present)[OPP]) {
+#pragma unroll
+      for (int o = 0; o < OPP; ++o) {
+        const bool there = item + o < items;
+        const int it = there ? item + o : items - 1;
+        const int got = load_rows(it, rows[o]);
+        present[o] = there ? got : 0;
+        request_filter(it, buffer * OPP + o);
       }
-      multiply_present(present, cur, s_w + (item & 1) * W_BYTES);
+    };
+    // The OPP offsets from `item` on with the rows in `cur`, while the rows and the filters of
+    // the next ones travel.  Everything requested here has landed when the barrier is
+    // passed, and every wave has left the buffers that the phase after the next writes to.
+    auto phase = [&](int item, const int (&present)[OPP], const vec8 (&cur)[OPP][G][KB],
+                     vec8 (&nxt)[OPP][G][KB], int (&present_next)[OPP]) {
+      const int buffer = (item / OPP) & 1;
+      if (item + OPP < items) request_phase(item + OPP, buffer ^ 1, nxt, present_next);
+#pragma unroll
+      for (int o = 0; o < OPP; ++o)
+        multiply_present(present[o], cur[o], s_w + (buffer * OPP + o) * W_BYTES);
       landed(nxt);
       ldsBarrier();
-      return present_next;
     };
 
-    vec8 rows_a[G][KB], rows_b[G][KB];
-    int present = load_rows(0, rows_a);
-    request_filter(0, 0);
+    vec8 rows_a[OPP][G][KB], rows_b[OPP][G][KB];
+    int present_a[OPP], present_b[OPP];
+    request_phase(0, 0, rows_a, present_a);
     landed(rows_a);
     ldsBarrier();
-    for (int i = 0; i < items; i += 2) {
-      present = phase(i, present, rows_a, rows_b);
-      if (i + 1 < items) present = phase(i + 1, present, rows_b, rows_a);
+    for (int i = 0; i < items; i += 2 * OPP) {
+      phase(i, present_a, rows_a, rows_b, present_b);
+      if (i + OPP < items) phase(i + OPP, present_b, rows_b, rows_a, present_a);
     }
   }
   // lane holds result columns 16*nb + 4*quad + (0..3) of row 16*g + pair of its wave's rows
