@@ -11,14 +11,16 @@
 // offset, pairs are listed by ascending input row; unused tails are -1.
 //
 // Kernel set
-//   submanifold:  clear hash -> insert rows (and set every pair slot to -1) ->
-//                 probe + compact: a workgroup of 256 rows resolves its pairs,
-//                 learns how many pairs earlier rows hold at every offset by
-//                 looking back over the workgroups before it, and writes its
-//                 pairs at their final positions
-//   regular:      clear bitmap, pair slots to -1 -> mark output cells + compact
-//                 (output cell in place of the output row) -> bitmap popcount
-//                 scan (ranks, out_indices) -> cells to ranks in place
+//   submanifold:  prepare (copy out_indices, clear the hash table, write the sorted-cell
+//                 arrays and decide whether the rows are in strict cell order) -> insert
+//                 rows into the hash table (returns at once for rows in order) -> probe
+//                 (rows in order: search the sorted cells, offsets below the centre only
+//                 where the kernel is centred; otherwise: the hash table), every wave of
+//                 64 rows staging the pairs it found -> place: sums the staged counts in
+//                 front of each wave and moves the pairs to their final positions
+//   regular:      clear bitmap -> mark output cells + stage (output cell in place of the
+//                 output row) -> bitmap popcount scan (ranks, out_indices) -> place, cells
+//                 to ranks
 // The stable order needs no sort: rows are visited in ascending order by
 // construction (lane = row) and positions come from exclusive prefix sums.
 #include <hip/hip_runtime.h>
@@ -130,10 +132,16 @@ __device__ __forceinline__ void noteRowOrder(const int32_t *indices, int j, int4
   if (j > 0 && !coordBelow(loadCoord(indices, j - 1, aligned), c)) *rows_in_order = 0;
 }
 
-// The rulebook's report to the host: the flag first, then the stamp the host looks for.
-__device__ __forceinline__ void fileReport(const int32_t *rows_in_order, const RulebookReportTarget &report) {
+// The rulebook's report: the flag first, then the stamp the reader looks for.  One copy goes
+// to device memory (read by later kernels of the stream), one to pinned host memory (read by
+// the host without waiting for anything).
+__device__ __forceinline__ void fileReport(bool rows_in_order, const RulebookReportTarget &report) {
+  if (report.device_words != nullptr) {
+    report.device_words[1] = rows_in_order ? 1ull : 0ull;
+    report.device_words[0] = report.stamp;
+  }
   if (report.stamp_word == nullptr) return;
-  *report.order_word = *rows_in_order != 0 ? 1u : 0u;
+  *report.order_word = rows_in_order ? 1u : 0u;
   __threadfence_system();
   __hip_atomic_store(report.stamp_word, report.stamp, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
@@ -165,25 +173,95 @@ __global__ __launch_bounds__(kBlock) void rbFill(FillRanges r, int32_t *rows_in_
   }
 }
 
-// Open-addressing table over linear cell indices: keys[] holds the cell (or
-// kEmptyKey), vals[] the highest row index stored for that cell.  32-bit
-// atomics only: a 64-bit compare-and-swap costs several times more here.
+// Rows that arrive in strict cell order (every coordinate inside the space, every row's
+// linear cell above its predecessor's) need no table: the array of their cells is sorted, a
+// cell's place in it is the row that sits there, and looking a neighbour up is a search.
+// What the searching kernel reads:
+//   cells[i]    the linear cell of row i, then 0xffffffff up to the array's capacity
+//   samples[s]  cells[s << shift], then 0xffffffff up to n_pad (a power of two that the
+//               searching workgroup keeps in LDS: the search's first steps cost no memory
+//               round trip, the last `shift` steps walk 2^shift consecutive cells)
+//   unordered   a 64-bit word that holds this call's stamp (a value no earlier call wrote)
+//               when the rows are NOT in strict cell order: nothing needs clearing first
+struct SortedCells {
+  uint32_t *cells;
+  uint32_t *samples;
+  unsigned long long *unordered;
+  unsigned long long stamp;
+  int capacity;  // entries of cells[]
+  int shift;
+  int n_pad;     // entries of samples[]
+  // kernel edges odd and padding = dilation * (edge - 1) / 2: offset K - 1 - k mirrors k
+  bool mirror;
+  int mirror_groups_per_slice;  // groups of offsets a blockIdx.y slice of the probe takes then
+};
+constexpr int kMaxSamples = 4096;
+
+__device__ __forceinline__ bool rowsUnordered(const SortedCells &sc) { return *sc.unordered == sc.stamp; }
+
+// First launch of a submanifold rulebook: clears the hash table (needed only when the rows
+// turn out unordered, which no launch knows before this one has finished), copies the
+// coordinates to out_indices, writes the sorted-cell arrays and decides whether they may be
+// used.
+__global__ __launch_bounds__(kBlock) void rbSubmPrepare(GeomDev g, const int32_t *indices, bool aligned,
+                                                        int32_t *out_indices, int out_rows,
+                                                        FillRanges table, SortedCells sc,
+                                                        bool never_sorted) {
+  const size_t n_threads = (size_t)gridDim.x * kBlock;
+  const size_t tid = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  {
+    uint4 *d4 = reinterpret_cast<uint4 *>(table.dst[0]);  // capacity is a multiple of 64
+    const size_t n4 = table.n[0] / 4;
+    const uint32_t v = table.value[0];
+    for (size_t t = tid; t < n4; t += n_threads) d4[t] = make_uint4(v, v, v, v);
+  }
+  if (never_sorted) {
+    if (tid == 0) *sc.unordered = sc.stamp;
+  } else {
+    const int n_real = (g.L + (1 << sc.shift) - 1) >> sc.shift;
+    for (size_t t = tid; t < (size_t)sc.n_pad; t += n_threads)
+      if ((int)t >= n_real) sc.samples[t] = kEmptyKey;
+  }
+  const int j = (int)tid;
+  if (j < g.L) {
+    const int4 c = loadCoord(indices, j, aligned);
+    if (j < out_rows) storeCoord(out_indices, j, c, aligned);
+    if (!never_sorted) {
+      const bool in_range = (unsigned)c.x < (unsigned)g.batch && (unsigned)c.y < (unsigned)g.out[0] &&
+                            (unsigned)c.z < (unsigned)g.out[1] && (unsigned)c.w < (unsigned)g.out[2];
+      const uint32_t cell =
+          in_range ? (uint32_t)(((c.x * g.out[0] + c.y) * g.out[1] + c.z) * g.out[2] + c.w) : kEmptyKey;
+      bool bad = !in_range;
+      if (j > 0 && !coordBelow(loadCoord(indices, j - 1, aligned), c)) bad = true;
+      if (bad) *sc.unordered = sc.stamp;
+      sc.cells[j] = cell;
+      if ((j & ((1 << sc.shift) - 1)) == 0) sc.samples[j >> sc.shift] = cell;
+    }
+  } else {
+    if (j < out_rows) storeCoord(out_indices, j, make_int4(-1, -1, -1, -1), aligned);
+    if (!never_sorted && j < sc.capacity) sc.cells[j] = kEmptyKey;
+  }
+}
+
+// Open-addressing table over linear cell indices, for rows in any order: keys[] holds the
+// cell (or kEmptyKey), vals[] the highest row index stored for that cell.  32-bit atomics
+// only: a 64-bit compare-and-swap costs several times more here.  Returns at once when the
+// rows are in cell order.
 __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t *indices,
                                                        bool aligned, uint32_t *keys,
                                                        int32_t *vals, uint32_t mask,
-                                                       int32_t *out_indices, int out_rows,
-                                                       int32_t *rows_in_order, int32_t *pairs) {
+                                                       SortedCells sc, int32_t *pairs) {
+  if (!rowsUnordered(sc)) return;
   int j = blockIdx.x * kBlock + threadIdx.x;
   if (j < g.L) {
-    // Every pair slot starts as -1; the probe kernel overwrites the slots in front of each
-    // offset's pair count.  Plain stores that nobody waits for, under the table's atomics.
+    // Every pair slot starts as -1; the kernel that places the pairs overwrites the slots in
+    // front of each offset's pair count.  Plain stores that nobody waits for, under the
+    // table's atomics.
     for (int k = 0; k < g.K; ++k) {
       pairs[(size_t)k * 2 * g.L + j] = -1;
       pairs[((size_t)k * 2 + 1) * g.L + j] = -1;
     }
     int4 c = loadCoord(indices, j, aligned);
-    noteRowOrder(indices, j, c, aligned, rows_in_order);
-    if (j < out_rows) storeCoord(out_indices, j, c, aligned);
     bool in_range = (unsigned)c.x < (unsigned)g.batch && (unsigned)c.y < (unsigned)g.out[0] &&
                     (unsigned)c.z < (unsigned)g.out[1] && (unsigned)c.w < (unsigned)g.out[2];
     if (in_range) {
@@ -199,43 +277,57 @@ __global__ __launch_bounds__(kBlock) void rbSubmInsert(GeomDev g, const int32_t 
         slot = (slot + 1) & mask;
       }
     }
-  } else if (j < out_rows) {
-    storeCoord(out_indices, j, make_int4(-1, -1, -1, -1), aligned);
   }
 }
 
 // ---- pairs to their final positions -----------------------------------------------
 //
 // A pair's position inside its offset is the number of pairs earlier rows hold there.
-// The probe kernels do not know it yet; a wave (64 consecutive rows) stages the pairs it
-// found at offset k compactly at the start of its own 64 slots of stage[k][.] and writes
-// their number to counts[k][wave], so that what crosses the kernel boundary is the pairs
-// (a few per wave and offset) and not a slot for every (row, offset).  rbPlacePairs then
-// moves them: a workgroup adds up the counts in front of its 256 waves, scans its own, and
-// copies the staged pairs to their final positions.
+// The probe kernels do not know it yet.  A wave (64 consecutive rows) resolving a slice of
+// the offsets (blockIdx.y) owns one block of the staging buffer and stages the pairs it
+// found there back to back, offset after offset, each offset's pairs in lane order:
+// what crosses the kernel boundary is the pairs (a few per wave and offset) and not a slot
+// for every (row, offset), and the block's lines are written whole (a slot array per
+// offset with a few words used per wave left every line partly written, which the memory
+// behind the cache turns into read-modify-write; that layout spent as long on staging as
+// on probing).  counts[k][wave] gets the number of pairs of (offset, wave) in its low 8
+// bits and their start inside the block above them.  rbPlacePairs then moves them: a
+// workgroup adds up the counts in front of its 64 waves, scans its own, and copies the
+// staged pairs to their final positions.
 // (Looking back over earlier workgroups inside the probe kernel instead, single-pass-scan
 // style, was built and measured: all workgroups finish probing at the same moment, so
 // the look-back degenerates into a chain over hundreds of workgroups per offset; 400 us.)
 struct Staging {
-  int32_t *stage;       // [K, L]: submanifold: output row << 6 | lane; regular: output cell
-  uint8_t *stage_lane;  // [K, L], regular mode only: lane of the staged pair
-  int32_t *counts;      // [K, n_wave]
+  int32_t *stage;       // blocks of block_ints: submanifold: output row << 6 | lane; regular: output cell
+  uint8_t *stage_lane;  // same blocks, regular mode only: lane of the staged pair
+  int32_t *counts;      // [K, n_wave]: pairs | start in the block << 8
   int n_wave;
+  int k_per_slice;      // offsets per blockIdx.y slice
+  int block_ints;       // k_per_slice * 64
+  int mirror_k_per_slice;  // offsets per slice where only the offsets below the centre are probed
 };
 
+__device__ __forceinline__ size_t stageBlock(const Staging &st, int slice, int wave) {
+  return ((size_t)slice * st.n_wave + wave) * (size_t)st.block_ints;
+}
+
+// Stages the pairs of offsets k_first .. k_first + N - 1 (those below k_end); `run` is the
+// number of pairs the wave has staged in its block so far (the same in every lane).
 template <bool SUBM, int N>
-__device__ __forceinline__ void stagePairs(const int (&res)[N], int k_first, int k_end, int j, int L,
-                                           const Staging &st) {
+__device__ __forceinline__ void stagePairs(const int (&res)[N], int k_first, int k_end, int j,
+                                           const Staging &st, int *run) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wt = j >> 6;
   const unsigned long long lt_mask = (1ull << lane) - 1ull;
+  const size_t block = stageBlock(st, blockIdx.y, wt);
+  int my_entry = 0;  // lane u keeps the count word of offset k_first + u
 #pragma unroll
   for (int u = 0; u < N; ++u) {
     const int k = k_first + u;
     if (k < k_end) {
       const unsigned long long b = __ballot(res[u] >= 0);
       if (res[u] >= 0) {
-        const size_t at = (size_t)k * L + (size_t)wt * kWave + __popcll(b & lt_mask);
+        const size_t at = block + (size_t)(*run + __popcll(b & lt_mask));
         if (SUBM) {
           st.stage[at] = (res[u] << 6) | lane;
         } else {
@@ -243,9 +335,12 @@ __device__ __forceinline__ void stagePairs(const int (&res)[N], int k_first, int
           st.stage_lane[at] = (uint8_t)lane;
         }
       }
-      if (lane == 0) st.counts[(size_t)k * st.n_wave + wt] = __popcll(b);
+      const int n = __popcll(b);
+      if (lane == u) my_entry = n | (*run << 8);
+      *run += n;
     }
   }
+  if (lane < N && k_first + lane < k_end) st.counts[(size_t)(k_first + lane) * st.n_wave + wt] = my_entry;
 }
 
 // One wavefront per 64 consecutive rows, offsets in groups of kGroup so that a
@@ -280,6 +375,7 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g,
   // kd changes, once in ks[2] offsets.
   int base_d = 0, plane = -1;
   bool new_d = true, new_h = true;
+  int staged = 0;
   for (int k0 = k_lo; k0 < k_hi; k0 += kGroup) {
     uint32_t cell[kGroup];
     int res[kGroup];
@@ -402,24 +498,252 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g,
         }
       }
     }
-    stagePairs<SUBM, kGroup>(res, k0, k_hi, j, g.L, staging);
+    stagePairs<SUBM, kGroup>(res, k0, k_hi, j, staging, &staged);
   }
 }
 
-// Submanifold probe for unit strides (the usual case), kernel edges <= 32 and
-// K <= kMaxInlineOffsets.  With stride 1 the output cell of (row, offset) is the
-// row's own padded cell minus a per-offset constant, and whether it lies inside
-// the output space is one bit per axis and kernel position, computed once per
-// row: the per-offset work shrinks to a few integer instructions around the
-// probe itself.
+// Offsets of a unit-stride kernel volume (at most kMaxInlineOffsets of them, kernel edges
+// <= 32).  With stride 1 the output cell of (row, offset) is the row's own padded cell
+// minus a per-offset constant, and whether it lies inside the output space is one bit per
+// axis and kernel position, computed once per row.
 struct UnitStrideOffsets {
   uint32_t packed[kMaxInlineOffsets];  // kd | kh << 8 | kw << 16
   uint32_t delta[kMaxInlineOffsets];   // linear distance from the padded cell
 };
 
+// Number of elements below t in a sorted array of n elements (n a power of two >= 4),
+// three pivots a step; at(i) reads element i.
+template <typename F>
+__device__ __forceinline__ int countBelow(F at, int n, uint32_t t) {
+  int base = 0;
+  int len = n;
+  while (len >= 4) {
+    const int q = len >> 2;
+    const uint32_t p1 = at(base + q - 1);
+    const uint32_t p2 = at(base + 2 * q - 1);
+    const uint32_t p3 = at(base + 3 * q - 1);
+    base += ((p1 < t ? 1 : 0) + (p2 < t ? 1 : 0) + (p3 < t ? 1 : 0)) * q;
+    len = q;
+  }
+  if (len == 2) base += at(base) < t ? 1 : 0;
+  return base + (at(base) < t ? 1 : 0);
+}
+
+// Probe over the sorted cell array (rows in strict cell order, unit strides).  Offsets are
+// taken in groups of KW consecutive ones that look at KW consecutive cells (KW = the kernel's
+// width along W at dilation 1, or 1: every offset its own group), G groups a pass.
+//
+// The lowest cells that the 64 rows of a wave look for in one group ascend with the rows, so
+// everything the wave can find lies between the places of its first and its last row's
+// cell.  Two lanes per group search these two among the samples in LDS (one search for all
+// groups of the pass), the wave copies the kSpan cells from there on to LDS with a few
+// coalesced loads, and every lane finishes its own search inside that copy: no memory
+// round trip per search step and a tenth of the instructions of a search per lane over the
+// whole array.  A wave whose rows are spread so thin that its span is longer falls back to
+// exactly that: per lane over the samples, then with three pivots a step over the 2^shift
+// cells between two samples down to a stretch of kChunk cells, which is read in one go.
+// Either way the cells found that belong to the group are the neighbours that exist, and
+// their places are their rows.
+//
+// With `mirror` (kernel edges odd, padding = dilation * (edge - 1) / 2) only the offsets
+// below the centre are probed: row o found from row i at offset k finds i at offset
+// K - 1 - k, and since o ascends with i the list of K - 1 - k is the list of k with its
+// columns exchanged; the centre offset pairs every row with itself.
+//
+// The wave also sets the pair slots of its rows to -1 for the offsets it resolves (and
+// their mirror images), stores that nobody waits for; the kernel that places the pairs
+// overwrites the front of each list afterwards.
+constexpr int kChunk = 8;
+constexpr int kSpan = 256;
+constexpr int kSpanPad = 8;
+struct CellQuad {
+  uint32_t v[4];
+};
+
+template <int KW, int G>
+__device__ __forceinline__ void sortedProbe(const GeomDev &g, const UnitStrideOffsets &tab,
+                                            const int32_t *indices, bool aligned, const SortedCells &sc,
+                                            const Staging &staging, int groups_per_slice, int32_t *pairs) {
+  constexpr int N = G * KW;
+  constexpr int QUADS = (kChunk + KW + 3) / 4;
+  static_assert(N <= 32 && 2 * G <= kWave && KW <= kSpanPad, "bit masks, lanes, padding");
+  __shared__ uint32_t s_samples[kMaxSamples];
+  __shared__ uint32_t s_span[kBlock / kWave][G][kSpan + kSpanPad];
+  if ((sc.n_pad & 1023) == 0) {
+    for (int i = threadIdx.x; i < sc.n_pad / 4; i += kBlock)
+      reinterpret_cast<uint4 *>(s_samples)[i] = reinterpret_cast<const uint4 *>(sc.samples)[i];
+  } else {
+    for (int i = threadIdx.x; i < sc.n_pad; i += kBlock) s_samples[i] = sc.samples[i];
+  }
+  const int j = blockIdx.x * kBlock + threadIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wv = threadIdx.x >> 6;
+  // offsets below k_all are probed, in groups [t_lo, t_hi) by this slice
+  const int k_all = sc.mirror ? g.K / 2 : g.K;
+  const int n_groups = (k_all + KW - 1) / KW;
+  const int per_slice = sc.mirror ? sc.mirror_groups_per_slice : groups_per_slice;
+  const int t_lo = blockIdx.y * per_slice;
+  const int t_hi = t_lo + per_slice < n_groups ? t_lo + per_slice : n_groups;
+  const int k_end = KW * t_hi < k_all ? KW * t_hi : k_all;
+  const bool active = j < g.L;
+  int4 c = make_int4(0, 0, 0, 0);
+  if (active) {
+    c = loadCoord(indices, j, aligned);
+    for (int k = KW * t_lo; k < k_end; ++k) {
+      pairs[(size_t)(2 * k) * g.L + j] = -1;
+      pairs[(size_t)(2 * k + 1) * g.L + j] = -1;
+      if (sc.mirror) {
+        pairs[(size_t)(2 * (g.K - 1 - k)) * g.L + j] = -1;
+        pairs[(size_t)(2 * (g.K - 1 - k) + 1) * g.L + j] = -1;
+      }
+    }
+  }
+  __syncthreads();
+  if ((j >> 6) >= staging.n_wave || t_lo >= t_hi) return;  // nothing for this wave
+  uint32_t ok_d = 0, ok_h = 0, ok_w = 0;
+  for (int t = 0; t < g.ks[0]; ++t)
+    ok_d |= (uint32_t)((unsigned)(c.y + g.pad[0] - t * g.dil[0]) < (unsigned)g.out[0]) << t;
+  for (int t = 0; t < g.ks[1]; ++t)
+    ok_h |= (uint32_t)((unsigned)(c.z + g.pad[1] - t * g.dil[1]) < (unsigned)g.out[1]) << t;
+  for (int t = 0; t < g.ks[2]; ++t)
+    ok_w |= (uint32_t)((unsigned)(c.w + g.pad[2] - t * g.dil[2]) < (unsigned)g.out[2]) << t;
+  if (!active) ok_d = 0;
+  const uint32_t padded = (((uint32_t)c.x * g.out[0] + (uint32_t)(c.y + g.pad[0])) * g.out[1] +
+                           (uint32_t)(c.z + g.pad[1])) * g.out[2] + (uint32_t)(c.w + g.pad[2]);
+  const uint32_t *cells = sc.cells;
+  auto sample = [&](int i) { return s_samples[i]; };
+  int staged = 0;
+  for (int t0 = t_lo; t0 < t_hi; t0 += G) {
+    uint32_t low[G];     // lowest cell of the group (modulo 2^32: it may lie below cell 0)
+    uint32_t target[G];  // what is searched for: the lowest cell, or cell 0
+    uint32_t want = 0;
+    int res[N];
+    unsigned long long wanting[G];  // lanes that look for something in the group
+#pragma unroll
+    for (int a = 0; a < G; ++a) {
+      const int t = t0 + a < t_hi ? t0 + a : t_hi - 1;  // clamped: a valid table entry
+      low[a] = padded - tab.delta[KW * t + KW - 1];
+#pragma unroll
+      for (int d = 0; d < KW; ++d) {
+        const int u = KW * a + (KW - 1 - d);
+        const int k = KW * t + (KW - 1 - d);
+        const uint32_t pk = tab.packed[k];
+        res[u] = -1;
+        if (t0 + a < t_hi && k < k_end &&
+            ((ok_d >> (pk & 0xff)) & (ok_h >> ((pk >> 8) & 0xff)) & (ok_w >> (pk >> 16)) & 1u))
+          want |= 1u << u;
+      }
+      const bool any = ((want >> (KW * a)) & ((1u << KW) - 1u)) != 0;
+      target[a] = any && (int32_t)low[a] >= 0 ? low[a] : 0u;
+      wanting[a] = __ballot(any);
+    }
+    // where the wave's span of every group starts, and whether kSpan cells cover it
+    int start[G];
+    bool fits = true;
+    {
+      uint32_t bound = 0;
+#pragma unroll
+      for (int a = 0; a < G; ++a) {
+        const int l_first = wanting[a] ? __ffsll((long long)wanting[a]) - 1 : 0;
+        const int l_last = wanting[a] ? 63 - __clzll((long long)wanting[a]) : 0;
+        const uint32_t t_first = (uint32_t)__builtin_amdgcn_readlane((int)target[a], l_first);
+        const uint32_t t_last = (uint32_t)__builtin_amdgcn_readlane((int)target[a], l_last);
+        if (lane == 2 * a) bound = t_first;
+        if (lane == 2 * a + 1) bound = t_last;
+      }
+      const int below = countBelow(sample, sc.n_pad, bound);
+      // the first cell >= bound lies in (sample below - 1 .. sample below] << shift
+      const int from = (below - 1) * (1 << sc.shift) + 1;
+      const int edge = (lane & 1) ? below << sc.shift : (from > 0 ? from : 0);
+#pragma unroll
+      for (int a = 0; a < G; ++a) {
+        start[a] = __builtin_amdgcn_readlane(edge, 2 * a);
+        const int last = __builtin_amdgcn_readlane(edge, 2 * a + 1);
+        if (wanting[a] != 0 && last - start[a] > kSpan) fits = false;
+      }
+    }
+    if (fits) {
+#pragma unroll
+      for (int a = 0; a < G; ++a) {
+        if (wanting[a] == 0) continue;
+        uint32_t piece[kSpan / kWave], extra = 0;
+#pragma unroll
+        for (int i = 0; i < kSpan / kWave; ++i) piece[i] = cells[start[a] + i * kWave + lane];
+        if (lane < kSpanPad) extra = cells[start[a] + kSpan + lane];
+#pragma unroll
+        for (int i = 0; i < kSpan / kWave; ++i) s_span[wv][a][i * kWave + lane] = piece[i];
+        if (lane < kSpanPad) s_span[wv][a][kSpan + lane] = extra;
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int a = 0; a < G; ++a) {
+        if (wanting[a] == 0) continue;
+        const uint32_t *span = s_span[wv][a];
+        const int at = countBelow([&](int i) { return span[i]; }, kSpan, target[a]);
+#pragma unroll
+        for (int i = 0; i < KW; ++i) {
+          const uint32_t rel = span[at + i] - low[a];
+#pragma unroll
+          for (int d = 0; d < KW; ++d) {
+            const int u = KW * a + (KW - 1 - d);
+            if (rel == (uint32_t)d && (want & (1u << u))) res[u] = start[a] + at + i;
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    } else {
+#pragma unroll
+      for (int a = 0; a < G; ++a) {
+        if (wanting[a] == 0) continue;
+        const int below = countBelow(sample, sc.n_pad, target[a]);
+        const int from = (below - 1) * (1 << sc.shift) + 1;
+        int first = from > 0 ? from : 0;
+        int len = 1 << sc.shift;
+        while (len > kChunk) {
+          if (len >= 4 * kChunk) {
+            const int q = len >> 2;
+            const uint32_t p1 = cells[first + q - 1];
+            const uint32_t p2 = cells[first + 2 * q - 1];
+            const uint32_t p3 = cells[first + 3 * q - 1];
+            first += ((p1 < target[a] ? 1 : 0) + (p2 < target[a] ? 1 : 0) + (p3 < target[a] ? 1 : 0)) * q;
+            len = q;
+          } else {
+            const int half = len >> 1;
+            first += cells[first + half - 1] < target[a] ? half : 0;
+            len = half;
+          }
+        }
+        // the first cell >= target is one of first .. first + kChunk
+        CellQuad found[QUADS];
+#pragma unroll
+        for (int i = 0; i < QUADS; ++i) found[i] = *reinterpret_cast<const CellQuad *>(cells + first + 4 * i);
+#pragma unroll
+        for (int i = 0; i < 4 * QUADS; ++i) {
+          const uint32_t rel = found[i >> 2].v[i & 3] - low[a];
+#pragma unroll
+          for (int d = 0; d < KW; ++d) {
+            const int u = KW * a + (KW - 1 - d);
+            if (rel == (uint32_t)d && (want & (1u << u))) res[u] = first + i;
+          }
+        }
+      }
+    }
+    stagePairs<true, N>(res, KW * t0, k_end, j, staging, &staged);
+  }
+}
+
+// Submanifold probe for unit strides (the usual case), kernel edges <= 32 and
+// K <= kMaxInlineOffsets: over the sorted cells when the rows came in cell order, through
+// the hash table otherwise (the per-offset work is a few integer instructions around the
+// probe itself).
 __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
     GeomDev g, UnitStrideOffsets tab, const int32_t *indices, bool aligned, const uint32_t *keys,
-    const int32_t *vals, uint32_t mask, Staging staging, int k_per_slice) {
+    const int32_t *vals, uint32_t mask, Staging staging, int k_per_slice, SortedCells sc,
+    int32_t *pairs) {
+  if (!rowsUnordered(sc)) {
+    sortedProbe<1, 4>(g, tab, indices, aligned, sc, staging, k_per_slice, pairs);
+    return;
+  }
   const int j = blockIdx.x * kBlock + threadIdx.x;
   const int k_lo = blockIdx.y * k_per_slice;
   const int k_hi = k_lo + k_per_slice < g.K ? k_lo + k_per_slice : g.K;
@@ -440,6 +764,7 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
   // modulo 2^32; exact for every cell inside the output space
   const uint32_t padded = (((uint32_t)c.x * g.out[0] + (uint32_t)(c.y + g.pad[0])) * g.out[1] +
                            (uint32_t)(c.z + g.pad[1])) * g.out[2] + (uint32_t)(c.w + g.pad[2]);
+  int staged = 0;
   for (int k0 = k_lo; k0 < k_hi; k0 += kGroup) {
     uint32_t cell[kGroup], slot[kGroup];
     int res[kGroup];
@@ -482,7 +807,7 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeUnitStride(
     for (int u = 0; u < kGroup; ++u) {
       if (hit & (1u << u)) res[u] = vals[slot[u]];
     }
-    stagePairs<true, kGroup>(res, k0, k_hi, j, g.L, staging);
+    stagePairs<true, kGroup>(res, k0, k_hi, j, staging, &staged);
   }
 }
 
@@ -505,9 +830,14 @@ constexpr int kGroupsPerPass = 3;  // (kd, kh) pairs resolved together per lane
 template <int KW>
 __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
     GeomDev g, UnitStrideOffsets tab, const int32_t *indices, bool aligned, const uint32_t *keys,
-    const int32_t *vals, uint32_t mask, Staging staging, int groups_per_slice) {
+    const int32_t *vals, uint32_t mask, Staging staging, int groups_per_slice, SortedCells sc,
+    int32_t *pairs) {
   constexpr int N = kGroupsPerPass * KW;
   static_assert(KW <= kWindow && N <= 32, "window and bit masks");
+  if (!rowsUnordered(sc)) {
+    sortedProbe<KW, KW == 3 ? 2 : 3>(g, tab, indices, aligned, sc, staging, groups_per_slice, pairs);
+    return;
+  }
   const int j = blockIdx.x * kBlock + threadIdx.x;
   const int n_groups = g.K / KW;
   const int t_lo = blockIdx.y * groups_per_slice;
@@ -528,6 +858,7 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
   if (!n_ok) ok_d = 0;
   const uint32_t padded = (((uint32_t)c.x * g.out[0] + (uint32_t)(c.y + g.pad[0])) * g.out[1] +
                            (uint32_t)(c.z + g.pad[1])) * g.out[2] + (uint32_t)(c.w + g.pad[2]);
+  int staged = 0;
   for (int t0 = t_lo; t0 < t_hi; t0 += kGroupsPerPass) {
     uint32_t cell[N], slot[N];
     int res[N];
@@ -635,7 +966,7 @@ __global__ __launch_bounds__(kBlock) void rbSubmProbeRuns(
     for (int u = 0; u < N; ++u) {
       if (hit & (1u << u)) res[u] = vals[slot[u]];
     }
-    stagePairs<true, N>(res, KW * t0, KW * t_hi, j, g.L, staging);
+    stagePairs<true, N>(res, KW * t0, KW * t_hi, j, staging, &staged);
   }
 }
 
@@ -790,67 +1121,122 @@ __global__ __launch_bounds__(kBlock) void rbRankAndDecode(GeomDev g,
 // final positions: the pairs in front of the chunk are the sum of the earlier waves'
 // counts (a few kilobytes, read by every workgroup of the offset rather than scanned in a
 // launch of its own), wave 0 scans the chunk's own counts, and every wave of the
-// workgroup copies a quarter of the chunk's staged pieces, one piece per step, a lane per
-// pair.  In regular mode the staged output cell becomes the output row, its rank among
-// the marked cells.  One thread also files the rulebook's report.
+// workgroup copies four of the chunk's staged pieces, a lane per pair, all four in flight
+// at once.  In regular mode the staged output cell becomes the output row, its rank among
+// the marked cells.  One thread files the rulebook's report.
 constexpr int kPlaceWaves = 64;
+constexpr int kPlaceBlock = 1024;
 template <bool SUBM>
-__global__ __launch_bounds__(kBlock) void rbPlacePairs(int L, Staging st,
-                                                        const unsigned long long *bitmap,
-                                                        const uint32_t *word_rank, int32_t *pairs,
-                                                        int32_t *indice_num,
-                                                        const int32_t *rows_in_order,
-                                                        RulebookReportTarget report) {
+__global__ __launch_bounds__(kPlaceBlock) void rbPlacePairs(int L, Staging st,
+                                                             const unsigned long long *bitmap,
+                                                             const uint32_t *word_rank, int32_t *pairs,
+                                                             int32_t *indice_num,
+                                                             const int32_t *rows_in_order,
+                                                             const unsigned long long *unordered,
+                                                             bool mirror_geometry,
+                                                             RulebookReportTarget report) {
   static_assert(kPlaceWaves == kWave, "one lane per wave count in the scan");
+  constexpr int kWaves = kPlaceBlock / kWave;
+  constexpr int kPieces = kPlaceWaves / kWaves;  // staged pieces per wave
   __shared__ int s_first[kPlaceWaves];  // staged pairs in front of each wave of the chunk
   __shared__ int s_count[kPlaceWaves];
-  __shared__ int s_wave_sum[kBlock / kWave];
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) fileReport(rows_in_order, report);
+  __shared__ int s_start[kPlaceWaves];  // where the wave's pairs start in its staging block
+  __shared__ int s_wave_sum[kWaves];
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+    // submanifold: the rows were in cell order unless the word holds the call's stamp
+    fileReport(SUBM ? *unordered != report.stamp : *rows_in_order != 0, report);
+  }
   const int k = blockIdx.y;
   const int w0 = blockIdx.x * kPlaceWaves;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
+  // Submanifold rows in cell order with a centred kernel: the probe resolved the offsets
+  // below the centre only; offset K - 1 - k gets k's pairs with the columns exchanged and
+  // the centre pairs every row with itself.
+  const bool mirror = SUBM && mirror_geometry && *unordered != report.stamp;
+  int32_t *mirror_in = nullptr, *mirror_out = nullptr;
+  if (mirror) {
+    const int K = gridDim.y;
+    if (k > K / 2) return;
+    if (k == K / 2) {
+      int32_t *in_col = pairs + (size_t)k * 2 * L;
+      const int hi = (w0 + kPlaceWaves) * kWave < L ? (w0 + kPlaceWaves) * kWave : L;
+      for (int r = w0 * kWave + tid; r < hi; r += kPlaceBlock) {
+        in_col[r] = r;
+        in_col[L + r] = r;
+      }
+      if (blockIdx.x == 0 && tid == 0) indice_num[k] = L;
+      return;
+    }
+    mirror_in = pairs + (size_t)(K - 1 - k) * 2 * L;
+    mirror_out = mirror_in + L;
+  }
+  const int slice = k / (mirror ? st.mirror_k_per_slice : st.k_per_slice);
   const int32_t *counts = st.counts + (size_t)k * st.n_wave;
   // pairs of the waves in front of the chunk
   int part = 0;
-  for (int i = tid; i < w0; i += kBlock) part += counts[i];
+  for (int i = tid; i < w0; i += kPlaceBlock) part += counts[i] & 0xff;
   part = waveInclusiveScan(part);
   if (lane == kWave - 1) s_wave_sum[wave] = part;
   if (wave == 0) {
-    const int mine = w0 + lane < st.n_wave ? counts[w0 + lane] : 0;
+    const int entry = w0 + lane < st.n_wave ? counts[w0 + lane] : 0;
+    const int mine = entry & 0xff;
     const int incl = waveInclusiveScan(mine);
     s_count[lane] = mine;
+    s_start[lane] = entry >> 8;
     s_first[lane] = incl - mine;
   }
   __syncthreads();
   int before = 0;
 #pragma unroll
-  for (int w = 0; w < kBlock / kWave; ++w) before += s_wave_sum[w];
-  if (blockIdx.x == gridDim.x - 1 && tid == 0)
-    indice_num[k] = before + s_first[kPlaceWaves - 1] + s_count[kPlaceWaves - 1];
+  for (int w = 0; w < kWaves; ++w) before += s_wave_sum[w];
+  if (blockIdx.x == gridDim.x - 1 && tid == 0) {
+    const int total = before + s_first[kPlaceWaves - 1] + s_count[kPlaceWaves - 1];
+    indice_num[k] = total;
+    if (mirror) indice_num[gridDim.y - 1 - k] = total;
+  }
   int32_t *in_col = pairs + (size_t)k * 2 * L;
   int32_t *out_col = in_col + L;
-  constexpr int kPieces = kPlaceWaves / (kBlock / kWave);  // staged pieces per wave
-#pragma unroll 4
+  int v[kPieces], from_lane[kPieces];
+#pragma unroll
+  for (int i = 0; i < kPieces; ++i) {
+    const int seg = wave * kPieces + i;
+    v[i] = from_lane[i] = 0;
+    if (lane < s_count[seg]) {
+      const size_t at = stageBlock(st, slice, w0 + seg) + (size_t)(s_start[seg] + lane);
+      v[i] = st.stage[at];
+      if (!SUBM) from_lane[i] = (int)st.stage_lane[at];
+    }
+  }
+  int out[kPieces];
+  if (!SUBM) {
+    unsigned long long word[kPieces];
+    uint32_t rank[kPieces];
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      const bool live = lane < s_count[wave * kPieces + i];
+      word[i] = live ? bitmap[v[i] >> 6] : 0ull;
+      rank[i] = live ? word_rank[v[i] >> 6] : 0u;
+    }
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i)
+      out[i] = (int)(rank[i] + (uint32_t)__popcll(word[i] & ((1ull << (v[i] & 63)) - 1ull)));
+  }
+#pragma unroll
   for (int i = 0; i < kPieces; ++i) {
     const int seg = wave * kPieces + i;
     if (lane < s_count[seg]) {
       const int first_row = (w0 + seg) * kWave;
-      const size_t at = (size_t)k * L + (size_t)first_row + lane;
-      const int v = st.stage[at];
-      int row, out;
-      if (SUBM) {
-        row = first_row + (v & 63);
-        out = v >> 6;
-      } else {
-        row = first_row + (int)st.stage_lane[at];
-        const unsigned long long below = bitmap[v >> 6] & ((1ull << (v & 63)) - 1ull);
-        out = (int)(word_rank[v >> 6] + (uint32_t)__popcll(below));
-      }
       const int to = before + s_first[seg] + lane;
+      const int row = first_row + (SUBM ? (v[i] & 63) : from_lane[i]);
+      const int partner = SUBM ? v[i] >> 6 : out[i];
       in_col[to] = row;
-      out_col[to] = out;
+      out_col[to] = partner;
+      if (mirror) {
+        mirror_in[to] = partner;
+        mirror_out[to] = row;
+      }
     }
   }
 }
@@ -888,7 +1274,14 @@ struct Workspace {
   uint8_t *stage_lane = nullptr;     // [K, L], regular mode only
   int32_t *counts = nullptr;         // [K, n_wave]
   int n_wave = 0;
-  int32_t *rows_in_order = nullptr;  // 1 until a kernel finds two rows out of cell order
+  int32_t *rows_in_order = nullptr;  // regular: 1 until a kernel finds two rows out of cell order
+  // submanifold: the sorted-cell arrays and the word that says they cannot be used
+  uint32_t *cells = nullptr;
+  uint32_t *samples = nullptr;
+  unsigned long long *unordered = nullptr;
+  int cells_capacity = 0;
+  int sample_shift = 0;
+  int n_samples_pad = 0;
   size_t bytes = 0;
 };
 
@@ -908,6 +1301,16 @@ Workspace carve(const RulebookGeom &g, void *base) {
     ws.table_cap = tableCapacity(g.L);
     ws.keys = reinterpret_cast<uint32_t *>(take((size_t)ws.table_cap * 8));
     ws.vals = ws.keys ? reinterpret_cast<int32_t *>(ws.keys + ws.table_cap) : nullptr;
+    // one sample every 2^shift rows, at most kMaxSamples of them
+    while (((g.L + (1 << ws.sample_shift) - 1) >> ws.sample_shift) > kMaxSamples) ++ws.sample_shift;
+    const int n_real = (g.L + (1 << ws.sample_shift) - 1) >> ws.sample_shift;
+    ws.n_samples_pad = 64;
+    while (ws.n_samples_pad < n_real) ws.n_samples_pad <<= 1;
+    // a wave's span starts at (n_real << shift) + 1 at most and is read kSpan + kSpanPad cells far
+    ws.cells_capacity = ((n_real << ws.sample_shift) + kSpan + kSpanPad + 4 + 3) / 4 * 4;
+    ws.cells = reinterpret_cast<uint32_t *>(take((size_t)ws.cells_capacity * 4));
+    ws.samples = reinterpret_cast<uint32_t *>(take((size_t)ws.n_samples_pad * 4));
+    ws.unordered = reinterpret_cast<unsigned long long *>(take(8));
   } else {
     const size_t cells = (size_t)g.batch * g.out_space[0] * g.out_space[1] * g.out_space[2];
     ws.n_words = (cells + 63) / 64;
@@ -919,8 +1322,10 @@ Workspace carve(const RulebookGeom &g, void *base) {
     ws.num_act_out = reinterpret_cast<int32_t *>(take(4));
 
   }
-  ws.stage = reinterpret_cast<int32_t *>(take((size_t)g.K * g.L * 4));
-  if (!g.sub_m) ws.stage_lane = reinterpret_cast<uint8_t *>(take((size_t)g.K * g.L));
+  // one block of 64 slots per (offset, wave); slices of the offsets round the offsets up
+  const size_t stage_slots = (size_t)(g.K + 32) * ws.n_wave * kWave;
+  ws.stage = reinterpret_cast<int32_t *>(take(stage_slots * 4));
+  if (!g.sub_m) ws.stage_lane = reinterpret_cast<uint8_t *>(take(stage_slots));
   ws.counts = reinterpret_cast<int32_t *>(take((size_t)g.K * ws.n_wave * 4));
   ws.rows_in_order = reinterpret_cast<int32_t *>(take(4));
   ws.bytes = off + 256;
@@ -975,29 +1380,39 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
   const GeomDev d = toDev(g);
   const bool al = aligned16(indices, out_indices);
   const uint32_t mask = ws.table_cap - 1;
-  const int rows = g.L > g.out_rows ? g.L : g.out_rows;
-  const int row_blocks = (rows + kBlock - 1) / kBlock;
   const int l_blocks = (g.L + kBlock - 1) / kBlock;
+  const bool unit_stride = g.stride[0] == 1 && g.stride[1] == 1 && g.stride[2] == 1 &&
+                           g.ksize[0] <= 32 && g.ksize[1] <= 32 && g.ksize[2] <= 32 &&
+                           g.K <= kMaxInlineOffsets;
+  bool mirror = unit_stride;
+  for (int a = 0; a < 3; ++a)
+    if (g.ksize[a] % 2 == 0 || 2 * g.pad[a] != g.dilation[a] * (g.ksize[a] - 1)) mirror = false;
+  SortedCells sc = {ws.cells, ws.samples, ws.unordered, report.stamp,
+                    ws.cells_capacity, ws.sample_shift, ws.n_samples_pad, mirror, 0};
 
   // cells become kEmptyKey and rows -1 with the same all-ones pattern
   FillRanges fill = {};
   fill.dst[0] = ws.keys;
   fill.n[0] = (size_t)ws.table_cap * 2;
   fill.value[0] = kEmptyKey;
-  lc.begin("rbFill");
-  rbFill<<<fillBlocks((size_t)ws.table_cap / 2), kBlock, 0, lc.stream>>>(fill, ws.rows_in_order);
+  int rows = g.L > g.out_rows ? g.L : g.out_rows;
+  if (ws.cells_capacity > rows) rows = ws.cells_capacity;
+  lc.begin("rbSubmPrepare");
+  rbSubmPrepare<<<(rows + kBlock - 1) / kBlock, kBlock, 0, lc.stream>>>(
+      d, indices, al, out_indices, g.out_rows, fill, sc, !unit_stride);
   lc.end();
   lc.begin("rbSubmInsert");
-  rbSubmInsert<<<row_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.keys, ws.vals, mask,
-                                                     out_indices, g.out_rows, ws.rows_in_order,
-                                                     indice_pairs);
+  rbSubmInsert<<<l_blocks, kBlock, 0, lc.stream>>>(d, indices, al, ws.keys, ws.vals, mask, sc, indice_pairs);
   lc.end();
-  const Staging staging = {ws.stage, nullptr, ws.counts, ws.n_wave};
   const int k_per = offsetsPerSlice(g.K);
+  Staging staging = {ws.stage, nullptr, ws.counts, ws.n_wave, k_per, k_per * kWave, 0};
+  // groups of `width` offsets below the centre, spread over `slices` slices
+  auto mirrorSlices = [&](int width, int slices) {
+    const int groups = (g.K / 2 + width - 1) / width;
+    sc.mirror_groups_per_slice = (groups + slices - 1) / slices;
+    staging.mirror_k_per_slice = sc.mirror_groups_per_slice * width;
+  };
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
-  const bool unit_stride = g.stride[0] == 1 && g.stride[1] == 1 && g.stride[2] == 1 &&
-                           g.ksize[0] <= 32 && g.ksize[1] <= 32 && g.ksize[2] <= 32 &&
-                           g.K <= kMaxInlineOffsets;
   if (unit_stride) {
     UnitStrideOffsets ut;
     int k = 0;
@@ -1015,30 +1430,34 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
       const int n_groups = g.K / g.ksize[2];
       const int t_per = n_groups > 4 * kGroupsPerPass ? 2 * kGroupsPerPass : kGroupsPerPass;
       const dim3 grid(l_blocks, (n_groups + t_per - 1) / t_per);
+      staging.k_per_slice = t_per * g.ksize[2];
+      staging.block_ints = staging.k_per_slice * kWave;
+      mirrorSlices(g.ksize[2], (int)grid.y);
       lc.begin("rbSubmProbeRuns");
       if (g.ksize[2] == 3)
         rbSubmProbeRuns<3><<<grid, kBlock, 0, lc.stream>>>(d, ut, indices, al, ws.keys, ws.vals, mask,
-                                                           staging, t_per);
+                                                           staging, t_per, sc, indice_pairs);
       else
         rbSubmProbeRuns<5><<<grid, kBlock, 0, lc.stream>>>(d, ut, indices, al, ws.keys, ws.vals, mask,
-                                                           staging, t_per);
+                                                           staging, t_per, sc, indice_pairs);
       lc.end();
     } else {
+      mirrorSlices(1, (int)slice_grid.y);
       lc.begin("rbSubmProbeUnitStride");
       rbSubmProbeUnitStride<<<slice_grid, kBlock, 0, lc.stream>>>(d, ut, indices, al, ws.keys, ws.vals,
-                                                                  mask, staging, k_per);
+                                                                  mask, staging, k_per, sc, indice_pairs);
       lc.end();
     }
   } else {
     lc.begin("rbProbeCount");
     rbProbeCount<true><<<slice_grid, kBlock, 0, lc.stream>>>(d, indices, al, ws.keys, ws.vals,
                                                              mask, nullptr, staging, k_per,
-                                                             ws.rows_in_order, nullptr);
+                                                             nullptr, nullptr);
     lc.end();
   }
   lc.begin("rbPlacePairs");
-  rbPlacePairs<true><<<dim3((ws.n_wave + kPlaceWaves - 1) / kPlaceWaves, g.K), kBlock, 0, lc.stream>>>(
-      g.L, staging, nullptr, nullptr, indice_pairs, indice_num, ws.rows_in_order, report);
+  rbPlacePairs<true><<<dim3((ws.n_wave + kPlaceWaves - 1) / kPlaceWaves, g.K), kPlaceBlock, 0, lc.stream>>>(
+      g.L, staging, nullptr, nullptr, indice_pairs, indice_num, nullptr, ws.unordered, mirror, report);
   lc.end();
   return hipGetLastError();
 }
@@ -1062,9 +1481,9 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
   rbFill<<<fillBlocks((ws.bitmap_fill_words + fill.n[1]) / 4 + 1), kBlock, 0, lc.stream>>>(
       fill, ws.rows_in_order);
   lc.end();
-  const Staging staging = {ws.stage, ws.stage_lane, ws.counts, ws.n_wave};
-  lc.begin("rbProbeCount");
   const int k_per = offsetsPerSlice(g.K);
+  const Staging staging = {ws.stage, ws.stage_lane, ws.counts, ws.n_wave, k_per, k_per * kWave, 0};
+  lc.begin("rbProbeCount");
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
   rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, indices, al_in, nullptr,
                                                             nullptr, 0, ws.bitmap, staging, k_per,
@@ -1088,8 +1507,8 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                   hipMemcpyDeviceToHost, lc.stream);
   if (err != hipSuccess) return err;
   lc.begin("rbPlacePairs");
-  rbPlacePairs<false><<<dim3((ws.n_wave + kPlaceWaves - 1) / kPlaceWaves, g.K), kBlock, 0, lc.stream>>>(
-      g.L, staging, ws.bitmap, ws.word_rank, indice_pairs, indice_num, ws.rows_in_order, report);
+  rbPlacePairs<false><<<dim3((ws.n_wave + kPlaceWaves - 1) / kPlaceWaves, g.K), kPlaceBlock, 0, lc.stream>>>(
+      g.L, staging, ws.bitmap, ws.word_rank, indice_pairs, indice_num, ws.rows_in_order, nullptr, false, report);
   lc.end();
   return hipGetLastError();
 }

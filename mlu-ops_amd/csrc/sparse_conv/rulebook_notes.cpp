@@ -20,9 +20,18 @@ RulebookReportTarget openRulebookNote(mluOpContext *handle, const void *pairs, i
   handle->rulebook_reports[slot].stamp = 0;
   handle->rulebook_reports[slot].rows_in_order = 0;
   RulebookReportTarget t;
-  t.stamp_word = &handle->rulebook_reports[slot].stamp;
-  t.order_word = &handle->rulebook_reports[slot].rows_in_order;
   t.stamp = note.stamp;
+  if (handle->device_reports != nullptr) t.device_words = handle->device_reports + 2 * slot;
+  // A captured rulebook files no report in host memory: nothing runs now, so no report of
+  // this call could arrive, and a replay must not write into a slot that by then belongs to
+  // another rulebook (or to a handle that is gone).  The device copy is written on every
+  // replay, under the stamp taken here.
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(handle->queue, &capturing) != hipSuccess) (void)hipGetLastError();
+  if (capturing == hipStreamCaptureStatusNone) {
+    t.stamp_word = &handle->rulebook_reports[slot].stamp;
+    t.order_word = &handle->rulebook_reports[slot].rows_in_order;
+  }
   return t;
 }
 
