@@ -33,9 +33,17 @@ typedef enum {
   MLUOP_EXT_KERNEL_FLAT_SCATTER = 4,   /* row maps built on a flat grid */
   MLUOP_EXT_KERNEL_SMALL_MAP_CHUNKS = 5, /* 1: row maps cover 2048 result rows at a time instead of
                                             as many as 64 MiB hold (runs the chunked path on small inputs) */
-  MLUOP_EXT_KERNEL_FILTER_STORES = 6    /* 1: backward filter transposes its operands with element-sized
+  MLUOP_EXT_KERNEL_FILTER_STORES = 6,   /* 1: backward filter transposes its operands with element-sized
                                            LDS stores also for 2-byte types of 32 to 128 channels, where
                                            transposing LDS reads are the default */
+  MLUOP_EXT_KERNEL_LISTS_ON_TRUST = 7   /* forward on a rulebook of this handle whose report (were the input
+                                           rows in cell order?) has not reached the host yet, as under graph
+                                           capture or without any wait between the two calls.  -1: start on
+                                           the pair lists and enqueue the row-map kernels behind them; the
+                                           first kernel's check decides on the device which of the two do the
+                                           work, the others return at once.  0: build the row map.  1: a test
+                                           switch: the pair lists only; a call whose lists fail the check
+                                           leaves its output as it was */
 } mluOpExtKernelChoice_t;
 
 mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelChoice(mluOpHandle_t handle,

@@ -77,18 +77,6 @@ mluOpStatus_t MLUOP_WIN_API mluOpCreate(mluOpHandle_t *handle) {
   memset(pinned, 0, pinned_bytes);
   ctx->rulebook_reports =
       reinterpret_cast<mluOpContext::RulebookReport *>(static_cast<char *>(pinned) + 64);
-  void *device_reports = nullptr;
-  const size_t device_report_bytes = 2 * sizeof(unsigned long long) * mluOpContext::kRulebookNotes;
-  err = hipMalloc(&device_reports, device_report_bytes);
-  if (err == hipSuccess) err = hipMemset(device_reports, 0, device_report_bytes);
-  if (err != hipSuccess) {
-    MLUOP_LOG(ERROR) << "[mluOpCreate] hipMalloc of the report slots failed: " << hipGetErrorString(err);
-    if (device_reports != nullptr) (void)hipFree(device_reports);
-    (void)hipHostFree(pinned);
-    delete ctx;
-    return MLUOP_STATUS_ALLOC_FAILED;
-  }
-  ctx->device_reports = static_cast<unsigned long long *>(device_reports);
   // Stamps and tickets only have to differ from what earlier calls, of this handle or of
   // another, left in memory: start somewhere no other handle starts.
   ctx->next_stamp = ((unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count()
@@ -117,7 +105,6 @@ mluOpStatus_t MLUOP_WIN_API mluOpDestroy(mluOpHandle_t handle) {
     if (capturing == hipStreamCaptureStatusNone && hipStreamSynchronize(handle->queue) != hipSuccess)
       (void)hipGetLastError();
   }
-  if (handle->device_reports != nullptr) (void)hipFree(handle->device_reports);
   if (handle->pinned_scalar != nullptr) (void)hipHostFree(handle->pinned_scalar);
   handle->timer.destroy();
   delete handle;
@@ -199,6 +186,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtSetKernelChoice(mluOpHandle_t handle,
     case MLUOP_EXT_KERNEL_FLAT_SCATTER: c.flat_scatter = value; break;
     case MLUOP_EXT_KERNEL_SMALL_MAP_CHUNKS: c.small_map_chunks = value; break;
     case MLUOP_EXT_KERNEL_FILTER_STORES: c.filter_stores = value; break;
+    case MLUOP_EXT_KERNEL_LISTS_ON_TRUST: c.lists_on_trust = value; break;
     default:
       MLUOP_LOG(ERROR) << "[mluOpExtSetKernelChoice] unknown kernel choice " << as_int;
       return MLUOP_STATUS_BAD_PARAM;

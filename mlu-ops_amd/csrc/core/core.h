@@ -69,9 +69,6 @@ struct mluOpContext {
   static constexpr int kRulebookNotes = 32;
   RulebookNote rulebook_notes[kRulebookNotes];
   RulebookReport *rulebook_reports = nullptr;  // kRulebookNotes slots behind pinned_scalar
-  // The same reports in device memory, two 64-bit words a slot (stamp, flag): what a
-  // convolution enqueued before the pinned copy can have arrived lets its kernels read.
-  unsigned long long *device_reports = nullptr;
   int next_rulebook_note = 0;
   unsigned long long next_stamp = 1;   // also the source of per-call tickets
 

@@ -57,6 +57,7 @@ struct KernelChoices {
   int flat_scatter = -1;    // 1: row maps built on the flat grid
   int small_map_chunks = -1;  // 1: row maps cover 2048 result rows at a time (the chunked path, on small inputs)
   int filter_stores = -1;   // 1: backward filter transposes with element-sized LDS stores also where transposing reads serve
+  int lists_on_trust = -1;  // pair lists of unreported order: -1 lists with the row-map kernels behind, 0 row map, 1 lists only
 };
 
 class LaunchCtx {

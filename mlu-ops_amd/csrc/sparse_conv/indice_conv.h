@@ -27,6 +27,13 @@ struct FilterView {
   int64_t stride_co;
 };
 
+// What the caller knows about the pair column that names a launch's result rows.
+enum class ListTrust {
+  kNone,     // nothing, or that it is out of order: the launch builds a row map
+  kInOrder,  // it ascends inside every offset (checked again on the device)
+  kUnknown,  // a rulebook of this handle whose report has not arrived: the kernels decide
+};
+
 struct ConvProblem {
   ElemType dtype;
   int K;          // kernel volume = indice_pairs.dim[0]
@@ -50,7 +57,7 @@ struct ConvProblem {
   // device) that inside every offset the pair column naming the result rows ascends strictly
   // and all indices are in range, so the kernels read the lists cut by tile instead of
   // building a row map.  `ticket` is a value no earlier launch on this workspace used.
-  bool lists_in_order = false;
+  ListTrust list_trust = ListTrust::kNone;
   unsigned long long ticket = 0;
   // Backward filter only: element strides of dW(k, ci, co) in filters_grad;
   // all zero = the positional [K, Ci, Co].

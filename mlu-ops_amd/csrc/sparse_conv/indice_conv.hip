@@ -124,6 +124,16 @@ struct FloatElem {
 
 // ---- row map ---------------------------------------------------------------
 
+// A launch that is enqueued before anyone knows whether it is needed: it runs when `word` is
+// null or holds `value`, and returns at once otherwise.  The row-map kernels of a forward
+// call that started on the pair lists without knowing whether they are in order carry the
+// verdict word and the call's ticket here.
+struct RunIf {
+  const unsigned long long *word;
+  unsigned long long value;
+};
+__device__ __forceinline__ bool notWanted(const RunIf &r) { return r.word != nullptr && *r.word != r.value; }
+
 __global__ __launch_bounds__(256) void fillInt32(int32_t *dst, size_t n, int32_t value) {
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * 256;
@@ -147,7 +157,8 @@ __global__ __launch_bounds__(256) void scatterRowMap(const int32_t *pairs, int L
                                                      OffsetCounts inl, const int32_t *dev_counts,
                                                      int row_col, int src_col, int row_base,
                                                      int n_rows, int n_src, int32_t *map,
-                                                     int32_t *accepted) {
+                                                     int32_t *accepted, RunIf run_if) {
+  if (notWanted(run_if)) return;
   const int k = blockIdx.y;
   const int n = offsetCount(inl, dev_counts, k);
   const int32_t *base = pairs + (size_t)k * 2 * L;
@@ -181,7 +192,8 @@ __global__ __launch_bounds__(256) void scatterRowMapFlat(const int32_t *pairs, i
                                                          OffsetCounts inl, OffsetBlocks blocks,
                                                          int K, int row_col, int src_col,
                                                          int row_base, int n_rows, int n_src,
-                                                         int32_t *map, int32_t *accepted) {
+                                                         int32_t *map, int32_t *accepted, RunIf run_if) {
+  if (notWanted(run_if)) return;
   // last offset whose first workgroup is not behind this one (an offset without
   // pairs shares its prefix with the next one and is never chosen)
   int lo = 0, hi = K - 1;
@@ -289,7 +301,9 @@ __global__ __launch_bounds__(256) void fillMapPackFilter(int32_t *map, size_t ma
                                                          int fill_blocks,
                                                          const typename E::storage *W, int64_t sK,
                                                          int64_t sQ, int64_t sC, int K, int Q,
-                                                         int C, typename E::storage *packed) {
+                                                         int C, typename E::storage *packed,
+                                                         RunIf run_if) {
+  if (notWanted(run_if)) return;
   if ((int)blockIdx.x < fill_blocks) {
     const size_t quads = map_elems / 4;
     int4 *dst = reinterpret_cast<int4 *>(map);
@@ -334,6 +348,7 @@ struct MapSource {
   static constexpr bool kSegments = false;
   const int32_t *map;
   int32_t *filled;
+  RunIf run_if;
 };
 
 struct SegmentSource {
@@ -342,6 +357,9 @@ struct SegmentSource {
   const int32_t *cuts;                // [K, cut_stride]: first pair of every tile, then the count
   const unsigned long long *verdict;  // holds `ticket` when some list is not in order
   unsigned long long ticket;
+  // Lists out of order: true = the kernel returns at once (row-map kernels enqueued behind
+  // it do the call's work), false = every tile collects its pairs by reading all of them.
+  bool leave_if_unordered;
   int L, row_col, src_col, n_src, cut_stride;
   const void *W;                      // the filter as the caller passed it, for lists out of order
   int64_t sK, sQ, sC;
@@ -601,6 +619,9 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   const int tiles_per_xcd = gridDim.x >> 3;
   const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
   const int r0 = tile * TR;
+  if constexpr (!SRC::kSegments) {
+    if (notWanted(source.run_if)) return;
+  }
   if (r0 >= R) {
     if constexpr (!SRC::kSegments) {
       if (tid == 0 && blockIdx.y == 0) source.filled[blockIdx.x] = 0;
@@ -617,6 +638,7 @@ void gatherConvMfma(const typename E::storage *A, const typename E::storage *pac
   bool in_order = true;
   if constexpr (SRC::kSegments) {
     in_order = *source.verdict != source.ticket;
+    if (!in_order && source.leave_if_unordered) return;
     if (!in_order) {
       __syncthreads();
       scanAllPairsForTile<E, NT>(A, Q, source, K, r0, r0 + TR < R ? r0 + TR : R, C, blockIdx.y * C,
@@ -982,6 +1004,7 @@ __global__ __launch_bounds__(64) void gatherConvWave(
     }
   };
   if (verdict == source.ticket) {
+    if (source.leave_if_unordered) return;
     // lists out of order: every pair of every offset is looked at
     scanAllPairsForTile<E, 64>(A, Q, source, K, r0, r0 + TR < R ? r0 + TR : R, C, 0, s_acc, ACC_STRIDE);
     write_out();
@@ -1215,6 +1238,9 @@ __global__ __launch_bounds__(64 * kDenseWaves) __attribute__((amdgpu_waves_per_e
   const int tiles_per_xcd = gridDim.x >> 3;  // neighbouring tiles on one XCD, as above
   const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
   const int r0 = tile * TR;
+  if constexpr (!SRC::kSegments) {
+    if (notWanted(source.run_if)) return;
+  }
   if (r0 >= R) {
     if constexpr (!SRC::kSegments) {
       if (tid == 0 && blockIdx.y == 0) source.filled[blockIdx.x] = 0;
@@ -1223,6 +1249,7 @@ __global__ __launch_bounds__(64 * kDenseWaves) __attribute__((amdgpu_waves_per_e
   }
   const int col_group = blockIdx.y;
   if constexpr (SRC::kSegments) {
+    if (*source.verdict == source.ticket && source.leave_if_unordered) return;
     if (*source.verdict == source.ticket) {
       // pair lists out of order: fp32 rows where the row map would be, 16 columns at a
       // time, every pair looked at by every workgroup
@@ -1512,7 +1539,8 @@ __global__ __launch_bounds__(256) void repairLostPairs(
     int64_t sC, const int32_t *pairs, int L, int row_col, int src_col, int R, int n_src, int K,
     int row_base, OffsetCounts inl, const int32_t *dev_counts, int32_t *map,
     const int32_t *filled, int n_filled, const int32_t *accepted, int n_accepted, int C,
-    RepairScratch scratch, typename E::storage *result) {
+    RepairScratch scratch, typename E::storage *result, RunIf run_if) {
+  if (notWanted(run_if)) return;
   __shared__ int s_found;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -2381,7 +2409,7 @@ GatherDims gatherDims(const ConvProblem &p, GatherDirection dir) {
 // the call is used instead.
 bool listsUsable(const ConvProblem &p, const GatherDims &d) {
   (void)d;
-  return p.lists_in_order && p.K <= kMaxInlineK && p.row_map == nullptr;
+  return p.list_trust != ListTrust::kNone && p.K <= kMaxInlineK && p.row_map == nullptr;
 }
 
 struct GatherWorkspace {
@@ -2667,7 +2695,7 @@ constexpr int kFlatScatterFromBlocks = 16384;
 int enqueueScatterRowMap(const LaunchCtx &lc, const int32_t *pairs, int L, int K,
                          const OffsetCounts &inl, const int32_t *dev_counts, int max_count,
                          int row_col, int src_col, int row_base, int n_rows, int n_src,
-                         int32_t *map, int32_t *accepted) {
+                         int32_t *map, int32_t *accepted, RunIf run_if) {
   const int gx = (max_count + 255) / 256 > 1024 ? 1024 : (max_count + 255) / 256;
   if (dev_counts == nullptr && K <= kMaxInlineK &&
       (lc.choices.flat_scatter == 1 ||
@@ -2680,22 +2708,23 @@ int enqueueScatterRowMap(const LaunchCtx &lc, const int32_t *pairs, int L, int K
     }
     if (blocks > 0)
       scatterRowMapFlat<<<blocks, 256, 0, lc.stream>>>(pairs, L, inl, ob, K, row_col, src_col,
-                                                   row_base, n_rows, n_src, map, accepted);
+                                                   row_base, n_rows, n_src, map, accepted, run_if);
     return blocks;
   }
   scatterRowMap<<<dim3(gx, K), 256, 0, lc.stream>>>(pairs, L, inl, dev_counts, row_col, src_col,
-                                                 row_base, n_rows, n_src, map, accepted);
+                                                 row_base, n_rows, n_src, map, accepted, run_if);
   return gx * K;
 }
 
 // The map of result rows [row_base, row_base + n_rows); returns the entries of ws.accepted written.
 int launchScatterRowMap(const LaunchCtx &lc, const ConvProblem &p, const GatherDims &d,
                         const GatherWorkspace &ws, const OffsetCounts &inl, int max_count,
-                        int row_base, int n_rows) {
+                        int row_base, int n_rows, RunIf run_if) {
   if (max_count <= 0) return 0;
   lc.begin("scatterRowMap");
   const int n = enqueueScatterRowMap(lc, p.indice_pairs, p.L, p.K, inl, ws.dev_counts, max_count,
-                                     d.row_col, d.src_col, row_base, n_rows, d.n_src, ws.map, ws.accepted);
+                                     d.row_col, d.src_col, row_base, n_rows, d.n_src, ws.map, ws.accepted,
+                                     run_if);
   lc.end();
   return n;
 }
@@ -2708,7 +2737,14 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
   // B(k, q, c): forward q = ci, c = co; backward data q = co, c = ci.
   const int64_t sQ = d.filter_forward ? f.stride_ci : f.stride_co;
   const int64_t sC = d.filter_forward ? f.stride_co : f.stride_ci;
-  if (use_mfma && listsUsable(p, d)) {
+  const bool single_chunk = p.row_map == nullptr && ws.map_rows >= d.R && lc.choices.small_map_chunks != 1;
+  // Pair lists whose order nobody has reported yet: the call starts on them all the same,
+  // and the row-map kernels are enqueued behind, each of them told to return at once unless
+  // the first kernel found the lists out of order (then the list kernel returns at once
+  // instead).  Worth it only where the row map is a single chunk of four launches.
+  const bool speculate = p.list_trust == ListTrust::kUnknown && single_chunk && lc.choices.lists_on_trust != 0;
+  const bool lists = use_mfma && listsUsable(p, d) && (p.list_trust == ListTrust::kInOrder || speculate);
+  if (lists) {
     // Pair lists in order (as far as the caller knows: the first kernel checks): the
     // gather kernel reads them cut by tile, no row map.
     const bool dense = useDenseKernel(lc, p, d);
@@ -2737,6 +2773,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
     src.cuts = ws.cuts;
     src.verdict = ws.verdict;
     src.ticket = p.ticket;
+    src.leave_if_unordered = speculate;
     src.L = p.L;
     src.row_col = d.row_col;
     src.src_col = d.src_col;
@@ -2753,8 +2790,10 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
       launchWave<E>(lc, d.Q, d.C, gathered, ws.packed, src, d.R, p.K, result);
     else
       launchMfma<E, SegmentSource>(lc, d.Q, d.C, tile_cols, gathered, ws.packed, src, d.R, p.K, result);
-    return;
+    if (!speculate || lc.choices.lists_on_trust == 1) return;
   }
+  // What follows runs always, or (behind lists taken on trust) only when they failed the check.
+  const RunIf run_if = lists ? RunIf{ws.verdict, p.ticket} : RunIf{nullptr, 0};
   const bool own_map = p.row_map == nullptr;  // else: built ahead, nothing to clear or fill
   // A map of the library's own covers a chunk of result rows at a time: filled, used by the
   // gather kernel for those rows, checked for lost pairs, and filled again for the next rows.
@@ -2770,19 +2809,20 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
     int n_filled = 0;    // workgroups along x of the gather kernel = slot counts it leaves
     int n_accepted = 0;  // workgroups of the map scatter = counts of pairs it leaves
     if (use_mfma) {
-      // the filter is repacked with the first chunk's map fill
+      // the filter is repacked with the first chunk's map fill (the list kernels' first
+      // launch has done it already where they ran)
       const size_t frags = (size_t)p.K * (d.C / 16) * ((d.Q + E::kChunk - 1) / E::kChunk) * 64;
       const int fill_blocks = own_map ? gridFor(map_elems / 4 + 1, 2048) : 0;
-      const int pack_blocks = row_base == 0 ? gridFor(frags, 512) : 0;
+      const int pack_blocks = row_base == 0 && !lists ? gridFor(frags, 512) : 0;
       if (fill_blocks + pack_blocks > 0) {
         lc.begin("fillMapPackFilter");
         fillMapPackFilter<E><<<fill_blocks + pack_blocks, 256, 0, lc.stream>>>(
             ws.map, map_elems, fill_blocks, static_cast<const S *>(f.base), f.stride_k, sQ, sC, p.K,
-            d.Q, d.C, static_cast<S *>(ws.packed));
+            d.Q, d.C, static_cast<S *>(ws.packed), run_if);
         lc.end();
       }
-      if (own_map) n_accepted = launchScatterRowMap(lc, p, d, ws, inl, max_count, row_base, rows);
-      const MapSource map = {entries, ws.filled};
+      if (own_map) n_accepted = launchScatterRowMap(lc, p, d, ws, inl, max_count, row_base, rows, run_if);
+      const MapSource map = {entries, ws.filled, run_if};
       if (dense) {
         n_filled = denseGridX(rows, d.Q, d.C);
         launchDense<E, MapSource>(lc, d.Q, d.C, gathered, ws.packed, map, rows, p.K, result_rows);
@@ -2795,7 +2835,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
         lc.begin("fillInt32");
         fillInt32<<<gridFor(map_elems), 256, 0, lc.stream>>>(ws.map, map_elems, -1);
         lc.end();
-        n_accepted = launchScatterRowMap(lc, p, d, ws, inl, max_count, row_base, rows);
+        n_accepted = launchScatterRowMap(lc, p, d, ws, inl, max_count, row_base, rows, run_if);
       }
       dim3 grid((rows + 31) / 32, (d.C + 63) / 64);
       n_filled = (int)grid.x;
@@ -2813,7 +2853,7 @@ void launchGatherTyped(const LaunchCtx &lc, const ConvProblem &p, const GatherDi
         static_cast<const S *>(gathered), d.Q, static_cast<const S *>(f.base), f.stride_k, sQ, sC,
         p.indice_pairs, p.L, d.row_col, d.src_col, rows, d.n_src, p.K, row_base, inl, ws.dev_counts,
         ws.map, ws.filled, n_filled, ws.accepted, n_accepted, d.C,
-        RepairScratch{ws.shadow, ws.pool_row, ws.pool}, result_rows);
+        RepairScratch{ws.shadow, ws.pool_row, ws.pool}, result_rows, run_if);
     lc.end();
   }
 }
@@ -3088,7 +3128,7 @@ hipError_t buildRowMap(const LaunchCtx &lc, const int32_t *indice_pairs, const i
     lc.begin("scatterRowMap");
     enqueueScatterRowMap(lc, indice_pairs, shape.L, shape.K, inl,
                          shape.K > kMaxInlineK ? dev_counts : nullptr, max_count, shape.row_column,
-                         1 - shape.row_column, 0, shape.rows, shape.source_rows, map, nullptr);
+                         1 - shape.row_column, 0, shape.rows, shape.source_rows, map, nullptr, RunIf{nullptr, 0});
     lc.end();
   }
   if (filled_host == nullptr) return hipGetLastError();

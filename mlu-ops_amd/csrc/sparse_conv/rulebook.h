@@ -33,9 +33,6 @@ struct RulebookGeom {
 struct RulebookReportTarget {
   unsigned long long *stamp_word = nullptr;
   unsigned int *order_word = nullptr;
-  // The same report in device memory, for kernels enqueued before the host can have seen
-  // the pinned copy: word 0 the stamp, word 1 the flag.  Null: no device copy.
-  unsigned long long *device_words = nullptr;
   // A value no earlier rulebook of any handle used (never 0); also marks this call's words
   // in the workspace, so it is set whether or not a report is wanted.
   unsigned long long stamp = 0;

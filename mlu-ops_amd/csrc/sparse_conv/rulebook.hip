@@ -132,14 +132,8 @@ __device__ __forceinline__ void noteRowOrder(const int32_t *indices, int j, int4
   if (j > 0 && !coordBelow(loadCoord(indices, j - 1, aligned), c)) *rows_in_order = 0;
 }
 
-// The rulebook's report: the flag first, then the stamp the reader looks for.  One copy goes
-// to device memory (read by later kernels of the stream), one to pinned host memory (read by
-// the host without waiting for anything).
+// The rulebook's report to the host: the flag first, then the stamp the host looks for.
 __device__ __forceinline__ void fileReport(bool rows_in_order, const RulebookReportTarget &report) {
-  if (report.device_words != nullptr) {
-    report.device_words[1] = rows_in_order ? 1ull : 0ull;
-    report.device_words[0] = report.stamp;
-  }
   if (report.stamp_word == nullptr) return;
   *report.order_word = rows_in_order ? 1u : 0u;
   __threadfence_system();

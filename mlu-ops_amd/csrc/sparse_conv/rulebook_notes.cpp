@@ -21,11 +21,9 @@ RulebookReportTarget openRulebookNote(mluOpContext *handle, const void *pairs, i
   handle->rulebook_reports[slot].rows_in_order = 0;
   RulebookReportTarget t;
   t.stamp = note.stamp;
-  if (handle->device_reports != nullptr) t.device_words = handle->device_reports + 2 * slot;
   // A captured rulebook files no report in host memory: nothing runs now, so no report of
   // this call could arrive, and a replay must not write into a slot that by then belongs to
-  // another rulebook (or to a handle that is gone).  The device copy is written on every
-  // replay, under the stamp taken here.
+  // another rulebook (or to a handle that is gone).
   hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(handle->queue, &capturing) != hipSuccess) (void)hipGetLastError();
   if (capturing == hipStreamCaptureStatusNone) {
@@ -37,18 +35,22 @@ RulebookReportTarget openRulebookNote(mluOpContext *handle, const void *pairs, i
 
 void consultRulebookNotes(mluOpContext *handle, int row_column, ConvProblem *p) {
   p->ticket = handle->next_stamp++;
-  p->lists_in_order = false;
+  p->list_trust = ListTrust::kNone;
   if (handle->rulebook_reports == nullptr) return;
   for (int slot = 0; slot < mluOpContext::kRulebookNotes; ++slot) {
     const mluOpContext::RulebookNote &note = handle->rulebook_notes[slot];
     if (note.pairs != p->indice_pairs || note.K != p->K || note.L != p->L) continue;
     if (row_column == 0) {
-      p->lists_in_order = true;
+      p->list_trust = ListTrust::kInOrder;
       return;
     }
     const volatile mluOpContext::RulebookReport *report = &handle->rulebook_reports[slot];
-    if (__atomic_load_n(&report->stamp, __ATOMIC_ACQUIRE) != note.stamp) return;
-    p->lists_in_order = report->rows_in_order != 0;
+    if (__atomic_load_n(&report->stamp, __ATOMIC_ACQUIRE) != note.stamp) {
+      // not arrived (or never sent: a captured rulebook files none)
+      p->list_trust = ListTrust::kUnknown;
+      return;
+    }
+    p->list_trust = report->rows_in_order != 0 ? ListTrust::kInOrder : ListTrust::kNone;
     return;
   }
 }

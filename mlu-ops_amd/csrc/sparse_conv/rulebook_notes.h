@@ -13,10 +13,10 @@ namespace sparse_conv {
 // kernel reports to.
 RulebookReportTarget openRulebookNote(mluOpContext *handle, const void *pairs, int K, int L);
 
-// Sets p->lists_in_order and p->ticket for a forward / backward-data launch whose result rows
+// Sets p->list_trust and p->ticket for a forward / backward-data launch whose result rows
 // are named by pair column `row_column`.  Column 0 of a rulebook this handle built ascends by
 // construction; column 1 does when the report says the input rows were in cell order.  A
-// report that has not arrived yet counts as "no".
+// report that has not arrived yet leaves the question to the kernels.
 void consultRulebookNotes(mluOpContext *handle, int row_column, ConvProblem *p);
 
 }  // namespace sparse_conv

@@ -192,7 +192,8 @@ class Handle:
         check(lib().mluOpExtSetKernelTiming(self.ptr, 1 if enable else 0))
 
     KERNEL_CHOICES = {"gather_simt": 0, "dense_tiles": 1, "wave_per_tile": 2, "flat_slice_sum": 3,
-                      "flat_scatter": 4, "small_map_chunks": 5, "filter_stores": 6}   # mluOpExtKernelChoice_t
+                      "flat_scatter": 4, "small_map_chunks": 5, "filter_stores": 6,
+                      "lists_on_trust": 7}   # mluOpExtKernelChoice_t
 
     def set_kernel_choice(self, which, value):
         """mluOpExtSetKernelChoice: value None (the shape decides), False or True."""

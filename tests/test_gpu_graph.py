@@ -10,12 +10,13 @@ from spconv_cases import random_voxels
 pytestmark = pytest.mark.gpu
 
 
-def test_captured_step_replays_bit_exactly():
+@pytest.mark.parametrize("rows_in_order", [False, True])
+def test_captured_step_replays_bit_exactly(rows_in_order):
     import torch
     import mluop_hip as m
     rng = np.random.default_rng(31)
     batch, space, L, ci, co, ks = 2, (12, 24, 24), 5000, 64, 64, (3, 3, 3)
-    idx = torch.from_numpy(random_voxels(rng, batch, space, L)).cuda()
+    idx = torch.from_numpy(random_voxels(rng, batch, space, L, shuffle=not rows_in_order)).cuda()
     feats = torch.from_numpy(rng.standard_normal((L, ci)).astype(np.float32)).cuda().half()
     w = torch.from_numpy((rng.standard_normal(ks + (ci, co)) * 0.1).astype(np.float32)).cuda().half()
     dy = torch.from_numpy(rng.standard_normal((L, co)).astype(np.float32)).cuda().half()
@@ -40,9 +41,17 @@ def test_captured_step_replays_bit_exactly():
         eager = [t.clone() for t in step(num_host)]
         side.synchronize()
 
+        # Nothing runs during capture, so the captured forward cannot know whether the rows are
+        # in order: list kernels and row-map kernels are both captured, and every replay decides
+        # on the device which of them do the work.  For rows in order the test switch leaves the
+        # row-map kernels out of the graph, so a replay that reproduces the eager bits shows that
+        # the list kernels did the work; the shuffled rows need the row-map kernels.
+        if rows_in_order:
+            handle.set_kernel_choice("lists_on_trust", True)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=side):
             captured = step(num_host)
+        handle.set_kernel_choice("lists_on_trust", None)
         for replay in range(4):
             for t in captured:
                 t.fill_(0)                               # eager work between the replays
