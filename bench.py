@@ -119,6 +119,8 @@ class Step:
             idx = m.datagen.scene_voxels(grid, wl["rows"], wl["seed"], **wl.get("scene", {}))
         else:
             idx = m.datagen.uniform_voxels(grid, wl["per_batch"] * grid[0], wl["seed"])
+        if wl.get("shuffle"):
+            idx = np.ascontiguousarray(idx[np.random.default_rng(wl["seed"]).permutation(idx.shape[0])])
         self.idx_np = idx
         L = idx.shape[0]
         ks = wl["ks"]
@@ -242,6 +244,10 @@ class Step:
         s = self.elem
         return self.L * self.ci * s + self.n_out * self.co * s + self.K * self.ci * self.co * s + 8.0 * self.P
 
+    def backward_filter_bytes(self):
+        s = self.elem
+        return self.L * self.ci * s + self.n_out * self.co * s + self.K * self.ci * self.co * 4.0 + 8.0 * self.P
+
 
 def median(v):
     v = sorted(v)
@@ -353,6 +359,36 @@ def measured_traffic(workload, kernel):
         return doc["kernels"][kernel]["total_bytes"], None
     except (OSError, KeyError, ValueError):
         return None, "no counter summary for this kernel and workload"
+
+
+def operator_roofline(workload, kernels, names, op_ms, alg_bytes, bytes_model, flops=None, mfma_peak=None):
+    """Roofline object of one operator: its algorithmic bytes over its device time `op_ms` (HIP
+    events around back-to-back calls, launch gaps between its kernels included), the counter
+    traffic summed over its kernels `names` (those of them that ran).  `kernel_sum_us` adds up
+    the library's per-kernel event timing of the same kernels, which reads about 2 us a launch
+    above the kernel trace."""
+    ran = [n for n in names if n in kernels]
+    if not ran:
+        return None
+    kernel_sum = sum(kernels[n]["avg_us"] * kernels[n].get("launches_per_step", kernels[n].get("launches", 1.0))
+                     for n in ran)
+    us = op_ms * 1e3
+    traffic, note = 0.0, None
+    for n in ran:
+        t, why = measured_traffic(workload, n)
+        if t is None:
+            traffic, note = None, why
+            break
+        traffic += t
+    achieved = alg_bytes / (us * 1e-6) / 1e9
+    out = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+           "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernels": ran, "operator_us": us,
+           "kernel_sum_us": kernel_sum, "algorithmic_bytes": alg_bytes, "bytes_model": bytes_model}
+    if note:
+        out["traffic_note"] = note
+    if flops is not None:
+        out["mfma_frac"] = flops / (us * 1e-6) / 1e12 / mfma_peak
+    return out
 
 
 UPSTREAM = {
@@ -596,6 +632,10 @@ def main():
                               "kernel_avg_us": dom_ms * 1e3, "algorithmic_bytes": alg_bytes, "bytes_model": what}
     if traffic_note:
         result["roofline"]["traffic_note"] = traffic_note
+    # the other half of the metric: the rulebook's kernels against its algorithmic bytes
+    result["rulebook_roofline"] = operator_roofline(
+        args.workload, kernels, [n for n in kernels if n.startswith("rb")], rb_ms, step.rulebook_bytes(),
+        "rulebook bytes 16L + 8KL + 4K + 16N_out")
     gather = [n for n in agg if n.startswith("gatherConv")]
     if gather:
         g = max(gather, key=lambda n: agg[n][0])
@@ -620,16 +660,42 @@ def main():
     result["backward_kernels"] = {n: {"avg_us": t / c * 1e3, "launches": c / 5} for n, (t, c) in agg_b.items()}
     result["backward_data_ms"] = median(per_b["backward_data"])
     result["backward_filter_ms"] = median(per_b["backward_filter"])
+    bk = result["backward_kernels"]
+    filter_kernels = [n for n in bk if n.startswith("backwardFilter") or n.startswith("sliceSum")
+                      or n.startswith("reduceFilter")]
+    result["backward_data_roofline"] = operator_roofline(
+        args.workload, bk, [n for n in bk if n not in filter_kernels], result["backward_data_ms"],
+        step.forward_bytes(), "backward-data bytes N*Co*s + L*Ci*s + K*Ci*Co*s + 8P", step.conv_flops(), mfma_peak)
+    result["backward_filter_roofline"] = operator_roofline(
+        args.workload, bk, filter_kernels, result["backward_filter_ms"], step.backward_filter_bytes(),
+        "backward-filter bytes L*Ci*s + N*Co*s + K*Ci*Co*4 + 8P", step.conv_flops(), mfma_peak)
     result["backward_data_tflops"] = step.conv_flops() / (result["backward_data_ms"] * 1e-3) / 1e12
     result["backward_filter_tflops"] = step.conv_flops() / (result["backward_filter_ms"] * 1e-3) / 1e12
 
     # Not part of the metric: the step without the copy of indice_num (a caller that kept the counts
     # of an identical rulebook).  The forward operator then cannot know yet whether the rulebook's
-    # input rows were in cell order and takes the way that assumes nothing.
+    # input rows were in cell order: it starts on the pair lists and enqueues the row-map kernels
+    # behind them, and the device decides which of the two do the work.
     wall_nr, per_nr = time_ops(torch, [("get_indice_pairs", step.rulebook), ("forward", step.forward)],
                                max(args.steps // 2, 5))
     result["without_count_readback"] = {"ms_per_step": wall_nr * 1e3 / max(args.steps // 2, 5),
                                         "forward_ms": median(per_nr["forward"])}
+    # Not part of the metric either: the same voxels in shuffled row order (what a voxelizer that
+    # numbers voxels by first point hands over): the rulebook goes through its hash table and
+    # forward through a row map.
+    shuffled = Step(handle, dict(wl, shuffle=True))
+    sh_ops = [("get_indice_pairs", shuffled.rulebook), ("read_counts", shuffled.read_counts),
+              ("forward", shuffled.forward)]
+    for _ in range(max(args.warmup // 4, 2)):
+        for _, fn in sh_ops:
+            fn()
+    n_sh = max(args.steps // 4, 5)
+    _, per_srb = time_ops(torch, [("get_indice_pairs", shuffled.rulebook)], n_sh)
+    shuffled.read_counts()
+    _, per_sfw = time_ops(torch, [("forward", shuffled.forward)], n_sh)
+    result["shuffled_rows"] = {"rulebook_ms": median(per_srb["get_indice_pairs"]),
+                               "forward_ms": median(per_sfw["forward"]), "pairs": shuffled.P}
+    del shuffled
     if step.sub_m:
         result["graph_replay"] = graph_replay_step(
             torch, m, handle, step, [("get_indice_pairs", step.rulebook), ("forward", step.forward)], args.steps)

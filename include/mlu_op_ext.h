@@ -124,13 +124,18 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtForgetRowMap(mluOpHandle_t handle, const voi
 
 /* mluOpIndiceConvolutionBackwardFilter for callers that cannot allocate device memory (code
  * under HIP graph capture, serving loops, harnesses that forbid hipMalloc) and therefore have
- * no workspace to hand over.  No counterpart in the reference.  Same arguments, checks and
- * result bits as mluOpIndiceConvolutionBackwardFilter (mlu_op.h), without `workspace` and
- * `workspace_size`: the partial sums live in an array of MLUOP_EXT_NO_ALLOC_SCRATCH_BYTES that
- * the library holds on every GPU it runs on until the process ends.  The call allocates and
- * frees nothing and does not wait for the queue.  MLUOP_STATUS_NOT_SUPPORTED when the shape
- * needs more scratch memory than that (mluOpGetIndiceConvolutionBackwardFilterWorkspaceSize
- * reports the need) or more than 128 kernel offsets.  All calls on one GPU share the array:
+ * no workspace to hand over.  No counterpart in the reference.  Same arguments and checks as
+ * mluOpIndiceConvolutionBackwardFilter (mlu_op.h), without `workspace` and `workspace_size`:
+ * the partial sums live in an array of MLUOP_EXT_NO_ALLOC_SCRATCH_BYTES that the library
+ * holds on every GPU it runs on until the process ends.  The call allocates and frees nothing,
+ * does not wait for the queue, follows the handle's kernel choices and is left out of its
+ * per-kernel timing (which creates events).  Shapes of the matrix-core kernels (16 to 128
+ * channels) whose usual number of partial tiles exceeds the array are cut into fewer, longer
+ * slices: the result then agrees with the workspace entry point within the accuracy standard
+ * (the additions are grouped differently), and bit for bit otherwise (up to 64 x 64 channels at
+ * 27 offsets).  MLUOP_STATUS_NOT_SUPPORTED when the array is too small all the same (the generic
+ * kernels' tiles at large channel counts) or with more than 128 kernel offsets.  All calls on
+ * one GPU share the array:
  * calls that can overlap there (different queues, different handles) race and must be ordered
  * by the caller. */
 #define MLUOP_EXT_NO_ALLOC_SCRATCH_BYTES (16 * 1024 * 1024)

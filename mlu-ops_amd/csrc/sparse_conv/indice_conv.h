@@ -59,6 +59,9 @@ struct ConvProblem {
   // building a row map.  `ticket` is a value no earlier launch on this workspace used.
   ListTrust list_trust = ListTrust::kNone;
   unsigned long long ticket = 0;
+  // Backward filter only: the most Ci x Co fp32 partial tiles the workspace may hold (0: as
+  // many as the kernels like to use); the pair lists are cut into fewer, longer slices then.
+  int max_partial_tiles = 0;
   // Backward filter only: element strides of dW(k, ci, co) in filters_grad;
   // all zero = the positional [K, Ci, Co].
   int64_t grad_stride_k = 0, grad_stride_ci = 0, grad_stride_co = 0;

@@ -2870,6 +2870,14 @@ bool filterMfmaShapeOk(const ConvProblem &p) {
   return ok(p.Ci) && ok(p.Co) && p.K <= kMaxInlineK;
 }
 
+// Slices the MFMA kernels cut the pair lists into at most: kFilterMaxSlices, or what a capped
+// workspace leaves beside one tile per offset.
+int filterMaxSlices(const ConvProblem &p) {
+  if (p.max_partial_tiles <= 0) return kFilterMaxSlices;
+  const int room = p.max_partial_tiles - p.K;
+  return room < 1 ? 1 : (room > kFilterMaxSlices ? kFilterMaxSlices : room);
+}
+
 int filterGradSplits(const ConvProblem &p) {
   // Bounded by the tensor shape only, so the workspace query and the launch
   // agree whatever indice_num holds.
@@ -2891,9 +2899,9 @@ FilterGradWorkspace carveFilterGrad(const ConvProblem &p, void *base) {
   if (p.K > kMaxInlineK) ws.dev_counts = reinterpret_cast<int32_t *>(take((size_t)p.K * 4));
   ws.splits = filterGradSplits(p);
   size_t tiles = ws.splits > 1 ? (size_t)ws.splits * p.K : 0;
-  // the MFMA path writes at most kFilterMaxSlices + K partial tiles
-  if (filterMfmaShapeOk(p) && (size_t)kFilterMaxSlices + p.K > tiles)
-    tiles = (size_t)kFilterMaxSlices + p.K;
+  // the MFMA path writes at most filterMaxSlices + K partial tiles
+  if (filterMfmaShapeOk(p) && (size_t)filterMaxSlices(p) + p.K > tiles)
+    tiles = (size_t)filterMaxSlices(p) + p.K;
   if (tiles > 0) ws.partial = reinterpret_cast<float *>(take(tiles * p.Ci * p.Co * 4));
   ws.bytes = off + kBaseAlign;
   return ws;
@@ -2989,7 +2997,8 @@ void launchFilterMfma(const LaunchCtx &lc, const ConvProblem &p, const FilterGra
     SliceTable tab;
     long long total = 0;
     for (int k = 0; k < p.K; ++k) total += inl.n[k];
-    int slice_len = (int)((total + kFilterMaxSlices - 1) / kFilterMaxSlices);
+    const int max_slices = filterMaxSlices(p);
+    int slice_len = (int)((total + max_slices - 1) / max_slices);
     slice_len = (slice_len + kFilterStepPairs - 1) / kFilterStepPairs * kFilterStepPairs;
     // A slice has fixed costs (the first rows' round trip, a Ci x Co fp32 tile written and summed
     // again): few pairs are not cut finer than this, at the price of idle CUs (config 5b, 128 x

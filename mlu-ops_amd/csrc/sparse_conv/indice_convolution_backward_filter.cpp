@@ -316,9 +316,12 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtIndiceConvolutionBackwardFilterNoAlloc(
   PARAM_CHECK(api, output_grad != nullptr);
   PARAM_CHECK(api, indice_pairs != nullptr);
   PARAM_CHECK(api, filters_grad != nullptr);
-  const ConvProblem p =
+  ConvProblem p =
       makeProblem(handle, features_desc, output_grad_desc, indice_pairs_desc, filters_grad_desc,
                   indice_num, inverse, indice_pairs);
+  // the pair lists are cut into as many slices as the array has room for partial tiles
+  p.max_partial_tiles = (int)(((size_t)MLUOP_EXT_NO_ALLOC_SCRATCH_BYTES - 4096) /
+                              ((size_t)p.Ci * p.Co * sizeof(float)));
   if (!mluop::sparse_conv::backwardFilterLaunchesOnly(p)) {
     MLUOP_LOG(ERROR) << api << " a kernel volume of " << p.K << " offsets needs a staging copy "
                      << "and a wait for the queue; use mluOpIndiceConvolutionBackwardFilter.";
@@ -332,14 +335,18 @@ mluOpStatus_t MLUOP_WIN_API mluOpExtIndiceConvolutionBackwardFilterNoAlloc(
     return MLUOP_STATUS_NOT_SUPPORTED;
   }
   DEVICE_HANDLE_CHECK(api, handle);
-  void *ptr = handle->device < kMaxScratchDevices ? g_scratch_ptr[handle->device] : nullptr;
+  void *ptr = nullptr;
+  if (handle->device < kMaxScratchDevices) {
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    ptr = g_scratch_ptr[handle->device];
+  }
   if (ptr == nullptr) {
     MLUOP_LOG(ERROR) << api << " the scratch memory of device " << handle->device
                      << " was not found when the handle was created.";
     return MLUOP_STATUS_NOT_INITIALIZED;
   }
-  // no event pairs here: the per-kernel timer creates events on demand
-  const mluop::LaunchCtx lc(handle->queue, nullptr);
+  // the handle's kernel choices, but no event pairs: the per-kernel timer creates events on demand
+  const mluop::LaunchCtx lc(handle->queue, nullptr, &handle->kernel_choices);
   HIP_CHECK_RETURN(api, mluop::sparse_conv::launchBackwardFilter(lc, p, features, output_grad,
                                                                 ptr, filters_grad));
   return MLUOP_STATUS_SUCCESS;

@@ -347,9 +347,23 @@ def mean_voxel_features(voxels, num_points_per_voxel):
     return voxels.sum(dim=1) / num_points_per_voxel.clamp(min=1).to(voxels.dtype).unsqueeze(1)
 
 
-def sparse_tensor_from_voxels(features, coors, spatial_shape, batch_index=0, batch_size=1):
-    """SparseTensor of one cloud's voxels: indices (n, z, y, x) with n = batch_index."""
+def sparse_tensor_from_voxels(features, coors, spatial_shape, batch_index=0, batch_size=1, order_by_cell=True):
+    """SparseTensor of one cloud's voxels: indices (n, z, y, x) with n = batch_index.
+
+    A voxelizer numbers its voxels by their first point, not by their place in the grid.  With
+    `order_by_cell` (the default) the voxels are put in ascending order of their linear cell
+    index here, once: every rulebook built from them, and from the outputs of the layers that
+    follow, then sees rows in cell order, which mluOpGetIndicePairs resolves without its hash
+    table and the convolutions read as pair lists without a row map.  The rows of the returned
+    tensor are a permutation of the voxelizer's; `order_by_cell=False` keeps its order."""
+    coors = coors.to(torch.int32)
+    if order_by_cell and coors.shape[0] > 1:
+        d, h, w = (int(v) for v in spatial_shape)
+        key = (coors[:, 0].to(torch.int64) * h + coors[:, 1].to(torch.int64)) * w + coors[:, 2].to(torch.int64)
+        order = torch.argsort(key)
+        coors = coors[order]
+        features = features[order]
     n = torch.full((coors.shape[0], 1), int(batch_index), dtype=torch.int32, device=coors.device)
     # a voxelizer emits every voxel once
-    return SparseTensor(features, torch.cat([n, coors.to(torch.int32)], dim=1), spatial_shape, batch_size,
+    return SparseTensor(features, torch.cat([n, coors], dim=1).contiguous(), spatial_shape, batch_size,
                         distinct=True)

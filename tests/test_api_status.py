@@ -529,6 +529,25 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(m.SIGNATURES), declared ^ set(m.SIGNATURES)
 
 
+def test_library_exports_the_c_api_and_nothing_else():
+    """The dynamic symbol table of libmluops.so holds the declared mluOp* functions only: the C++
+    helpers behind them are local (the reference links with a symbol map for the same reason,
+    CMakeLists.txt:226, scripts/gen_symbol_visibility_map.py)."""
+    import shutil
+    import subprocess
+    nm = shutil.which("nm")
+    if nm is None:
+        pytest.skip("nm is not installed")
+    out = subprocess.run([nm, "-D", "--defined-only", m.LIB_PATH], check=True, capture_output=True, text=True).stdout
+    exported = {line.split()[-1] for line in out.splitlines() if line.strip()}
+    declared = set()
+    for name in ("mlu_op.h", "mlu_op_ext.h"):
+        text = open(os.path.join(ROOT, "include", name)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        declared |= set(re.findall(r"\b(mluOp[A-Za-z0-9_]+)\s*\(", text))
+    assert exported == declared, sorted(exported ^ declared)
+
+
 # --- extended modes (mluOpExtSetSparseConvExtendedModes): inverse = 1, tagged filters_grad ------
 
 def _d(dims, dtype="MLUOP_DTYPE_FLOAT", layout="MLUOP_LAYOUT_ARRAY"):
@@ -760,11 +779,11 @@ def test_row_map_entry_points(handle):
 def test_kernel_choice_setter_checks_its_arguments(handle):
     ok, bad = STATUS["MLUOP_STATUS_SUCCESS"], STATUS["MLUOP_STATUS_BAD_PARAM"]
     f = m.lib().mluOpExtSetKernelChoice
-    for which in range(7):
+    for which in range(8):
         for value in (-1, 0, 1, -1):
             assert f(handle.ptr, which, value) == ok
     assert f(None, 0, 1) == bad
-    assert f(handle.ptr, 7, 1) == bad and f(handle.ptr, -1, 1) == bad
+    assert f(handle.ptr, 8, 1) == bad and f(handle.ptr, -1, 1) == bad
     assert f(handle.ptr, 0, 2) == bad and f(handle.ptr, 0, -2) == bad
 
 

@@ -174,17 +174,33 @@ def test_points_to_voxels_to_submanifold_layer(gpu_handle):
     assert V == len({tuple(r) for r in c.tolist()}) and (c >= 0).all() and (c < np.array(space)).all()
     assert int(npv.sum().item()) <= 4000 and int(npv.min().item()) >= 1
     feats = spnn.mean_voxel_features(voxels, npv)
-    st = spnn.sparse_tensor_from_voxels(feats, coors, space)
     torch.manual_seed(5)
     layer = spnn.SubMConv3d(4, 16, 3).cuda()
-    y = layer(st).features.detach().cpu().double()
     dense = torch.zeros((1, 4) + space, dtype=torch.float64)
     ci = torch.from_numpy(c.astype(np.int64))
     dense[0, :, ci[:, 0], ci[:, 1], ci[:, 2]] = feats.cpu().double().t()
     w = layer.weight.detach().cpu().double().permute(4, 3, 0, 1, 2)
-    ref = F.conv3d(dense, w, padding=1)[0][:, ci[:, 0], ci[:, 1], ci[:, 2]].t()
-    d1 = (y - ref).abs().sum() / ref.abs().sum()
-    assert d1 <= 1e-5, float(d1)
+    full = F.conv3d(dense, w, padding=1)[0]
+    # The voxelizer numbers voxels by first point; the sparse tensor puts them in cell order, so
+    # the layer's rulebook needs no hash table and its forward no row map.
+    handle = spnn._handle()
+    for order_by_cell in (True, False):
+        st = spnn.sparse_tensor_from_voxels(feats, coors, space, order_by_cell=order_by_cell)
+        rows = st.indices[:, 1:].cpu().numpy().astype(np.int64)
+        assert sorted(map(tuple, rows.tolist())) == sorted(map(tuple, c.tolist()))
+        if order_by_cell:
+            lin = (rows[:, 0] * space[1] + rows[:, 1]) * space[2] + rows[:, 2]
+            assert (np.diff(lin) > 0).all()
+        handle.set_kernel_timing(True)
+        y = layer(st).features.detach().cpu().double()
+        names = [n for n, _ in handle.kernel_timings()]
+        handle.set_kernel_timing(False)
+        assert any(n.startswith("gatherConv") for n in names), names
+        took_the_map = [n for n in names if n in ("scatterRowMap", "fillMapPackFilter", "fillInt32")]
+        assert (not took_the_map) == order_by_cell, names
+        ref = full[:, rows[:, 0], rows[:, 1], rows[:, 2]].t()
+        d1 = (y - ref).abs().sum() / ref.abs().sum()
+        assert d1 <= 1e-5, float(d1)
 
 
 def test_small_channel_counts_are_padded_for_the_matrix_cores(gpu_handle):
