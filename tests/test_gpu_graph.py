@@ -223,3 +223,48 @@ def test_four_host_threads_with_a_handle_each():
     for i, (got, want) in enumerate(zip(results, alone)):
         for g, w_ in zip(got, want):
             assert torch.equal(g, w_), "thread %d" % i
+
+
+def test_a_captured_rulebook_files_no_report_in_host_memory():
+    """The last kernel of an eager rulebook tells the host, through the handle's pinned memory,
+    whether the rows were in cell order.  A captured rulebook must not: its replays would write
+    into a slot that by then belongs to another rulebook, or to a handle that is gone.  Seen from
+    outside: after a replay (and a wait) a forward call on the captured rulebook still does not
+    know the order, so it enqueues the list kernels and the row-map kernels behind them."""
+    import torch
+    import mluop_hip as m
+    rng = np.random.default_rng(35)
+    batch, space, L, c, ks = 1, (10, 20, 20), 2000, 32, (3, 3, 3)
+    idx = torch.from_numpy(random_voxels(rng, batch, space, L, shuffle=False)).cuda()
+    feats = torch.from_numpy(rng.standard_normal((L, c)).astype(np.float32)).cuda().half()
+    w = torch.from_numpy((rng.standard_normal(ks + (c, c)) * 0.1).astype(np.float32)).cuda().half()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    guard_bytes, m.GUARD_BYTES = m.GUARD_BYTES, 0
+    try:
+        with torch.cuda.stream(side):
+            handle = m.make_handle_on_current_stream()
+
+            def rulebook():
+                return m.get_indice_pairs(handle, idx, batch, space, ks, list(space), [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+
+            pairs0, _, num0, _ = rulebook()
+            side.synchronize()
+            num_host = num0.cpu().tolist()
+            want = m.indice_conv_forward(handle, feats, w, m.LAYOUT_ARRAY, pairs0, num_host, L, True)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                pairs, _, _, _ = rulebook()
+            graph.replay()
+            side.synchronize()
+            assert torch.equal(pairs, pairs0)
+            handle.set_kernel_timing(True)
+            got = m.indice_conv_forward(handle, feats, w, m.LAYOUT_ARRAY, pairs, num_host, L, True)
+            names = [n for n, _ in handle.kernel_timings()]
+            handle.set_kernel_timing(False)
+            assert "packFilterCutPairLists" in names and "scatterRowMap" in names, names
+            assert torch.equal(got, want)
+        torch.cuda.current_stream().wait_stream(side)
+        handle.close()
+    finally:
+        m.GUARD_BYTES = guard_bytes
