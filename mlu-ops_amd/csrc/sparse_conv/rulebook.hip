@@ -337,6 +337,55 @@ __device__ __forceinline__ void stagePairs(const int (&res)[N], int k_first, int
   if (lane < N && k_first + lane < k_end) st.counts[(size_t)(k_first + lane) * st.n_wave + wt] = my_entry;
 }
 
+// Marks the output cells cell[0..N) of the 64 lanes (kEmptyKey: none) in the bitmap.
+// Rows in cell order walk along w, so the lanes of a wavefront mark runs of cells
+// in the same bitmap word: a run's bits are gathered at its last lane, which alone
+// goes to memory (atomics on the bitmap are what a marking kernel would wait for).  Lanes
+// with no output cell join the run in front of them; a lane whose word is below one
+// in front of it (rows out of order) marks its cell by itself.
+template <int N>
+__device__ __forceinline__ void markCells(const uint32_t (&cell)[N], unsigned long long *bitmap) {
+  const int lane = threadIdx.x & (kWave - 1);
+  uint32_t word_at[N];
+  unsigned long long bits[N];
+  uint32_t alone = 0;
+#pragma unroll
+  for (int u = 0; u < N; ++u) {
+    const bool valid = cell[u] != kEmptyKey;
+    const uint32_t mine = cell[u] >> 6;
+    const uint32_t run = waveInclusiveMax(valid ? mine : 0u);
+    const bool joins = valid && run == mine;
+    if (valid && !joins) alone |= 1u << u;
+    uint32_t lo = 0, hi = 0;
+    if (joins) {
+      lo = (cell[u] & 32u) ? 0u : 1u << (cell[u] & 31u);
+      hi = (cell[u] & 32u) ? 1u << (cell[u] & 31u) : 0u;
+    }
+    waveRunInclusiveOr(run, &lo, &hi);
+    const uint32_t run_next = __shfl_down(run, 1, kWave);
+    const bool last = lane == kWave - 1 || run_next != run;
+    word_at[u] = run;
+    bits[u] = last ? ((unsigned long long)hi << 32) | lo : 0ull;
+  }
+  // (a stale word from the cache only costs an atomic that changes nothing)
+  unsigned long long seen[N];
+#pragma unroll
+  for (int u = 0; u < N; ++u) seen[u] = bits[u] ? bitmap[word_at[u]] : ~0ull;
+#pragma unroll
+  for (int u = 0; u < N; ++u)
+    if ((seen[u] & bits[u]) != bits[u]) atomicOr(bitmap + word_at[u], bits[u]);
+  if (__any(alone != 0)) {
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+      if (alone & (1u << u)) {
+        const unsigned long long bit = 1ull << (cell[u] & 63);
+        unsigned long long *word = bitmap + (cell[u] >> 6);
+        if ((*word & bit) == 0) atomicOr(word, bit);
+      }
+    }
+  }
+}
+
 // One wavefront per 64 consecutive rows, offsets in groups of kGroup so that a
 // lane keeps kGroup independent table probes in flight.  For every offset:
 // resolve the pair (submanifold: table lookup -> output row; regular: output
@@ -438,51 +487,10 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g,
         if (hit & (1u << u)) res[u] = vals[slot[u]];
       }
     } else {
-      // Rows in cell order walk along w, so the lanes of a wavefront mark runs of cells
-      // in the same bitmap word: a run's bits are gathered at its last lane, which alone
-      // goes to memory (atomics on the bitmap are what this kernel would wait for).  Lanes
-      // with no output cell join the run in front of them; a lane whose word is below one
-      // in front of it (rows out of order) marks its cell by itself.
-      const int lane = threadIdx.x & (kWave - 1);
-      uint32_t word_at[kGroup];
-      unsigned long long bits[kGroup];
-      uint32_t alone = 0;
-#pragma unroll
-      for (int u = 0; u < kGroup; ++u) {
-        const bool valid = cell[u] != kEmptyKey;
-        if (valid) res[u] = (int)cell[u];
-        const uint32_t mine = cell[u] >> 6;
-        const uint32_t run = waveInclusiveMax(valid ? mine : 0u);
-        const bool joins = valid && run == mine;
-        if (valid && !joins) alone |= 1u << u;
-        uint32_t lo = 0, hi = 0;
-        if (joins) {
-          lo = (cell[u] & 32u) ? 0u : 1u << (cell[u] & 31u);
-          hi = (cell[u] & 32u) ? 1u << (cell[u] & 31u) : 0u;
-        }
-        waveRunInclusiveOr(run, &lo, &hi);
-        const uint32_t run_next = __shfl_down(run, 1, kWave);
-        const bool last = lane == kWave - 1 || run_next != run;
-        word_at[u] = run;
-        bits[u] = last ? ((unsigned long long)hi << 32) | lo : 0ull;
-      }
-      // (a stale word from the cache only costs an atomic that changes nothing)
-      unsigned long long seen[kGroup];
-#pragma unroll
-      for (int u = 0; u < kGroup; ++u) seen[u] = bits[u] ? bitmap[word_at[u]] : ~0ull;
 #pragma unroll
       for (int u = 0; u < kGroup; ++u)
-        if ((seen[u] & bits[u]) != bits[u]) atomicOr(bitmap + word_at[u], bits[u]);
-      if (__any(alone != 0)) {
-#pragma unroll
-        for (int u = 0; u < kGroup; ++u) {
-          if (alone & (1u << u)) {
-            const unsigned long long bit = 1ull << (cell[u] & 63);
-            unsigned long long *word = bitmap + (cell[u] >> 6);
-            if ((*word & bit) == 0) atomicOr(word, bit);
-          }
-        }
-      }
+        if (cell[u] != kEmptyKey) res[u] = (int)cell[u];
+      markCells<kGroup>(cell, bitmap);
       // every pair slot of this row and these offsets starts out as -1; the kernel that
       // places the pairs overwrites the front of each list afterwards
       if (active) {
@@ -493,6 +501,112 @@ __global__ __launch_bounds__(kBlock) void rbProbeCount(GeomDev g,
       }
     }
     stagePairs<SUBM, kGroup>(res, k0, k_hi, j, staging, &staged);
+  }
+}
+
+// Regular mode with a stride above 1 and a small kernel (KD x KH x KW known at compile
+// time).  Of the K offsets of a row only those whose kernel position has the right
+// remainder on every axis give an output cell: one in eight at stride 2.  Marking cells is
+// the expensive part (a dozen cross-lane steps per marked cell), so it runs over the
+// candidates of a row, the m-th valid kernel position of every axis (mark_n[a] of them at
+// most: 2 x 2 x 2 for a 3 x 3 x 3 kernel at stride 2, one for 2 x 2 x 2), and not over the
+// offsets; staging, which must go offset by offset, is a bit test and an addition per
+// offset once the output coordinate of every kernel position is known.  blockIdx.y
+// slices both: the candidates along d for marking, the offsets for staging.
+template <int KD, int KH, int KW>
+__global__ __launch_bounds__(kBlock) void rbProbeStrided(GeomDev g, const int32_t *indices, bool aligned,
+                                                          unsigned long long *bitmap, Staging staging,
+                                                          int k_per_slice, int mark_d, int mark_h,
+                                                          int32_t *rows_in_order, int32_t *pairs) {
+  constexpr int K = KD * KH * KW;
+  const int j = blockIdx.x * kBlock + threadIdx.x;
+  const int k_lo = blockIdx.y * k_per_slice;
+  const int k_hi = k_lo + k_per_slice < K ? k_lo + k_per_slice : K;
+  if ((j >> 6) >= staging.n_wave) return;  // whole wave beyond the last row
+  const bool active = j < g.L;
+  int4 c = make_int4(-1, 0, 0, 0);
+  if (active) {
+    c = loadCoord(indices, j, aligned);
+    if (blockIdx.y == 0) noteRowOrder(indices, j, c, aligned, rows_in_order);
+    // every pair slot of this row starts out as -1 for the slice's offsets; the kernel that
+    // places the pairs overwrites the front of each list afterwards
+    for (int k = k_lo; k < k_hi; ++k) {
+      pairs[(size_t)(2 * k) * g.L + j] = -1;
+      pairs[(size_t)(2 * k + 1) * g.L + j] = -1;
+    }
+  }
+  const bool n_ok = active && (unsigned)c.x < (unsigned)g.batch;
+  // output coordinate of every kernel position, or -1
+  int od[KD], oh[KH], ow[KW];
+#pragma unroll
+  for (int t = 0; t < KD; ++t)
+    od[t] = n_ok ? axisOut(c.y, g.pad[0], t, g.dil[0], g.stride[0], g.by_stride[0], g.out[0]) : -1;
+#pragma unroll
+  for (int t = 0; t < KH; ++t) oh[t] = axisOut(c.z, g.pad[1], t, g.dil[1], g.stride[1], g.by_stride[1], g.out[1]);
+#pragma unroll
+  for (int t = 0; t < KW; ++t) ow[t] = axisOut(c.w, g.pad[2], t, g.dil[2], g.stride[2], g.by_stride[2], g.out[2]);
+  // the valid ones in ascending kernel position: the candidates
+  int cd[KD], ch[KH], cw[KW];
+  {
+    int n = 0;
+#pragma unroll
+    for (int t = 0; t < KD; ++t) cd[t] = -1;
+#pragma unroll
+    for (int t = 0; t < KD; ++t) {
+#pragma unroll
+      for (int m = 0; m < KD; ++m)
+        if (od[t] >= 0 && n == m) cd[m] = od[t];
+      n += od[t] >= 0 ? 1 : 0;
+    }
+    n = 0;
+#pragma unroll
+    for (int t = 0; t < KH; ++t) ch[t] = -1;
+#pragma unroll
+    for (int t = 0; t < KH; ++t) {
+#pragma unroll
+      for (int m = 0; m < KH; ++m)
+        if (oh[t] >= 0 && n == m) ch[m] = oh[t];
+      n += oh[t] >= 0 ? 1 : 0;
+    }
+    n = 0;
+#pragma unroll
+    for (int t = 0; t < KW; ++t) cw[t] = -1;
+#pragma unroll
+    for (int t = 0; t < KW; ++t) {
+#pragma unroll
+      for (int m = 0; m < KW; ++m)
+        if (ow[t] >= 0 && n == m) cw[m] = ow[t];
+      n += ow[t] >= 0 ? 1 : 0;
+    }
+  }
+  // marking: candidate m_d along d goes to slice m_d % gridDim.y
+#pragma unroll
+  for (int md = 0; md < KD; ++md) {
+    if (md >= mark_d || md % (int)gridDim.y != (int)blockIdx.y) continue;
+#pragma unroll
+    for (int mh = 0; mh < KH; ++mh) {
+      if (mh >= mark_h) continue;
+      uint32_t cell[KW];
+      const int line = (cd[md] | ch[mh]) >= 0 ? ((c.x * g.out[0] + cd[md]) * g.out[1] + ch[mh]) * g.out[2] : -1;
+#pragma unroll
+      for (int mw = 0; mw < KW; ++mw) cell[mw] = (line | cw[mw]) >= 0 ? (uint32_t)(line + cw[mw]) : kEmptyKey;
+      markCells<KW>(cell, bitmap);
+    }
+  }
+  // staging: offset by offset, KW at a time
+  int staged = 0;
+#pragma unroll
+  for (int kd = 0; kd < KD; ++kd) {
+#pragma unroll
+    for (int kh = 0; kh < KH; ++kh) {
+      const int k_first = (kd * KH + kh) * KW;
+      if (k_first < k_lo || k_first >= k_hi) continue;
+      int res[KW];
+      const int line = (od[kd] | oh[kh]) >= 0 ? ((c.x * g.out[0] + od[kd]) * g.out[1] + oh[kh]) * g.out[2] : -1;
+#pragma unroll
+      for (int kw = 0; kw < KW; ++kw) res[kw] = (line | ow[kw]) >= 0 ? line + ow[kw] : -1;
+      stagePairs<false, KW>(res, k_first, k_hi, j, staging, &staged);
+    }
   }
 }
 
@@ -1476,13 +1590,45 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
       fill, ws.rows_in_order);
   lc.end();
   const int k_per = offsetsPerSlice(g.K);
-  const Staging staging = {ws.stage, ws.stage_lane, ws.counts, ws.n_wave, k_per, k_per * kWave, 0};
-  lc.begin("rbProbeCount");
+  Staging staging = {ws.stage, ws.stage_lane, ws.counts, ws.n_wave, k_per, k_per * kWave, 0};
   const dim3 slice_grid(l_blocks, (g.K + k_per - 1) / k_per);
-  rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, indices, al_in, nullptr,
-                                                            nullptr, 0, ws.bitmap, staging, k_per,
-                                                            ws.rows_in_order, indice_pairs);
-  lc.end();
+  // most kernel positions of one axis that can have an output cell for one input coordinate:
+  // those that share a remainder of position * dilation modulo the stride
+  auto candidates = [&](int a) {
+    int most = 0;
+    for (int r = 0; r < g.stride[a]; ++r) {
+      int n = 0;
+      for (int t = 0; t < g.ksize[a]; ++t) n += (t * g.dilation[a]) % g.stride[a] == r ? 1 : 0;
+      most = n > most ? n : most;
+    }
+    return most;
+  };
+  const bool strided = g.stride[0] > 1 || g.stride[1] > 1 || g.stride[2] > 1;
+  const bool cube3 = g.ksize[0] == 3 && g.ksize[1] == 3 && g.ksize[2] == 3;
+  const bool cube2 = g.ksize[0] == 2 && g.ksize[1] == 2 && g.ksize[2] == 2;
+  if (strided && (cube3 || cube2)) {
+    // slices of whole (kd, kh) groups of offsets
+    const int per = cube3 ? 9 : 4;
+    staging.k_per_slice = per;
+    staging.block_ints = per * kWave;
+    const dim3 grid(l_blocks, (g.K + per - 1) / per);
+    lc.begin("rbProbeStrided");
+    if (cube3)
+      rbProbeStrided<3, 3, 3><<<grid, kBlock, 0, lc.stream>>>(d, indices, al_in, ws.bitmap, staging, per,
+                                                              candidates(0), candidates(1),
+                                                              ws.rows_in_order, indice_pairs);
+    else
+      rbProbeStrided<2, 2, 2><<<grid, kBlock, 0, lc.stream>>>(d, indices, al_in, ws.bitmap, staging, per,
+                                                              candidates(0), candidates(1),
+                                                              ws.rows_in_order, indice_pairs);
+    lc.end();
+  } else {
+    lc.begin("rbProbeCount");
+    rbProbeCount<false><<<slice_grid, kBlock, 0, lc.stream>>>(d, indices, al_in, nullptr,
+                                                              nullptr, 0, ws.bitmap, staging, k_per,
+                                                              ws.rows_in_order, indice_pairs);
+    lc.end();
+  }
   lc.begin("rbBitmapBlockSum");
   rbBitmapBlockSum<<<ws.n_bitmap_blocks, kBlock, 0, lc.stream>>>(ws.bitmap, ws.n_words, ws.block_sum);
   lc.end();
