@@ -227,6 +227,10 @@ mluOpStatus_t MLUOP_WIN_API mluOpGetIndicePairs(
   int32_t *pairs = static_cast<int32_t *>(indice_pairs);
   int32_t *out_rows = static_cast<int32_t *>(out_indices);
   int32_t *counts = static_cast<int32_t *>(indice_num);
+  // the other outputs and the workspace are no pair tensors any more, whatever was noted there
+  mluop::sparse_conv::forgetRulebookNotesIn(handle, out_indices, out_indices_desc->total_tensor_size);
+  mluop::sparse_conv::forgetRulebookNotesIn(handle, indice_num, indice_num_desc->total_tensor_size);
+  mluop::sparse_conv::forgetRulebookNotesIn(handle, workspace, workspace_size);
   const mluop::sparse_conv::RulebookReportTarget report =
       mluop::sparse_conv::openRulebookNote(handle, indice_pairs, g.K, g.L);
   if (g.sub_m) {

@@ -301,6 +301,9 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardData(
   p.distinct_pairs = handle->distinct_pairs_promised;
   st = mluop::sparse_conv::takeRowMap(api, handle, announced_map, GatherDirection::kBackwardData, &p);
   if (st != MLUOP_STATUS_SUCCESS) return st;
+  // what this call overwrites is no pair tensor any more, whatever the handle noted there
+  mluop::sparse_conv::forgetRulebookNotesIn(handle, input_grad, input_grad_desc->total_tensor_size);
+  mluop::sparse_conv::forgetRulebookNotesIn(handle, workspace, workspace_size);
   // result rows are named by pair column 0 (the other one in an inverse convolution)
   mluop::sparse_conv::consultRulebookNotes(handle, p.inverse ? 1 : 0, &p);
   const size_t need =

@@ -12,6 +12,7 @@
 #include "core/gen_case.h"
 #include "mlu_op_ext.h"
 #include "sparse_conv/indice_conv.h"
+#include "sparse_conv/rulebook_notes.h"
 #include "sparse_conv/no_alloc_scratch.h"
 
 namespace {
@@ -292,6 +293,8 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionBackwardFilter(
     c.finish(0.003);
   }
   DEVICE_HANDLE_CHECK(api, handle);
+  mluop::sparse_conv::forgetRulebookNotesIn(handle, filters_grad, filters_grad_desc->total_tensor_size);
+  mluop::sparse_conv::forgetRulebookNotesIn(handle, workspace, workspace_size);
   HIP_CHECK_RETURN(api, mluop::sparse_conv::launchBackwardFilter(handle->launchCtx(), p, features,
                                                                 output_grad, workspace,
                                                                 filters_grad));

@@ -244,6 +244,9 @@ mluOpStatus_t MLUOP_WIN_API mluOpIndiceConvolutionForward(
   p.distinct_pairs = handle->distinct_pairs_promised;
   st = mluop::sparse_conv::takeRowMap(api, handle, announced_map, GatherDirection::kForward, &p);
   if (st != MLUOP_STATUS_SUCCESS) return st;
+  // what this call overwrites is no pair tensor any more, whatever the handle noted there
+  mluop::sparse_conv::forgetRulebookNotesIn(handle, features_out, features_out_desc->total_tensor_size);
+  mluop::sparse_conv::forgetRulebookNotesIn(handle, workspace, workspace_size);
   // result rows are named by pair column 1 (the other one in an inverse convolution)
   mluop::sparse_conv::consultRulebookNotes(handle, p.inverse ? 0 : 1, &p);
   const size_t need = mluop::sparse_conv::gatherConvWorkspaceBytes(p, GatherDirection::kForward);

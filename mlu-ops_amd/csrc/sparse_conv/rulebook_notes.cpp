@@ -55,5 +55,13 @@ void consultRulebookNotes(mluOpContext *handle, int row_column, ConvProblem *p) 
   }
 }
 
+void forgetRulebookNotesIn(mluOpContext *handle, const void *out, size_t bytes) {
+  const char *lo = static_cast<const char *>(out);
+  for (auto &n : handle->rulebook_notes) {
+    const char *at = static_cast<const char *>(n.pairs);
+    if (at != nullptr && at >= lo && at < lo + bytes) n.pairs = nullptr;
+  }
+}
+
 }  // namespace sparse_conv
 }  // namespace mluop

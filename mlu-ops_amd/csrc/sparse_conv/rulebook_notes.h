@@ -19,6 +19,10 @@ RulebookReportTarget openRulebookNote(mluOpContext *handle, const void *pairs, i
 // report that has not arrived yet leaves the question to the kernels.
 void consultRulebookNotes(mluOpContext *handle, int row_column, ConvProblem *p);
 
+// Memory [out, out + bytes) is about to be written by an operator of this handle: a note about
+// a pair tensor that starts inside it describes memory that was handed out again, and is dropped.
+void forgetRulebookNotesIn(mluOpContext *handle, const void *out, size_t bytes);
+
 }  // namespace sparse_conv
 }  // namespace mluop
 
