@@ -1228,12 +1228,32 @@ __global__ __launch_bounds__(kBlock) void rbRankAndDecode(GeomDev g,
 // Moves the staged pairs of kPlaceWaves waves of one offset (workgroup (x, k)) to their
 // final positions: the pairs in front of the chunk are the sum of the earlier waves'
 // counts (a few kilobytes, read by every workgroup of the offset rather than scanned in a
-// launch of its own), wave 0 scans the chunk's own counts, and every wave of the
-// workgroup copies four of the chunk's staged pieces, a lane per pair, all four in flight
-// at once.  In regular mode the staged output cell becomes the output row, its rank among
-// the marked cells.  One thread files the rulebook's report.
+// launch of its own), wave 0 scans the chunk's own counts, and the threads then take the
+// chunk's pairs in their final order, up to eight each with the loads in flight together.
+// In regular mode the staged output cell becomes the output row, its rank among the
+// marked cells.  One thread files the rulebook's report.
 constexpr int kPlaceWaves = 64;
-constexpr int kPlaceBlock = 1024;
+constexpr int kPlaceBlock = 512;
+constexpr int kPlacePer = 8;  // pairs a thread moves per pass, their loads in flight together
+constexpr int kPlaceMaxChunks = 8;
+// chunks of kPlaceWaves waves one workgroup moves in turn: one while the grid stays within a few
+// rounds of workgroups per CU
+static int placeChunksPerGroup(int n_wave, int K) {
+  const long chunks = (n_wave + kPlaceWaves - 1) / kPlaceWaves;
+  int m = 1;
+  while (m < kPlaceMaxChunks && chunks * K / m > 16384) m *= 2;
+  return m;
+}
+// A thread takes the t-th staged pair of the chunk, whichever wave of rows staged it (most
+// waves stage a handful of pairs per offset, so a lane per (wave, slot) would idle): the wave is
+// the last one whose pairs start at or before t.
+__device__ __forceinline__ int placeSegment(const int *s_first, int t) {
+  int seg = 0;
+#pragma unroll
+  for (int step = kPlaceWaves / 2; step > 0; step >>= 1)
+    if (s_first[seg + step] <= t) seg += step;
+  return seg;
+}
 template <bool SUBM>
 __global__ __launch_bounds__(kPlaceBlock) void rbPlacePairs(int L, Staging st,
                                                              const unsigned long long *bitmap,
@@ -1241,21 +1261,21 @@ __global__ __launch_bounds__(kPlaceBlock) void rbPlacePairs(int L, Staging st,
                                                              int32_t *indice_num,
                                                              const int32_t *rows_in_order,
                                                              const unsigned long long *unordered,
-                                                             bool mirror_geometry,
+                                                             bool mirror_geometry, int chunks_per_group,
                                                              RulebookReportTarget report) {
   static_assert(kPlaceWaves == kWave, "one lane per wave count in the scan");
   constexpr int kWaves = kPlaceBlock / kWave;
-  constexpr int kPieces = kPlaceWaves / kWaves;  // staged pieces per wave
   __shared__ int s_first[kPlaceWaves];  // staged pairs in front of each wave of the chunk
-  __shared__ int s_count[kPlaceWaves];
   __shared__ int s_start[kPlaceWaves];  // where the wave's pairs start in its staging block
+  __shared__ int s_total;
   __shared__ int s_wave_sum[kWaves];
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
     // submanifold: the rows were in cell order unless the word holds the call's stamp
     fileReport(SUBM ? *unordered != report.stamp : *rows_in_order != 0, report);
   }
   const int k = blockIdx.y;
-  const int w0 = blockIdx.x * kPlaceWaves;
+  const int w_first = blockIdx.x * chunks_per_group * kPlaceWaves;
+  const int w_end = min(w_first + chunks_per_group * kPlaceWaves, st.n_wave);
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
@@ -1269,8 +1289,8 @@ __global__ __launch_bounds__(kPlaceBlock) void rbPlacePairs(int L, Staging st,
     if (k > K / 2) return;
     if (k == K / 2) {
       int32_t *in_col = pairs + (size_t)k * 2 * L;
-      const int hi = (w0 + kPlaceWaves) * kWave < L ? (w0 + kPlaceWaves) * kWave : L;
-      for (int r = w0 * kWave + tid; r < hi; r += kPlaceBlock) {
+      const int hi = w_end * kWave < L ? w_end * kWave : L;
+      for (int r = w_first * kWave + tid; r < hi; r += kPlaceBlock) {
         in_col[r] = r;
         in_col[L + r] = r;
       }
@@ -1282,70 +1302,89 @@ __global__ __launch_bounds__(kPlaceBlock) void rbPlacePairs(int L, Staging st,
   }
   const int slice = k / (mirror ? st.mirror_k_per_slice : st.k_per_slice);
   const int32_t *counts = st.counts + (size_t)k * st.n_wave;
-  // pairs of the waves in front of the chunk
+  // (wave 0's share of the first chunk's counts, requested together with the sum's loads)
+  int entry = wave == 0 && w_first + lane < st.n_wave ? counts[w_first + lane] : 0;
+  // pairs of the waves in front of the group's chunks
   int part = 0;
-  for (int i = tid; i < w0; i += kPlaceBlock) part += counts[i] & 0xff;
+  for (int i0 = tid; i0 < w_first; i0 += kPlaceBlock * 8) {
+    int c[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = i0 + j * kPlaceBlock;
+      c[j] = i < w_first ? counts[i] : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) part += c[j] & 0xff;
+  }
   part = waveInclusiveScan(part);
   if (lane == kWave - 1) s_wave_sum[wave] = part;
-  if (wave == 0) {
-    const int entry = w0 + lane < st.n_wave ? counts[w0 + lane] : 0;
-    const int mine = entry & 0xff;
-    const int incl = waveInclusiveScan(mine);
-    s_count[lane] = mine;
-    s_start[lane] = entry >> 8;
-    s_first[lane] = incl - mine;
-  }
   __syncthreads();
   int before = 0;
 #pragma unroll
   for (int w = 0; w < kWaves; ++w) before += s_wave_sum[w];
-  if (blockIdx.x == gridDim.x - 1 && tid == 0) {
-    const int total = before + s_first[kPlaceWaves - 1] + s_count[kPlaceWaves - 1];
-    indice_num[k] = total;
-    if (mirror) indice_num[gridDim.y - 1 - k] = total;
-  }
   int32_t *in_col = pairs + (size_t)k * 2 * L;
   int32_t *out_col = in_col + L;
-  int v[kPieces], from_lane[kPieces];
-#pragma unroll
-  for (int i = 0; i < kPieces; ++i) {
-    const int seg = wave * kPieces + i;
-    v[i] = from_lane[i] = 0;
-    if (lane < s_count[seg]) {
-      const size_t at = stageBlock(st, slice, w0 + seg) + (size_t)(s_start[seg] + lane);
-      v[i] = st.stage[at];
-      if (!SUBM) from_lane[i] = (int)st.stage_lane[at];
+  for (int w0 = w_first; w0 < w_end; w0 += kPlaceWaves) {
+    if (w0 != w_first) __syncthreads();  // the chunk before has been moved
+    if (wave == 0) {
+      if (w0 != w_first) entry = w0 + lane < st.n_wave ? counts[w0 + lane] : 0;
+      const int mine = entry & 0xff;
+      const int incl = waveInclusiveScan(mine);
+      s_start[lane] = entry >> 8;
+      s_first[lane] = incl - mine;
+      if (lane == kWave - 1) s_total = incl;
     }
-  }
-  int out[kPieces];
-  if (!SUBM) {
-    unsigned long long word[kPieces];
-    uint32_t rank[kPieces];
+    __syncthreads();
+    const int total = s_total;
+    for (int t0 = tid; t0 < total; t0 += kPlaceBlock * kPlacePer) {
+      int v[kPlacePer], from_lane[kPlacePer], first_row[kPlacePer];
 #pragma unroll
-    for (int i = 0; i < kPieces; ++i) {
-      const bool live = lane < s_count[wave * kPieces + i];
-      word[i] = live ? bitmap[v[i] >> 6] : 0ull;
-      rank[i] = live ? word_rank[v[i] >> 6] : 0u;
-    }
+      for (int i = 0; i < kPlacePer; ++i) {
+        const int t = t0 + i * kPlaceBlock;
+        v[i] = from_lane[i] = first_row[i] = 0;
+        if (t < total) {
+          const int seg = placeSegment(s_first, t);
+          const size_t at = stageBlock(st, slice, w0 + seg) + (size_t)(s_start[seg] + t - s_first[seg]);
+          first_row[i] = (w0 + seg) * kWave;
+          v[i] = st.stage[at];
+          if (!SUBM) from_lane[i] = (int)st.stage_lane[at];
+        }
+      }
+      int out[kPlacePer];
+      if (!SUBM) {
+        unsigned long long word[kPlacePer];
+        uint32_t rank[kPlacePer];
 #pragma unroll
-    for (int i = 0; i < kPieces; ++i)
-      out[i] = (int)(rank[i] + (uint32_t)__popcll(word[i] & ((1ull << (v[i] & 63)) - 1ull)));
-  }
+        for (int i = 0; i < kPlacePer; ++i) {
+          const bool live = t0 + i * kPlaceBlock < total;
+          word[i] = live ? bitmap[v[i] >> 6] : 0ull;
+          rank[i] = live ? word_rank[v[i] >> 6] : 0u;
+        }
 #pragma unroll
-  for (int i = 0; i < kPieces; ++i) {
-    const int seg = wave * kPieces + i;
-    if (lane < s_count[seg]) {
-      const int first_row = (w0 + seg) * kWave;
-      const int to = before + s_first[seg] + lane;
-      const int row = first_row + (SUBM ? (v[i] & 63) : from_lane[i]);
-      const int partner = SUBM ? v[i] >> 6 : out[i];
-      in_col[to] = row;
-      out_col[to] = partner;
-      if (mirror) {
-        mirror_in[to] = partner;
-        mirror_out[to] = row;
+        for (int i = 0; i < kPlacePer; ++i)
+          out[i] = (int)(rank[i] + (uint32_t)__popcll(word[i] & ((1ull << (v[i] & 63)) - 1ull)));
+      }
+#pragma unroll
+      for (int i = 0; i < kPlacePer; ++i) {
+        const int t = t0 + i * kPlaceBlock;
+        if (t < total) {
+          const int to = before + t;
+          const int row = first_row[i] + (SUBM ? (v[i] & 63) : from_lane[i]);
+          const int partner = SUBM ? v[i] >> 6 : out[i];
+          in_col[to] = row;
+          out_col[to] = partner;
+          if (mirror) {
+            mirror_in[to] = partner;
+            mirror_out[to] = row;
+          }
+        }
       }
     }
+    before += total;
+  }
+  if (blockIdx.x == gridDim.x - 1 && tid == 0) {
+    indice_num[k] = before;
+    if (mirror) indice_num[gridDim.y - 1 - k] = before;
   }
 }
 
@@ -1564,8 +1603,10 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
     lc.end();
   }
   lc.begin("rbPlacePairs");
-  rbPlacePairs<true><<<dim3((ws.n_wave + kPlaceWaves - 1) / kPlaceWaves, g.K), kPlaceBlock, 0, lc.stream>>>(
-      g.L, staging, nullptr, nullptr, indice_pairs, indice_num, nullptr, ws.unordered, mirror, report);
+  const int per_group = placeChunksPerGroup(ws.n_wave, g.K);
+  const int place_groups = (ws.n_wave + kPlaceWaves * per_group - 1) / (kPlaceWaves * per_group);
+  rbPlacePairs<true><<<dim3(place_groups, g.K), kPlaceBlock, 0, lc.stream>>>(
+      g.L, staging, nullptr, nullptr, indice_pairs, indice_num, nullptr, ws.unordered, mirror, per_group, report);
   lc.end();
   return hipGetLastError();
 }
@@ -1647,8 +1688,11 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                   hipMemcpyDeviceToHost, lc.stream);
   if (err != hipSuccess) return err;
   lc.begin("rbPlacePairs");
-  rbPlacePairs<false><<<dim3((ws.n_wave + kPlaceWaves - 1) / kPlaceWaves, g.K), kPlaceBlock, 0, lc.stream>>>(
-      g.L, staging, ws.bitmap, ws.word_rank, indice_pairs, indice_num, ws.rows_in_order, nullptr, false, report);
+  const int per_group = placeChunksPerGroup(ws.n_wave, g.K);
+  const int place_groups = (ws.n_wave + kPlaceWaves * per_group - 1) / (kPlaceWaves * per_group);
+  rbPlacePairs<false><<<dim3(place_groups, g.K), kPlaceBlock, 0, lc.stream>>>(
+      g.L, staging, ws.bitmap, ws.word_rank, indice_pairs, indice_num, ws.rows_in_order, nullptr, false, per_group,
+      report);
   lc.end();
   return hipGetLastError();
 }
