@@ -75,6 +75,13 @@ mluOpStatus_t MLUOP_WIN_API mluOpCreate(mluOpHandle_t *handle) {
   }
   ctx->pinned_scalar = static_cast<int32_t *>(pinned);
   memset(pinned, 0, pinned_bytes);
+  err = hipEventCreateWithFlags(&ctx->readback_event, hipEventDisableTiming | hipEventReleaseToSystem);
+  if (err != hipSuccess) {
+    MLUOP_LOG(ERROR) << "[mluOpCreate] hipEventCreateWithFlags failed: " << hipGetErrorString(err);
+    (void)hipHostFree(pinned);
+    delete ctx;
+    return MLUOP_STATUS_INTERNAL_ERROR;
+  }
   ctx->rulebook_reports =
       reinterpret_cast<mluOpContext::RulebookReport *>(static_cast<char *>(pinned) + 64);
   // Stamps and tickets only have to differ from what earlier calls, of this handle or of
@@ -106,6 +113,7 @@ mluOpStatus_t MLUOP_WIN_API mluOpDestroy(mluOpHandle_t handle) {
       (void)hipGetLastError();
   }
   if (handle->pinned_scalar != nullptr) (void)hipHostFree(handle->pinned_scalar);
+  if (handle->readback_event != nullptr) (void)hipEventDestroy(handle->readback_event);
   handle->timer.destroy();
   delete handle;
   return MLUOP_STATUS_SUCCESS;

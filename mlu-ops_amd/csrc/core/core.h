@@ -33,6 +33,7 @@ struct mluOpContext {
   mluOpQuantizeRoundMode_t round_mode = MLUOP_ROUND_HALF_TO_EVEN;
   mluOpAtomicsMode_t atomics_mode = MLUOP_ATOMICS_NOT_ALLOWED;
   int32_t *pinned_scalar = nullptr;  // 64-byte pinned host slot for read-backs
+  hipEvent_t readback_event = nullptr;  // recorded behind a kernel that stores into the slot
   mluop::KernelTimer timer;          // per-kernel event timing, off by default
   // Modes the reference rejects (inverse convolution, filters_grad written in its
   // tagged layout): off unless mluOpExtSetSparseConvExtendedModes switched them on.

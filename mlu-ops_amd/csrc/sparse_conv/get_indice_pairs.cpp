@@ -222,6 +222,18 @@ mluOpStatus_t MLUOP_WIN_API mluOpGetIndicePairs(
     c.finish(0.0);
   }
   DEVICE_HANDLE_CHECK(api, handle);
+  if (!g.sub_m) {
+    // Regular mode hands the number of output rows to the host descriptor and has to wait for
+    // it: nothing a graph can record.  Refused before anything is enqueued, so that the
+    // caller's capture stays valid.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    HIP_CHECK_RETURN(api, hipStreamIsCapturing(handle->queue, &capturing));
+    if (capturing != hipStreamCaptureStatusNone) {
+      MLUOP_LOG(ERROR) << api << " the handle's queue is being captured into a graph, and a rulebook that is not "
+                       << "submanifold waits for its output row count: build it outside the capture.";
+      return MLUOP_STATUS_NOT_SUPPORTED;
+    }
+  }
 
   const int32_t *in_rows = static_cast<const int32_t *>(indices);
   int32_t *pairs = static_cast<int32_t *>(indice_pairs);
@@ -242,10 +254,13 @@ mluOpStatus_t MLUOP_WIN_API mluOpGetIndicePairs(
   }
   HIP_CHECK_RETURN(api, mluop::sparse_conv::launchRegularRulebook(handle->launchCtx(), g, in_rows, workspace,
                                                                   pairs, out_rows, counts,
-                                                                  handle->pinned_scalar, report));
-  // The output row count travels back through the host descriptor, which needs
-  // one wait on the queue (the reference waits at normal_get_indice_pairs.cpp:531-533).
-  HIP_CHECK_RETURN(api, hipStreamSynchronize(handle->queue));
+                                                                  handle->pinned_scalar, handle->readback_event,
+                                                                  report));
+  // The output row count travels back through the host descriptor, which needs one wait
+  // (the reference waits for its queue at normal_get_indice_pairs.cpp:531-533): here for the
+  // kernel that numbers the output cells; the one that writes the pair lists runs on behind
+  // it, in queue order like everything the caller enqueues next.
+  HIP_CHECK_RETURN(api, hipEventSynchronize(handle->readback_event));
   const int num_act_out = handle->pinned_scalar[0];
   sparse_conv_desc->num_act_out = num_act_out;
   if (num_act_out > g.out_rows) {

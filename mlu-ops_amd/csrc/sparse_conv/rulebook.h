@@ -46,13 +46,15 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
                               void *workspace, int32_t *indice_pairs, int32_t *out_indices,
                               int32_t *indice_num, const RulebookReportTarget &report);
 
-// Enqueues regular (strided / dilated) rulebook construction and
-// an asynchronous copy of the number of active outputs into `host_num_act_out`
-// (pinned host memory).  The caller synchronises the stream before reading it.
+// Enqueues regular (strided / dilated) rulebook construction.  The kernel that numbers the
+// output cells stores their count into `host_num_act_out` (pinned host memory) and
+// `count_ready` is recorded behind it: the caller waits for that event before reading the
+// count, while the kernel that writes the pair lists may still be running.
 hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                  const int32_t *indices, void *workspace, int32_t *indice_pairs,
                                  int32_t *out_indices, int32_t *indice_num,
-                                 int32_t *host_num_act_out, const RulebookReportTarget &report);
+                                 int32_t *host_num_act_out, hipEvent_t count_ready,
+                                 const RulebookReportTarget &report);
 
 }  // namespace sparse_conv
 }  // namespace mluop

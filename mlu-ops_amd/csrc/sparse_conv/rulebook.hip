@@ -1156,6 +1156,7 @@ __global__ __launch_bounds__(kBlock) void rbRankAndDecode(GeomDev g,
                                                           size_t n_words,
                                                           const int32_t *block_count,
                                                           bool scanned, int32_t *num_act_out,
+                                                          int32_t *host_num_act_out,
                                                           uint32_t *word_rank,
                                                           int32_t *out_indices, bool aligned,
                                                           int out_rows) {
@@ -1190,7 +1191,13 @@ __global__ __launch_bounds__(kBlock) void rbRankAndDecode(GeomDev g,
 #pragma unroll
   for (int x = 0; x < kBlock / kWave; ++x)
     if (x < wave) rank += s_wsum[x];
-  if (!scanned && blockIdx.x == gridDim.x - 1 && threadIdx.x == kBlock - 1) *num_act_out = rank + mine;
+  // the count of output cells, for the device and (pinned memory) for the host
+  if (!scanned && blockIdx.x == gridDim.x - 1 && threadIdx.x == kBlock - 1) {
+    *num_act_out = rank + mine;
+    __hip_atomic_store(host_num_act_out, rank + mine, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+  if (scanned && blockIdx.x == 0 && threadIdx.x == 0)
+    __hip_atomic_store(host_num_act_out, *num_act_out, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   if (w < n_words) word_rank[w] = (uint32_t)rank;
   auto put = [&](size_t cell64, int r) {
     if (r >= out_rows) return;
@@ -1614,7 +1621,8 @@ hipError_t launchSubmRulebook(const LaunchCtx &lc, const RulebookGeom &g, const 
 hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
                                  const int32_t *indices, void *workspace, int32_t *indice_pairs,
                                  int32_t *out_indices, int32_t *indice_num,
-                                 int32_t *host_num_act_out, const RulebookReportTarget &report) {
+                                 int32_t *host_num_act_out, hipEvent_t count_ready,
+                                 const RulebookReportTarget &report) {
   const Workspace ws = carve(g, workspace);
   const GeomDev d = toDev(g);
   const bool al_in = aligned16(indices, indices);
@@ -1681,11 +1689,10 @@ hipError_t launchRegularRulebook(const LaunchCtx &lc, const RulebookGeom &g,
   }
   lc.begin("rbRankAndDecode");
   rbRankAndDecode<<<ws.n_bitmap_blocks, kBlock, 0, lc.stream>>>(d, ws.bitmap, ws.n_words, ws.block_sum,
-                                                             scanned, ws.num_act_out, ws.word_rank,
-                                                             out_indices, al_out, g.out_rows);
+                                                             scanned, ws.num_act_out, host_num_act_out,
+                                                             ws.word_rank, out_indices, al_out, g.out_rows);
   lc.end();
-  hipError_t err = hipMemcpyAsync(host_num_act_out, ws.num_act_out, sizeof(int32_t),
-                                  hipMemcpyDeviceToHost, lc.stream);
+  hipError_t err = hipEventRecord(count_ready, lc.stream);
   if (err != hipSuccess) return err;
   lc.begin("rbPlacePairs");
   const int per_group = placeChunksPerGroup(ws.n_wave, g.K);

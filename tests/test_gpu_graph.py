@@ -268,3 +268,50 @@ def test_a_captured_rulebook_files_no_report_in_host_memory():
         handle.close()
     finally:
         m.GUARD_BYTES = guard_bytes
+
+
+def test_a_regular_rulebook_is_refused_under_capture_and_the_capture_goes_on():
+    """A rulebook that is not submanifold returns its number of output rows through the host
+    descriptor, which takes a wait: during capture the call is refused before it enqueues
+    anything, and what the caller captures after the refusal replays as usual."""
+    import torch
+    import mluop_hip as m
+    rng = np.random.default_rng(36)
+    batch, space, L, ks = 1, (10, 20, 20), 1500, (3, 3, 3)
+    idx = torch.from_numpy(random_voxels(rng, batch, space, L, shuffle=False)).cuda()
+    ospace = m.regular_output_space(space, ks, [1, 1, 1], [2, 2, 2], [1, 1, 1])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    guard_bytes, m.GUARD_BYTES = m.GUARD_BYTES, 0
+    try:
+        with torch.cuda.stream(side):
+            handle = m.make_handle_on_current_stream()
+
+            def submanifold():
+                return m.get_indice_pairs(handle, idx, batch, space, ks, list(space), [1, 1, 1], [1, 1, 1], [1, 1, 1], True)
+
+            def regular():
+                return m.get_indice_pairs(handle, idx, batch, space, ks, ospace, [1, 1, 1], [2, 2, 2], [1, 1, 1], False)
+
+            want_pairs, _, want_num, _ = submanifold()
+            eager = regular()
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                with pytest.raises(m.MluOpError) as refused:
+                    regular()
+                pairs, _, num, _ = submanifold()
+            assert refused.value.status == m.STATUS_NOT_SUPPORTED, refused.value
+            for _ in range(2):
+                pairs.fill_(7)
+                graph.replay()
+                side.synchronize()
+                assert torch.equal(pairs, want_pairs) and torch.equal(num, want_num)
+            # and outside the capture the handle builds regular rulebooks as before
+            again = regular()
+            side.synchronize()
+            assert again[3] == eager[3] and torch.equal(again[0], eager[0]) and torch.equal(again[2], eager[2])
+        torch.cuda.current_stream().wait_stream(side)
+        handle.close()
+    finally:
+        m.GUARD_BYTES = guard_bytes
