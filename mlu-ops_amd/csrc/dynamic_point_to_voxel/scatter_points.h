@@ -19,8 +19,7 @@ struct ScatterShape {
   bool reduce_max;   // max, else mean
 };
 
-// Per-point arrays only; the sort's temporary storage comes on top
-// (libraryWorkspaceBytes needs a current HIP device).
+// Per-point arrays only; the sort's counters come on top (libraryWorkspaceBytes).
 size_t scatterWorkspaceBytes(const ScatterShape &s, size_t library_bytes);
 hipError_t libraryWorkspaceBytes(const ScatterShape &s, hipStream_t stream, size_t *bytes);
 

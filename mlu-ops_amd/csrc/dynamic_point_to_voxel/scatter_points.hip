@@ -24,8 +24,7 @@
 #include <hip/hip_runtime.h>
 #include <cstring>
 
-#include <rocprim/device/device_radix_sort.hpp>
-#include <rocprim/device/device_scan.hpp>
+#include "core/device_sort.h"
 
 #include "dynamic_point_to_voxel/scatter_points.h"
 
@@ -241,7 +240,7 @@ struct Workspace {
 Workspace carve(void *base, const ScatterShape &s, size_t library_bytes) {
   const size_t n = (size_t)s.num_points;
   // Blocks start at the caller's pointer rounded up to 256 bytes (64-bit keys, packed sort
-  // keys and the library's temporary storage need their alignment whatever the caller
+  // keys and the sort's counters need their alignment whatever the caller
   // passes); the reported size includes that slack.  A null base only measures.
   char *p = base ? reinterpret_cast<char *>(alignUp(reinterpret_cast<uintptr_t>(base))) : nullptr;
   size_t off = 0;
@@ -278,21 +277,8 @@ size_t scatterWorkspaceBytes(const ScatterShape &s, size_t library_bytes) {
 }
 
 hipError_t libraryWorkspaceBytes(const ScatterShape &s, hipStream_t stream, size_t *bytes) {
-  size_t sort_bytes = 0, scan_bytes = 0;
-  uint32_t *u = nullptr;
-  hipError_t e = rocprim::radix_sort_pairs(nullptr, sort_bytes, u, u, u, u, (size_t)s.num_points, 0,
-                                           32, stream);
-  if (e != hipSuccess) return e;
-  size_t sort64_bytes = 0;
-  unsigned long long *u64 = nullptr;
-  e = rocprim::radix_sort_pairs(nullptr, sort64_bytes, u64, u64, u, u, (size_t)s.num_points, 0, 64,
-                                stream);
-  if (e != hipSuccess) return e;
-  e = rocprim::inclusive_scan(nullptr, scan_bytes, u, u, (size_t)s.num_points,
-                              rocprim::plus<uint32_t>(), stream);
-  if (e != hipSuccess) return e;
-  sort_bytes = sort_bytes > sort64_bytes ? sort_bytes : sort64_bytes;
-  *bytes = sort_bytes > scan_bytes ? sort_bytes : scan_bytes;
+  (void)stream;
+  *bytes = device_sort::workspaceBytes((size_t)s.num_points);
   return hipSuccess;
 }
 
@@ -331,20 +317,20 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
   uint32_t *pts_in = w.points_a, *pts_out = w.points_b;
   bool packed = false;
   const int total_bits = bits[0] + bits[1] + bits[2];
+  bool in_b = false;  // which pair of arrays a sort left its result in
   if (total_bits <= 64) {
-    size_t lib = library_bytes;
     if (total_bits <= 32) {
       lc.begin("dpvPackKeys");
       dpvPackKeys<uint32_t><<<blocks, kBlock, 0, lc.stream>>>(coors, n, bits[1], bits[2], w.keys_a);
       lc.end();
       if ((e = hipGetLastError()) != hipSuccess) return e;
       lc.begin("radixSortPairs");
-      e = rocprim::radix_sort_pairs(w.library, lib, w.keys_a, w.keys_b, pts_in, pts_out, (size_t)n,
-                                    0, total_bits, lc.stream);
+      e = device_sort::sortPairs<uint32_t>(lc.stream, w.library, w.keys_a, w.keys_b, pts_in, pts_out,
+                                           (size_t)n, total_bits, &in_b);
       lc.end();
       if (e != hipSuccess) return e;
       lc.begin("dpvHeads");
-      dpvHeadsFromKeys<uint32_t><<<blocks, kBlock, 0, lc.stream>>>(w.keys_b, n, w.head);
+      dpvHeadsFromKeys<uint32_t><<<blocks, kBlock, 0, lc.stream>>>(in_b ? w.keys_b : w.keys_a, n, w.head);
       lc.end();
     } else {
       unsigned long long *ka = reinterpret_cast<unsigned long long *>(w.keys_a);
@@ -354,16 +340,16 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
       lc.end();
       if ((e = hipGetLastError()) != hipSuccess) return e;
       lc.begin("radixSortPairs");
-      e = rocprim::radix_sort_pairs(w.library, lib, ka, kb, pts_in, pts_out, (size_t)n, 0,
-                                    total_bits, lc.stream);
+      e = device_sort::sortPairs<unsigned long long>(lc.stream, w.library, ka, kb, pts_in, pts_out,
+                                                     (size_t)n, total_bits, &in_b);
       lc.end();
       if (e != hipSuccess) return e;
       lc.begin("dpvHeads");
-      dpvHeadsFromKeys<unsigned long long><<<blocks, kBlock, 0, lc.stream>>>(kb, n, w.head);
+      dpvHeadsFromKeys<unsigned long long><<<blocks, kBlock, 0, lc.stream>>>(in_b ? kb : ka, n, w.head);
       lc.end();
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
-    pts_in = pts_out;
+    if (in_b) pts_in = pts_out;
     packed = true;
   } else {
     // last axis first; every pass is stable, so the final order is lexicographic
@@ -376,14 +362,15 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
         if ((e = hipGetLastError()) != hipSuccess) return e;
       }
       lc.begin("radixSortPairs");
-      size_t lib = library_bytes;
-      e = rocprim::radix_sort_pairs(w.library, lib, w.keys_a, w.keys_b, pts_in, pts_out, (size_t)n,
-                                    0, bits[axis], lc.stream);
+      e = device_sort::sortPairs<uint32_t>(lc.stream, w.library, w.keys_a, w.keys_b, pts_in, pts_out,
+                                           (size_t)n, bits[axis], &in_b);
       lc.end();
       if (e != hipSuccess) return e;
-      uint32_t *t = pts_in;
-      pts_in = pts_out;
-      pts_out = t;
+      if (in_b) {
+        uint32_t *t = pts_in;
+        pts_in = pts_out;
+        pts_out = t;
+      }
     }
   }
   const uint32_t *sorted_points = pts_in;
@@ -395,9 +382,7 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   lc.begin("inclusiveScan");
-  size_t lib = library_bytes;
-  e = rocprim::inclusive_scan(w.library, lib, w.head, w.triple_count, (size_t)n,
-                              rocprim::plus<uint32_t>(), lc.stream);
+  e = device_sort::prefixSums(lc.stream, w.library, w.head, w.triple_count, (size_t)n, true);
   lc.end();
   if (e != hipSuccess) return e;
 

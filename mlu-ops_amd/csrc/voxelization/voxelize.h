@@ -27,8 +27,7 @@ constexpr int64_t kMaxPoints = (int64_t)1 << 28;
 // `library_bytes` for the sort and the scan (from libraryWorkspaceBytes).
 size_t voxelizeWorkspaceBytes(const VoxelizeShape &s, size_t library_bytes);
 
-// Temporary storage the device-wide sort and scan ask for at this size; needs
-// a current HIP device.
+// Counters the sort and the scan want at this size.
 hipError_t libraryWorkspaceBytes(const VoxelizeShape &s, hipStream_t stream, size_t *bytes);
 
 // Enqueues the whole operator: outputs zero-filled, then written.

@@ -25,8 +25,7 @@
 #include <hip/hip_runtime.h>
 #include <cstring>
 
-#include <rocprim/device/device_radix_sort.hpp>
-#include <rocprim/device/device_scan.hpp>
+#include "core/device_sort.h"
 
 #include "voxelization/voxelize.h"
 
@@ -228,7 +227,7 @@ Workspace carve(void *base, const VoxelizeShape &s, size_t library_bytes) {
   const size_t n = (size_t)s.num_points;
   const uint32_t cap = tableSlots(s.num_points);
   // Blocks start at the caller's pointer rounded up to 256 bytes (64-bit keys, packed sort
-  // keys and the library's temporary storage need their alignment whatever the caller
+  // keys and the sort's counters need their alignment whatever the caller
   // passes); the reported size includes that slack.  A null base only measures.
   char *p = base ? reinterpret_cast<char *>(alignUp(reinterpret_cast<uintptr_t>(base))) : nullptr;
   size_t off = 0;
@@ -260,16 +259,8 @@ size_t voxelizeWorkspaceBytes(const VoxelizeShape &s, size_t library_bytes) {
 }
 
 hipError_t libraryWorkspaceBytes(const VoxelizeShape &s, hipStream_t stream, size_t *bytes) {
-  const uint32_t cap = tableSlots(s.num_points);
-  size_t sort_bytes = 0, scan_bytes = 0;
-  uint32_t *u = nullptr;
-  hipError_t e = rocprim::radix_sort_pairs(nullptr, sort_bytes, u, u, u, u, (size_t)s.num_points, 0,
-                                           bitsFor(cap), stream);
-  if (e != hipSuccess) return e;
-  e = rocprim::exclusive_scan(nullptr, scan_bytes, u, u, 0u, (size_t)s.num_points,
-                              rocprim::plus<uint32_t>(), stream);
-  if (e != hipSuccess) return e;
-  *bytes = sort_bytes > scan_bytes ? sort_bytes : scan_bytes;
+  (void)stream;
+  *bytes = device_sort::workspaceBytes((size_t)s.num_points);
   return hipSuccess;
 }
 
@@ -314,31 +305,32 @@ hipError_t launchVoxelize(const LaunchCtx &lc, const VoxelizeShape &s, const flo
   lc.end();
   if ((e = hipGetLastError()) != hipSuccess) return e;
 
+  // points grouped by table slot, the points of a slot in their input order
   lc.begin("radixSortPairs");
-  size_t lib = library_bytes;
-  e = rocprim::radix_sort_pairs(w.library, lib, w.slot_of, w.slot_sorted, w.point_of,
-                                w.point_sorted, (size_t)n, 0, bitsFor(cap), lc.stream);
+  bool in_b = false;
+  e = device_sort::sortPairs<uint32_t>(lc.stream, w.library, w.slot_of, w.slot_sorted, w.point_of,
+                                       w.point_sorted, (size_t)n, bitsFor(cap), &in_b);
   lc.end();
   if (e != hipSuccess) return e;
+  const uint32_t *slot_sorted = in_b ? w.slot_sorted : w.slot_of;
+  const uint32_t *point_sorted = in_b ? w.point_sorted : w.point_of;
 
   lc.begin("voxHeads");
-  voxHeads<<<blocks, kBlock, 0, lc.stream>>>(w.slot_sorted, n, cap, w.head);
+  voxHeads<<<blocks, kBlock, 0, lc.stream>>>(slot_sorted, n, cap, w.head);
   lc.end();
   if ((e = hipGetLastError()) != hipSuccess) return e;
 
-  // the unsorted pair arrays are free again: they take rank and first point
-  int32_t *rank = reinterpret_cast<int32_t *>(w.slot_of);
-  int32_t *first = reinterpret_cast<int32_t *>(w.point_of);
+  // the other pair of arrays is free again: it takes rank and first point
+  int32_t *rank = reinterpret_cast<int32_t *>(in_b ? w.slot_of : w.slot_sorted);
+  int32_t *first = reinterpret_cast<int32_t *>(in_b ? w.point_of : w.point_sorted);
   lc.begin("voxRanks");
-  voxRanks<<<blocks, kBlock, 0, lc.stream>>>(w.slot_sorted, w.point_sorted, w.head, n, cap, rank,
-                                              first, w.is_first);
+  voxRanks<<<blocks, kBlock, 0, lc.stream>>>(slot_sorted, point_sorted, w.head, n, cap, rank, first,
+                                              w.is_first);
   lc.end();
   if ((e = hipGetLastError()) != hipSuccess) return e;
 
   lc.begin("exclusiveScan");
-  lib = library_bytes;
-  e = rocprim::exclusive_scan(w.library, lib, w.is_first, w.voxel_of_first, 0u, (size_t)n,
-                              rocprim::plus<uint32_t>(), lc.stream);
+  e = device_sort::prefixSums(lc.stream, w.library, w.is_first, w.voxel_of_first, (size_t)n, false);
   lc.end();
   if (e != hipSuccess) return e;
 

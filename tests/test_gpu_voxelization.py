@@ -121,3 +121,46 @@ def test_points_at_an_odd_address(gpu_handle):
         torch.cuda.synchronize()
         got = (out[0].cpu().numpy(), out[1].cpu().numpy(), out[2].cpu().numpy(), int(out[3].item()))
         assert_same(got, expect)
+
+
+def test_captured_voxelization_replays_bit_exactly():
+    """The operator enqueues kernels only (its sort and prefix sums are the library's own: no
+    memset node, no wait), so a caller can capture it into a HIP graph.  Three replays with eager
+    work and waits between them, on points that change between replays, each against the eager
+    result for the same points."""
+    import torch
+    import mluop_hip
+    rng = np.random.default_rng(12)
+    n, max_points, max_voxels = 20000, 4, 3000
+    vs_np, cr_np = [0.4, 0.4, 1.0], [0.0, -4.0, -2.0, 8.0, 4.0, 1.0]
+    clouds = [lidar_like_points(rng, n, features=4, spread=(8.0, 4.0, 2.0)) for _ in range(3)]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    guard_bytes, mluop_hip.GUARD_BYTES = mluop_hip.GUARD_BYTES, 0
+    try:
+        with torch.cuda.stream(side):
+            handle = mluop_hip.make_handle_on_current_stream()
+            pts = torch.from_numpy(clouds[0]).cuda()
+            vs = torch.tensor(vs_np, dtype=torch.float32).cuda()
+            cr = torch.tensor(cr_np, dtype=torch.float32).cuda()
+            mluop_hip.voxelization(handle, pts, vs, cr, max_points, max_voxels)   # first call outside the capture
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                captured = mluop_hip.voxelization(handle, pts, vs, cr, max_points, max_voxels)
+            for cloud in clouds:
+                pts.copy_(torch.from_numpy(cloud).cuda())
+                for t in captured:
+                    t.fill_(-7)
+                graph.replay()
+                side.synchronize()
+                eager = mluop_hip.voxelization(handle, pts, vs, cr, max_points, max_voxels)
+                side.synchronize()
+                for name, got, want in zip(("voxels", "coors", "num_points_per_voxel", "voxel_num"), captured, eager):
+                    assert torch.equal(got, want), name
+                got = tuple(t.cpu().numpy() for t in captured[:3]) + (int(captured[3].item()),)
+                assert_same(got, vox.voxelization(cloud, vs_np, cr_np, max_points, max_voxels))
+        torch.cuda.current_stream().wait_stream(side)
+        handle.close()
+    finally:
+        mluop_hip.GUARD_BYTES = guard_bytes
