@@ -276,7 +276,9 @@ hipError_t sortPairs(hipStream_t stream, void *workspace, K *keys_a, K *keys_b, 
 
 // ---- prefix sums over n counts --------------------------------------------------------
 
-static __global__ __launch_bounds__(kSortThreads) void scanTileSums(const uint32_t *__restrict__ in, size_t n,
+// (BITS: the counts are the numbers of set bits of the words of `in`)
+template <bool BITS>
+__global__ __launch_bounds__(kSortThreads) void scanTileSums(const uint32_t *__restrict__ in, size_t n,
                                                              uint32_t *__restrict__ sums) {
   __shared__ uint32_t s_wave[kSortWaves];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -285,7 +287,8 @@ static __global__ __launch_bounds__(kSortThreads) void scanTileSums(const uint32
 #pragma unroll
   for (int j = 0; j < kScanTile / kSortThreads; ++j) {
     const size_t i = base + (size_t)j * kSortThreads + tid;
-    sum += i < n ? in[i] : 0u;
+    const uint32_t word = i < n ? in[i] : 0u;
+    sum += BITS ? (uint32_t)__popc(word) : word;
   }
   const uint32_t incl = waveInclusiveSum(sum);
   if (lane == 63) s_wave[wave] = incl;
@@ -297,7 +300,7 @@ static __global__ __launch_bounds__(kSortThreads) void scanTileSums(const uint32
   }
 }
 
-template <bool INCLUSIVE>
+template <bool INCLUSIVE, bool BITS>
 __global__ __launch_bounds__(kSortThreads) void scanTiles(const uint32_t *__restrict__ in,
                                                           uint32_t *__restrict__ out, size_t n,
                                                           const uint32_t *__restrict__ tile_first) {
@@ -309,7 +312,8 @@ __global__ __launch_bounds__(kSortThreads) void scanTiles(const uint32_t *__rest
 #pragma unroll
   for (int j = 0; j < kScanChunks; ++j) {
     const size_t i = base + (size_t)j * 64 + lane;
-    v[j] = i < n ? in[i] : 0u;
+    const uint32_t word = i < n ? in[i] : 0u;
+    v[j] = BITS ? (uint32_t)__popc(word) : word;
     mine += v[j];
   }
   // the wave's total, then the waves before it
@@ -329,18 +333,29 @@ __global__ __launch_bounds__(kSortThreads) void scanTiles(const uint32_t *__rest
   }
 }
 
-// out[i] = in[0] + ... + in[i] (inclusive) or without in[i] (exclusive).  `workspace` as above.
+// out[i] = c[0] + ... + c[i] (inclusive) or without c[i] (exclusive), where c[i] = in[i], or
+// the number of set bits of in[i] with `count_bits`.  `workspace` as above.
 inline hipError_t prefixSums(hipStream_t stream, void *workspace, const uint32_t *in, uint32_t *out,
-                             size_t n, bool inclusive) {
+                             size_t n, bool inclusive, bool count_bits = false) {
   if (n == 0) return hipSuccess;
   const int tiles = (int)((n + kScanTile - 1) / kScanTile);
   uint32_t *sums = reinterpret_cast<uint32_t *>((reinterpret_cast<uintptr_t>(workspace) + 255) / 256 * 256);
-  scanTileSums<<<tiles, kSortThreads, 0, stream>>>(in, n, sums);
-  scanCounters<<<1, kScanThreads, 0, stream>>>(sums, (size_t)tiles);
-  if (inclusive)
-    scanTiles<true><<<tiles, kSortThreads, 0, stream>>>(in, out, n, sums);
+  if (count_bits)
+    scanTileSums<true><<<tiles, kSortThreads, 0, stream>>>(in, n, sums);
   else
-    scanTiles<false><<<tiles, kSortThreads, 0, stream>>>(in, out, n, sums);
+    scanTileSums<false><<<tiles, kSortThreads, 0, stream>>>(in, n, sums);
+  scanCounters<<<1, kScanThreads, 0, stream>>>(sums, (size_t)tiles);
+  if (count_bits) {
+    if (inclusive)
+      scanTiles<true, true><<<tiles, kSortThreads, 0, stream>>>(in, out, n, sums);
+    else
+      scanTiles<false, true><<<tiles, kSortThreads, 0, stream>>>(in, out, n, sums);
+  } else {
+    if (inclusive)
+      scanTiles<true, false><<<tiles, kSortThreads, 0, stream>>>(in, out, n, sums);
+    else
+      scanTiles<false, false><<<tiles, kSortThreads, 0, stream>>>(in, out, n, sums);
+  }
   return hipGetLastError();
 }
 

@@ -13,13 +13,14 @@
 //   2 radix sort     (slot, point index) pairs by slot, least significant
 //                    digit first and therefore stable: every cell's points end
 //                    up adjacent and in point order
-//   3 voxHeads       first sorted position of every cell
-//   4 voxRanks       position of a point in its cell = sorted position - head;
-//                    the cell's first point = the point at the head
-//   5 exclusive scan over "is the first point of its cell" in point order:
-//                    the voxel number of every cell, as the sequential
-//                    numbering of the reference gives it
-//   6 voxAssign      copies points and coordinates, counts points per voxel
+//   3 voxMarkFirst   the first point of every cell (the point at the head of the cell's
+//                    run) raises its flag in an array over the points
+//   4 prefix sums over the flags: the voxel number of a cell is the number of first
+//                    points in front of its own, which is the sequential numbering of the
+//                    reference
+//   5 voxAssign      in sorted order: position in the cell = sorted position - head of the
+//                    run, voxel number from the bitmap; copies points and coordinates,
+//                    counts points per voxel
 // Integer atomics only (table insertion, per-voxel counts): the outputs are
 // the same bits on every run.
 #include <hip/hip_runtime.h>
@@ -56,16 +57,17 @@ int bitsFor(uint32_t cap) {  // slot numbers 0..cap (cap itself marks "no cell")
   return b;
 }
 
-// Up to four regions of 32-bit words filled by one launch.
+// Up to five regions of 32-bit words filled by one launch.
+constexpr int kFillRegions = 5;
 struct FillRegions {
-  uint32_t *base[4];
-  size_t words[4];
-  uint32_t value[4];
+  uint32_t *base[kFillRegions];
+  size_t words[kFillRegions];
+  uint32_t value[kFillRegions];
 };
 
 __global__ __launch_bounds__(kBlock) void voxFillRegions(FillRegions r) {
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
+  for (int g = 0; g < kFillRegions; ++g) {
     // words in front of the first 16-byte boundary, 16-byte stores, words behind the last
     size_t head = ((16 - (reinterpret_cast<uintptr_t>(r.base[g]) & 15)) & 15) / 4;
     head = head < r.words[g] ? head : r.words[g];
@@ -108,30 +110,41 @@ __device__ inline uint32_t mix64(unsigned long long k) {
   return (uint32_t)k;
 }
 
-__global__ __launch_bounds__(kBlock) void voxCellSlots(
-    const float *__restrict__ points, const float *__restrict__ voxel_size,
-    const float *__restrict__ range, int64_t n, int num_features, unsigned long long *keys,
-    uint32_t cap, int32_t *cell_zyx, uint32_t *slot_of, uint32_t *point_of) {
-  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i >= n) return;
+// The cell (z, y, x) of a point, or cz < 0 outside the grid.
+struct Cell {
+  int cz, cy, cx, gy, gx;
+  unsigned long long cells;
+};
+__device__ inline Cell cellOfPoint(const float *__restrict__ p, const float *__restrict__ voxel_size,
+                                   const float *__restrict__ range) {
   const float sx = voxel_size[0], sy = voxel_size[1], sz = voxel_size[2];
   const float x0 = range[0], y0 = range[1], z0 = range[2];
   const int gx = axisCells(x0, range[3], sx);
   const int gy = axisCells(y0, range[4], sy);
   const int gz = axisCells(z0, range[5], sz);
-  const float *p = points + i * num_features;
-  const int cx = cellIndex(p[0], x0, sx, gx);
-  const int cy = cx < 0 ? -1 : cellIndex(p[1], y0, sy, gy);
-  const int cz = cy < 0 ? -1 : cellIndex(p[2], z0, sz, gz);
+  Cell c;
+  c.gx = gx;
+  c.gy = gy;
+  c.cells = (unsigned long long)gz * (unsigned long long)gy * gx;
+  c.cx = cellIndex(p[0], x0, sx, gx);
+  c.cy = c.cx < 0 ? -1 : cellIndex(p[1], y0, sy, gy);
+  c.cz = c.cy < 0 ? -1 : cellIndex(p[2], z0, sz, gz);
+  return c;
+}
+
+__global__ __launch_bounds__(kBlock) void voxCellSlots(
+    const float *__restrict__ points, const float *__restrict__ voxel_size,
+    const float *__restrict__ range, int64_t n, int num_features, unsigned long long *keys,
+    uint32_t cap, uint32_t *slot_of, uint32_t *point_of) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const Cell c = cellOfPoint(points + i * num_features, voxel_size, range);
+  const int cz = c.cz, cy = c.cy, cx = c.cx, gy = c.gy, gx = c.gx;
   point_of[i] = (uint32_t)i;
   if (cz < 0) {
-    cell_zyx[3 * i] = cell_zyx[3 * i + 1] = cell_zyx[3 * i + 2] = -1;
     slot_of[i] = cap;
     return;
   }
-  cell_zyx[3 * i] = cz;
-  cell_zyx[3 * i + 1] = cy;
-  cell_zyx[3 * i + 2] = cx;
   const unsigned long long key =
       ((unsigned long long)cz * (unsigned long long)gy + cy) * (unsigned long long)gx + cx;
   uint32_t slot = mix64(key) & (cap - 1);
@@ -139,8 +152,7 @@ __global__ __launch_bounds__(kBlock) void voxCellSlots(
   // A grid of fewer than 2^32 - 1 cells (the same for every thread) keeps 32-bit
   // keys in the first half of the table: 32-bit compare-and-swap is several times
   // faster than the 64-bit one.
-  const unsigned long long cells = (unsigned long long)gz * (unsigned long long)gy * gx;
-  if (cells < 0xffffffffull) {
+  if (c.cells < 0xffffffffull) {
     uint32_t *keys32 = reinterpret_cast<uint32_t *>(keys);
     const uint32_t key32 = (uint32_t)key;
     while (true) {
@@ -158,66 +170,93 @@ __global__ __launch_bounds__(kBlock) void voxCellSlots(
   slot_of[i] = slot;
 }
 
-__global__ __launch_bounds__(kBlock) void voxHeads(const uint32_t *__restrict__ slot_sorted,
-                                                   int64_t n, uint32_t cap, uint32_t *head) {
+// is_first[f] = 1 <=> point f is the first of its cell (the array was cleared by the fill; a
+// plain store per cell: a bitmap would take an atomic per cell, four times as long).
+__global__ __launch_bounds__(kBlock) void voxMarkFirst(const uint32_t *__restrict__ slot_sorted,
+                                                       const uint32_t *__restrict__ point_sorted,
+                                                       int64_t n, uint32_t cap, uint32_t *is_first) {
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p >= n) return;
   const uint32_t s = slot_sorted[p];
   if (s == cap) return;
-  if (p == 0 || slot_sorted[p - 1] != s) head[s] = (uint32_t)p;
+  if (p == 0 || slot_sorted[p - 1] != s) is_first[point_sorted[p]] = 1u;
 }
 
-__global__ __launch_bounds__(kBlock) void voxRanks(const uint32_t *__restrict__ slot_sorted,
-                                                   const uint32_t *__restrict__ point_sorted,
-                                                   const uint32_t *__restrict__ head, int64_t n,
-                                                   uint32_t cap, int32_t *rank, int32_t *first,
-                                                   uint32_t *is_first) {
-  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (p >= n) return;
-  const uint32_t s = slot_sorted[p];
-  const uint32_t i = point_sorted[p];
-  if (s == cap) {
-    rank[i] = -1;
-    first[i] = -1;
-    is_first[i] = 0;
-    return;
+// First sorted position whose slot is `s`, which lies in front of position `from` (whose slot
+// is `s` as well): doubling steps backwards, then a binary search.
+__device__ inline int64_t headBefore(const uint32_t *__restrict__ slot_sorted, int64_t from, uint32_t s) {
+  int64_t hi = from;  // slot_sorted[hi] == s
+  int64_t step = 1;
+  int64_t lo = hi - step;
+  while (lo >= 0 && slot_sorted[lo] == s) {
+    hi = lo;
+    step *= 2;
+    lo = hi - step;
   }
-  const uint32_t h = head[s];
-  rank[i] = (int32_t)((uint32_t)p - h);
-  first[i] = (int32_t)point_sorted[h];
-  is_first[i] = (uint32_t)p == h ? 1u : 0u;
+  if (lo < 0) {
+    if (slot_sorted[0] == s) return 0;
+    lo = 0;
+  }
+  // slot_sorted[lo] != s, slot_sorted[hi] == s, the run starts in (lo, hi]
+  while (hi - lo > 1) {
+    const int64_t mid = lo + (hi - lo) / 2;
+    if (slot_sorted[mid] == s)
+      hi = mid;
+    else
+      lo = mid;
+  }
+  return hi;
 }
 
+// Thread p takes the point at sorted position p.  The head of its cell's run is the nearest
+// position at or in front of p where the slot changes: found among the lanes of the wave by a
+// running maximum, and looked up behind the wave only by the lanes of a run that began earlier.
 __global__ __launch_bounds__(kBlock) void voxAssign(
-    const float *__restrict__ points, const int32_t *__restrict__ cell_zyx,
-    const int32_t *__restrict__ rank, const int32_t *__restrict__ first,
-    const uint32_t *__restrict__ is_first, const uint32_t *__restrict__ voxel_of_first, int64_t n,
-    int num_features, int max_points, int max_voxels, float *voxels, int32_t *coors,
-    int32_t *num_points_per_voxel, int32_t *voxel_num) {
-  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i >= n) return;
-  if (i == n - 1) {
-    const uint32_t cells = voxel_of_first[i] + is_first[i];
+    const float *__restrict__ points, const float *__restrict__ voxel_size,
+    const float *__restrict__ range, const uint32_t *__restrict__ slot_sorted,
+    const uint32_t *__restrict__ point_sorted, const uint32_t *__restrict__ is_first,
+    const uint32_t *__restrict__ voxel_of_first, int64_t n, uint32_t cap, int num_features, int max_points,
+    int max_voxels, float *voxels, int32_t *coors, int32_t *num_points_per_voxel, int32_t *voxel_num) {
+  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  if (p == 0) {
+    uint32_t cells = 0;
+    if (n > 0) cells = voxel_of_first[n - 1] + is_first[n - 1];
     *voxel_num = cells < (uint32_t)max_voxels ? (int32_t)cells : max_voxels;
   }
-  const int32_t r = rank[i];
-  if (r < 0 || r >= max_points) return;
-  const uint32_t v = voxel_of_first[first[i]];
+  const bool live = p < n;
+  const uint32_t s = live ? slot_sorted[p] : cap;
+  const uint32_t before = (live && p > 0) ? slot_sorted[p - 1] : cap;
+  const bool starts = live && s != cap && (p == 0 || before != s);
+  // nearest run start at or below this lane, inside the wave (-1: none)
+  long long head = starts ? (long long)p : -1;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const long long up = __shfl_up(head, d, 64);
+    if (lane >= d && up > head) head = up;
+  }
+  if (!live || s == cap) return;
+  if (head < 0) head = headBefore(slot_sorted, p - lane, s);  // (position p - lane holds slot s too)
+  const int64_t r = p - head;
+  if (r >= max_points) return;
+  const uint32_t f = point_sorted[head];
+  const uint32_t v = voxel_of_first[f];  // first points in front of f
   if (v >= (uint32_t)max_voxels) return;
-  const float *src = points + i * num_features;
+  const uint32_t i = point_sorted[p];
+  const float *src = points + (size_t)i * num_features;
   float *dst = voxels + ((size_t)v * max_points + r) * num_features;
-  for (int f = 0; f < num_features; ++f) dst[f] = src[f];
+  for (int k = 0; k < num_features; ++k) dst[k] = src[k];
   atomicAdd(&num_points_per_voxel[v], 1);
   if (r == 0) {
-    coors[3 * (size_t)v] = cell_zyx[3 * i];
-    coors[3 * (size_t)v + 1] = cell_zyx[3 * i + 1];
-    coors[3 * (size_t)v + 2] = cell_zyx[3 * i + 2];
+    const Cell c = cellOfPoint(src, voxel_size, range);
+    coors[3 * (size_t)v] = c.cz;
+    coors[3 * (size_t)v + 1] = c.cy;
+    coors[3 * (size_t)v + 2] = c.cx;
   }
 }
 
 struct Workspace {
-  int32_t *cell_zyx;
-  uint32_t *slot_of, *point_of, *slot_sorted, *point_sorted, *is_first, *voxel_of_first, *head;
+  uint32_t *slot_of, *point_of, *slot_sorted, *point_sorted, *is_first, *voxel_of_first;
   unsigned long long *keys;
   void *library;
   size_t total;
@@ -237,14 +276,12 @@ Workspace carve(void *base, const VoxelizeShape &s, size_t library_bytes) {
     return q;
   };
   Workspace w;
-  w.cell_zyx = reinterpret_cast<int32_t *>(take(12 * n));
   w.slot_of = reinterpret_cast<uint32_t *>(take(4 * n));
   w.point_of = reinterpret_cast<uint32_t *>(take(4 * n));
   w.slot_sorted = reinterpret_cast<uint32_t *>(take(4 * n));
   w.point_sorted = reinterpret_cast<uint32_t *>(take(4 * n));
   w.is_first = reinterpret_cast<uint32_t *>(take(4 * n));
   w.voxel_of_first = reinterpret_cast<uint32_t *>(take(4 * n));
-  w.head = reinterpret_cast<uint32_t *>(take(4 * (size_t)cap));
   w.keys = reinterpret_cast<unsigned long long *>(take(8 * (size_t)cap));
   w.library = take(library_bytes);
   w.total = off + 256;
@@ -276,8 +313,8 @@ hipError_t launchVoxelize(const LaunchCtx &lc, const VoxelizeShape &s, const flo
   const Workspace w = carve(workspace, s, library_bytes);
   if (w.total > workspace_bytes) return hipErrorInvalidValue;
 
-  // outputs start from zero (reference kernels/voxelization/voxelization.cpp:283-309)
-  // and the cell table from "empty"
+  // outputs start from zero (reference kernels/voxelization/voxelization.cpp:283-309),
+  // the cell table from "empty" and the flags of first points from none raised
   FillRegions fr;
   fr.base[0] = reinterpret_cast<uint32_t *>(voxels);
   fr.words[0] = (size_t)s.max_voxels * s.max_points * s.num_features;
@@ -287,8 +324,10 @@ hipError_t launchVoxelize(const LaunchCtx &lc, const VoxelizeShape &s, const flo
   fr.words[2] = (size_t)s.max_voxels;
   fr.base[3] = reinterpret_cast<uint32_t *>(w.keys);
   fr.words[3] = (size_t)cap * 2;
+  fr.base[4] = w.is_first;
+  fr.words[4] = (size_t)n;
   size_t most = 0;
-  for (int g = 0; g < 4; ++g) {
+  for (int g = 0; g < kFillRegions; ++g) {
     fr.value[g] = g == 3 ? 0xffffffffu : 0u;
     most = fr.words[g] > most ? fr.words[g] : most;
   }
@@ -300,8 +339,7 @@ hipError_t launchVoxelize(const LaunchCtx &lc, const VoxelizeShape &s, const flo
   const int blocks = gridFor((size_t)n);
   lc.begin("voxCellSlots");
   voxCellSlots<<<blocks, kBlock, 0, lc.stream>>>(points, voxel_size, coors_range, n,
-                                                  s.num_features, w.keys, cap, w.cell_zyx,
-                                                  w.slot_of, w.point_of);
+                                                  s.num_features, w.keys, cap, w.slot_of, w.point_of);
   lc.end();
   if ((e = hipGetLastError()) != hipSuccess) return e;
 
@@ -315,30 +353,22 @@ hipError_t launchVoxelize(const LaunchCtx &lc, const VoxelizeShape &s, const flo
   const uint32_t *slot_sorted = in_b ? w.slot_sorted : w.slot_of;
   const uint32_t *point_sorted = in_b ? w.point_sorted : w.point_of;
 
-  lc.begin("voxHeads");
-  voxHeads<<<blocks, kBlock, 0, lc.stream>>>(slot_sorted, n, cap, w.head);
+  lc.begin("voxMarkFirst");
+  voxMarkFirst<<<blocks, kBlock, 0, lc.stream>>>(slot_sorted, point_sorted, n, cap, w.is_first);
   lc.end();
   if ((e = hipGetLastError()) != hipSuccess) return e;
 
-  // the other pair of arrays is free again: it takes rank and first point
-  int32_t *rank = reinterpret_cast<int32_t *>(in_b ? w.slot_of : w.slot_sorted);
-  int32_t *first = reinterpret_cast<int32_t *>(in_b ? w.point_of : w.point_sorted);
-  lc.begin("voxRanks");
-  voxRanks<<<blocks, kBlock, 0, lc.stream>>>(slot_sorted, point_sorted, w.head, n, cap, rank, first,
-                                              w.is_first);
-  lc.end();
-  if ((e = hipGetLastError()) != hipSuccess) return e;
-
+  // first points in front of every point
   lc.begin("exclusiveScan");
   e = device_sort::prefixSums(lc.stream, w.library, w.is_first, w.voxel_of_first, (size_t)n, false);
   lc.end();
   if (e != hipSuccess) return e;
 
   lc.begin("voxAssign");
-  voxAssign<<<blocks, kBlock, 0, lc.stream>>>(points, w.cell_zyx, rank, first, w.is_first,
-                                               w.voxel_of_first, n, s.num_features, s.max_points,
-                                               s.max_voxels, voxels, coors, num_points_per_voxel,
-                                               voxel_num);
+  voxAssign<<<blocks, kBlock, 0, lc.stream>>>(points, voxel_size, coors_range, slot_sorted, point_sorted,
+                                               w.is_first, w.voxel_of_first, n, cap, s.num_features,
+                                               s.max_points, s.max_voxels, voxels, coors,
+                                               num_points_per_voxel, voxel_num);
   lc.end();
   return hipGetLastError();
 }
