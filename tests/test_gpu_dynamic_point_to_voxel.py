@@ -64,6 +64,21 @@ def test_matches_oracle(gpu_handle, mode, case):
     assert_same(run_gpu(gpu_handle, mode, feats, coors), dpv.forward(mode, feats, coors))
 
 
+@pytest.mark.parametrize("n", [2, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 2049, 4095, 4097, 70001])
+def test_point_counts_around_the_sort_boundaries(gpu_handle, n):
+    """The grouping sort takes 64 pairs a wave at a time, 256 a wave, 1024 a workgroup: point
+    counts on both sides of those, with few distinct triples (long runs of equal keys, whose
+    points must keep their order for the mean to come out bit for bit) and with many."""
+    rng = np.random.default_rng(100 + n)
+    feats = rng.uniform(-100, 100, (n, 3)).astype(np.float32)
+    for span in (2, 300):
+        coors = rng.integers(0, span, (n, 3)).astype(np.int32)
+        coors[:: max(n // 7, 1), 2] = -1
+        assert_same(run_gpu(gpu_handle, "mean", feats, coors), dpv.forward("mean", feats, coors))
+    same = np.full((n, 3), 5, np.int32)   # one voxel holds every point
+    assert_same(run_gpu(gpu_handle, "mean", feats, same), dpv.forward("mean", feats, same))
+
+
 def test_fewer_output_rows_than_voxels_and_all_invalid(gpu_handle):
     rng = np.random.default_rng(7)
     feats = rng.uniform(-1, 1, (400, 3)).astype(np.float32)
