@@ -13,8 +13,9 @@
 //                (pairs of lower digits) + (of the digit in earlier tiles) + (in earlier waves of the tile) +
 //                (in earlier chunks of the wave) + (in lower lanes of the chunk), which is what
 //                keeps equal keys in their input order.
-// Lanes that hold the same digit find each other with eight ballots (one per bit), so a
-// digit that nearly every key shares costs what a rare one costs: no atomics anywhere.
+// In the scatter, lanes that hold the same digit find each other with eight ballots (one per
+// bit), so a digit that nearly every key shares costs what a rare one costs; the only atomics
+// are the count's integer adds in LDS.
 #ifndef MLUOP_AMD_CORE_DEVICE_SORT_H_
 #define MLUOP_AMD_CORE_DEVICE_SORT_H_
 
@@ -71,31 +72,23 @@ __device__ __forceinline__ unsigned long long lanesWithSameDigit(uint32_t digit,
 template <typename K>
 __global__ __launch_bounds__(kSortThreads) void sortCount(const K *__restrict__ keys, size_t n, int shift,
                                                           uint32_t *__restrict__ hist, int tiles) {
-  __shared__ uint32_t s_count[kSortWaves][kRadix];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int i = tid; i < kSortWaves * kRadix; i += kSortThreads) (&s_count[0][0])[i] = 0;
+  __shared__ uint32_t s_count[kRadix];
+  const int tid = threadIdx.x;
+  s_count[tid] = 0;
   __syncthreads();
-  const size_t base = (size_t)blockIdx.x * kSortTile + (size_t)wave * kSortWaveItems;
-  K key[kSortChunks];
+  const size_t base = (size_t)blockIdx.x * kSortTile;
+  K key[kSortTile / kSortThreads];
 #pragma unroll
-  for (int j = 0; j < kSortChunks; ++j) {
-    const size_t i = base + (size_t)j * 64 + lane;
+  for (int j = 0; j < kSortTile / kSortThreads; ++j) {
+    const size_t i = base + (size_t)j * kSortThreads + tid;
     key[j] = i < n ? keys[i] : (K)0;
   }
-  volatile uint32_t *mine = s_count[wave];
+  // (integer adds in LDS: the order they land in does not matter for a count)
 #pragma unroll
-  for (int j = 0; j < kSortChunks; ++j) {
-    const bool valid = base + (size_t)j * 64 + lane < n;
-    const uint32_t digit = (uint32_t)(key[j] >> shift) & (kRadix - 1);
-    const unsigned long long peers = lanesWithSameDigit(digit, valid);
-    // the lowest lane of a digit adds the chunk's count; a wave's LDS accesses keep their order
-    if (valid && lane == __ffsll((long long)peers) - 1) mine[digit] = mine[digit] + (uint32_t)__popcll(peers);
-  }
+  for (int j = 0; j < kSortTile / kSortThreads; ++j)
+    if (base + (size_t)j * kSortThreads + tid < n) atomicAdd(&s_count[(uint32_t)(key[j] >> shift) & (kRadix - 1)], 1u);
   __syncthreads();
-  uint32_t total = 0;
-#pragma unroll
-  for (int w = 0; w < kSortWaves; ++w) total += s_count[w][tid];
-  hist[(size_t)tid * tiles + blockIdx.x] = total;
+  hist[(size_t)tid * tiles + blockIdx.x] = s_count[tid];
 }
 
 // data[0..m) -> exclusive prefix sums in place, by one workgroup, in rounds of 16 counters a
@@ -177,7 +170,9 @@ static __global__ __launch_bounds__(64) void scanDigitRows(uint32_t *hist, int t
   if (lane == 0) totals[blockIdx.x] = carry;
 }
 
-template <typename K>
+// (VALUES false: keys only; a caller whose value fits beside its key in 64 bits sorts the
+// packed words as keys and halves the scattered stores)
+template <typename K, bool VALUES>
 __global__ __launch_bounds__(kSortThreads) void sortScatter(const K *__restrict__ keys_in,
                                                             const uint32_t *__restrict__ vals_in,
                                                             K *__restrict__ keys_out,
@@ -197,7 +192,7 @@ __global__ __launch_bounds__(kSortThreads) void sortScatter(const K *__restrict_
   for (int j = 0; j < kSortChunks; ++j) {
     const size_t i = base + (size_t)j * 64 + lane;
     key[j] = i < n ? keys_in[i] : (K)0;
-    val[j] = i < n ? vals_in[i] : 0u;
+    val[j] = (VALUES && i < n) ? vals_in[i] : 0u;
   }
   volatile uint32_t *mine = s_count[wave];
   const unsigned long long below = (1ull << lane) - 1ull;
@@ -241,14 +236,14 @@ __global__ __launch_bounds__(kSortThreads) void sortScatter(const K *__restrict_
       const uint32_t digit = (uint32_t)(key[j] >> shift) & (kRadix - 1);
       const size_t to = (size_t)s_first[digit] + s_count[wave][digit] + place[j];
       keys_out[to] = key[j];
-      vals_out[to] = val[j];
+      if (VALUES) vals_out[to] = val[j];
     }
   }
 }
 
 // Sorts the n pairs (keys_a[i], vals_a[i]) by the lowest `bits` bits of the key, equal keys
 // in input order.  Both pairs of arrays are written; *in_b tells which holds the result
-// (true: keys_b / vals_b).  `workspace`: workspaceBytes(n) bytes.
+// (true: keys_b / vals_b).  vals_a == nullptr: keys only.  `workspace`: workspaceBytes(n) bytes.
 template <typename K>
 hipError_t sortPairs(hipStream_t stream, void *workspace, K *keys_a, K *keys_b, uint32_t *vals_a,
                      uint32_t *vals_b, size_t n, int bits, bool *in_b) {
@@ -262,7 +257,11 @@ hipError_t sortPairs(hipStream_t stream, void *workspace, K *keys_a, K *keys_b, 
   for (int shift = 0; shift < bits; shift += kRadixBits) {
     sortCount<K><<<tiles, kSortThreads, 0, stream>>>(kin, n, shift, hist, tiles);
     scanDigitRows<<<kRadix, 64, 0, stream>>>(hist, tiles, totals);
-    sortScatter<K><<<tiles, kSortThreads, 0, stream>>>(kin, vin, kout, vout, n, shift, hist, tiles, totals);
+    if (vals_a != nullptr)
+      sortScatter<K, true><<<tiles, kSortThreads, 0, stream>>>(kin, vin, kout, vout, n, shift, hist, tiles, totals);
+    else
+      sortScatter<K, false><<<tiles, kSortThreads, 0, stream>>>(kin, nullptr, kout, nullptr, n, shift, hist, tiles,
+                                                                totals);
     K *tk = kin;
     kin = kout;
     kout = tk;
@@ -272,6 +271,12 @@ hipError_t sortPairs(hipStream_t stream, void *workspace, K *keys_a, K *keys_b, 
     *in_b = !*in_b;
   }
   return hipGetLastError();
+}
+
+// Keys only.
+template <typename K>
+hipError_t sortKeys(hipStream_t stream, void *workspace, K *keys_a, K *keys_b, size_t n, int bits, bool *in_b) {
+  return sortPairs<K>(stream, workspace, keys_a, keys_b, nullptr, nullptr, n, bits, in_b);
 }
 
 // ---- prefix sums over n counts --------------------------------------------------------

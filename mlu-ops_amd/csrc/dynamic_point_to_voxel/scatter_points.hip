@@ -106,6 +106,28 @@ __global__ __launch_bounds__(kBlock) void dpvPackKeys(const int32_t *__restrict_
   keys[i] = (k0 << (bits1 + bits2)) | (k1 << bits2) | k2;
 }
 
+// The 32-bit packed key in the low half of a 64-bit word and the point index in the high
+// half: sorted as one key by the low bits, the point travels with it (half the scattered
+// stores of a sort of pairs).
+__global__ __launch_bounds__(kBlock) void dpvPackRecords(const int32_t *__restrict__ coors, int n,
+                                                         int bits1, int bits2, unsigned long long *records) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t k0 = (uint32_t)(coors[3 * (size_t)i] + 1);
+  const uint32_t k1 = (uint32_t)(coors[3 * (size_t)i + 1] + 1);
+  const uint32_t k2 = (uint32_t)(coors[3 * (size_t)i + 2] + 1);
+  const uint32_t key = (k0 << (bits1 + bits2)) | (k1 << bits2) | k2;
+  records[i] = ((unsigned long long)(uint32_t)i << 32) | key;
+}
+
+// head[p] = 1 where the key half of the sorted records changes
+__global__ __launch_bounds__(kBlock) void dpvHeadsFromRecords(const unsigned long long *__restrict__ sorted,
+                                                              int n, uint32_t *head) {
+  const int p = blockIdx.x * kBlock + threadIdx.x;
+  if (p >= n) return;
+  head[p] = (p == 0 || (uint32_t)sorted[p] != (uint32_t)sorted[p - 1]) ? 1u : 0u;
+}
+
 // keys[p] = coordinate `axis` of the point at sorted position p, plus one
 __global__ __launch_bounds__(kBlock) void dpvGatherKeys(const int32_t *__restrict__ coors,
                                                         const uint32_t *__restrict__ points, int n,
@@ -137,8 +159,10 @@ __global__ __launch_bounds__(kBlock) void dpvHeads(const int32_t *__restrict__ c
   head[p] = (a[0] != b[0] || a[1] != b[1] || a[2] != b[2]) ? 1u : 0u;
 }
 
+// (`points` holds the sorted point indices `stride` words apart: 1, or 2 where they are the
+// high halves of sorted records)
 __global__ __launch_bounds__(kBlock) void dpvEmit(const int32_t *__restrict__ coors,
-                                                  const uint32_t *__restrict__ points,
+                                                  const uint32_t *__restrict__ points, int stride,
                                                   const uint32_t *__restrict__ head,
                                                   const uint32_t *__restrict__ triple_count, int n,
                                                   int rows, int32_t *point2voxel_map,
@@ -149,7 +173,7 @@ __global__ __launch_bounds__(kBlock) void dpvEmit(const int32_t *__restrict__ co
   // the (-1,-1,-1) triple sorts first and is not a voxel
   const int skipped = coors[3 * (size_t)points[0]] == -1 ? 1 : 0;
   const int v = (int)triple_count[p] - 1 - skipped;
-  const uint32_t i = points[p];
+  const uint32_t i = points[(size_t)p * stride];
   point2voxel_map[i] = v;
   if (head[p] && v >= 0 && v <= rows) {
     first_pos[v] = p;  // one past the last stored voxel included: it ends that voxel
@@ -163,7 +187,7 @@ __global__ __launch_bounds__(kBlock) void dpvEmit(const int32_t *__restrict__ co
 }
 
 __global__ __launch_bounds__(kBlock) void dpvReduce(const float *__restrict__ feats,
-                                                    const uint32_t *__restrict__ points,
+                                                    const uint32_t *__restrict__ points, int stride,
                                                     const int32_t *__restrict__ first_pos,
                                                     const int32_t *__restrict__ voxel_num, int n,
                                                     int num_features, int rows, bool reduce_max,
@@ -182,7 +206,7 @@ __global__ __launch_bounds__(kBlock) void dpvReduce(const float *__restrict__ fe
   if (reduce_max) {
     float best = -INFINITY;
     for (int p = begin; p < stop; ++p) {
-      const float x = feats[(size_t)points[p] * num_features + f];
+      const float x = feats[(size_t)points[(size_t)p * stride] * num_features + f];
       if (x >= best) best = x;
     }
     voxel_feats[t] = best;
@@ -190,7 +214,7 @@ __global__ __launch_bounds__(kBlock) void dpvReduce(const float *__restrict__ fe
     float sum = 0.f;
     const float fcount = (float)count;
     for (int p = begin; p < stop; ++p)
-      sum = __fadd_rn(sum, __fdiv_rn(feats[(size_t)points[p] * num_features + f], fcount));
+      sum = __fadd_rn(sum, __fdiv_rn(feats[(size_t)points[(size_t)p * stride] * num_features + f], fcount));
     voxel_feats[t] = sum;
   }
 }
@@ -318,20 +342,24 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
   bool packed = false;
   const int total_bits = bits[0] + bits[1] + bits[2];
   bool in_b = false;  // which pair of arrays a sort left its result in
+  const uint32_t *record_points = nullptr;  // sorted point indices inside 64-bit records
   if (total_bits <= 64) {
     if (total_bits <= 32) {
+      unsigned long long *ra = reinterpret_cast<unsigned long long *>(w.keys_a);
+      unsigned long long *rb = reinterpret_cast<unsigned long long *>(w.keys_b);
       lc.begin("dpvPackKeys");
-      dpvPackKeys<uint32_t><<<blocks, kBlock, 0, lc.stream>>>(coors, n, bits[1], bits[2], w.keys_a);
+      dpvPackRecords<<<blocks, kBlock, 0, lc.stream>>>(coors, n, bits[1], bits[2], ra);
       lc.end();
       if ((e = hipGetLastError()) != hipSuccess) return e;
       lc.begin("radixSortPairs");
-      e = device_sort::sortPairs<uint32_t>(lc.stream, w.library, w.keys_a, w.keys_b, pts_in, pts_out,
-                                           (size_t)n, total_bits, &in_b);
+      e = device_sort::sortKeys<unsigned long long>(lc.stream, w.library, ra, rb, (size_t)n, total_bits, &in_b);
       lc.end();
       if (e != hipSuccess) return e;
+      const unsigned long long *sorted = in_b ? rb : ra;
       lc.begin("dpvHeads");
-      dpvHeadsFromKeys<uint32_t><<<blocks, kBlock, 0, lc.stream>>>(in_b ? w.keys_b : w.keys_a, n, w.head);
+      dpvHeadsFromRecords<<<blocks, kBlock, 0, lc.stream>>>(sorted, n, w.head);
       lc.end();
+      record_points = reinterpret_cast<const uint32_t *>(sorted) + 1;  // the high halves
     } else {
       unsigned long long *ka = reinterpret_cast<unsigned long long *>(w.keys_a);
       unsigned long long *kb = reinterpret_cast<unsigned long long *>(w.keys_b);
@@ -349,7 +377,7 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
       lc.end();
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
-    if (in_b) pts_in = pts_out;
+    if (in_b && record_points == nullptr) pts_in = pts_out;
     packed = true;
   } else {
     // last axis first; every pass is stable, so the final order is lexicographic
@@ -373,7 +401,8 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
       }
     }
   }
-  const uint32_t *sorted_points = pts_in;
+  const uint32_t *sorted_points = record_points != nullptr ? record_points : pts_in;
+  const int point_stride = record_points != nullptr ? 2 : 1;
 
   if (!packed) {
     lc.begin("dpvHeads");
@@ -387,7 +416,7 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
   if (e != hipSuccess) return e;
 
   lc.begin("dpvEmit");
-  dpvEmit<<<blocks, kBlock, 0, lc.stream>>>(coors, sorted_points, w.head, w.triple_count, n,
+  dpvEmit<<<blocks, kBlock, 0, lc.stream>>>(coors, sorted_points, point_stride, w.head, w.triple_count, n,
                                              s.voxel_rows, point2voxel_map, voxel_coors,
                                              w.first_pos, voxel_num);
   lc.end();
@@ -395,7 +424,7 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
 
   lc.begin("dpvReduce");
   dpvReduce<<<gridFor(feat_words), kBlock, 0, lc.stream>>>(
-      feats, sorted_points, w.first_pos, voxel_num, n, s.num_features, s.voxel_rows, s.reduce_max,
+      feats, sorted_points, point_stride, w.first_pos, voxel_num, n, s.num_features, s.voxel_rows, s.reduce_max,
       voxel_feats, voxel_points_count);
   lc.end();
   return hipGetLastError();

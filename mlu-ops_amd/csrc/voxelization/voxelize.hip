@@ -10,7 +10,7 @@
 // from grouping instead of searching:
 //   1 voxCellSlots   cell of every point; the 64-bit cell id is entered into an
 //                    open-addressing table, whose slot number names the cell
-//   2 radix sort     (slot, point index) pairs by slot, least significant
+//   2 radix sort     (slot, point index) pairs, packed into 64-bit words, by slot, least significant
 //                    digit first and therefore stable: every cell's points end
 //                    up adjacent and in point order
 //   3 voxMarkFirst   the first point of every cell (the point at the head of the cell's
@@ -135,14 +135,16 @@ __device__ inline Cell cellOfPoint(const float *__restrict__ p, const float *__r
 __global__ __launch_bounds__(kBlock) void voxCellSlots(
     const float *__restrict__ points, const float *__restrict__ voxel_size,
     const float *__restrict__ range, int64_t n, int num_features, unsigned long long *keys,
-    uint32_t cap, uint32_t *slot_of, uint32_t *point_of) {
+    uint32_t cap, unsigned long long *slot_and_point) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= n) return;
   const Cell c = cellOfPoint(points + i * num_features, voxel_size, range);
   const int cz = c.cz, cy = c.cy, cx = c.cx, gy = c.gy, gx = c.gx;
-  point_of[i] = (uint32_t)i;
+  // (table slot in the low half, point index in the high half: sorted as one 64-bit key by
+  // the slot's bits, the point travels with it)
+  const unsigned long long point_half = (unsigned long long)i << 32;
   if (cz < 0) {
-    slot_of[i] = cap;
+    slot_and_point[i] = point_half | cap;
     return;
   }
   const unsigned long long key =
@@ -167,40 +169,40 @@ __global__ __launch_bounds__(kBlock) void voxCellSlots(
       slot = (slot + 1) & (cap - 1);
     }
   }
-  slot_of[i] = slot;
+  slot_and_point[i] = point_half | slot;
 }
 
 // is_first[f] = 1 <=> point f is the first of its cell (the array was cleared by the fill; a
 // plain store per cell: a bitmap would take an atomic per cell, four times as long).
-__global__ __launch_bounds__(kBlock) void voxMarkFirst(const uint32_t *__restrict__ slot_sorted,
-                                                       const uint32_t *__restrict__ point_sorted,
+__global__ __launch_bounds__(kBlock) void voxMarkFirst(const unsigned long long *__restrict__ sorted,
                                                        int64_t n, uint32_t cap, uint32_t *is_first) {
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p >= n) return;
-  const uint32_t s = slot_sorted[p];
+  const unsigned long long mine = sorted[p];
+  const uint32_t s = (uint32_t)mine;
   if (s == cap) return;
-  if (p == 0 || slot_sorted[p - 1] != s) is_first[point_sorted[p]] = 1u;
+  if (p == 0 || (uint32_t)sorted[p - 1] != s) is_first[(uint32_t)(mine >> 32)] = 1u;
 }
 
 // First sorted position whose slot is `s`, which lies in front of position `from` (whose slot
 // is `s` as well): doubling steps backwards, then a binary search.
-__device__ inline int64_t headBefore(const uint32_t *__restrict__ slot_sorted, int64_t from, uint32_t s) {
-  int64_t hi = from;  // slot_sorted[hi] == s
+__device__ inline int64_t headBefore(const unsigned long long *__restrict__ sorted, int64_t from, uint32_t s) {
+  int64_t hi = from;  // sorted[hi] holds slot s
   int64_t step = 1;
   int64_t lo = hi - step;
-  while (lo >= 0 && slot_sorted[lo] == s) {
+  while (lo >= 0 && (uint32_t)sorted[lo] == s) {
     hi = lo;
     step *= 2;
     lo = hi - step;
   }
   if (lo < 0) {
-    if (slot_sorted[0] == s) return 0;
+    if ((uint32_t)sorted[0] == s) return 0;
     lo = 0;
   }
-  // slot_sorted[lo] != s, slot_sorted[hi] == s, the run starts in (lo, hi]
+  // sorted[lo] is another slot's, sorted[hi] this one's, the run starts in (lo, hi]
   while (hi - lo > 1) {
     const int64_t mid = lo + (hi - lo) / 2;
-    if (slot_sorted[mid] == s)
+    if ((uint32_t)sorted[mid] == s)
       hi = mid;
     else
       lo = mid;
@@ -213,8 +215,8 @@ __device__ inline int64_t headBefore(const uint32_t *__restrict__ slot_sorted, i
 // running maximum, and looked up behind the wave only by the lanes of a run that began earlier.
 __global__ __launch_bounds__(kBlock) void voxAssign(
     const float *__restrict__ points, const float *__restrict__ voxel_size,
-    const float *__restrict__ range, const uint32_t *__restrict__ slot_sorted,
-    const uint32_t *__restrict__ point_sorted, const uint32_t *__restrict__ is_first,
+    const float *__restrict__ range, const unsigned long long *__restrict__ sorted,
+    const uint32_t *__restrict__ is_first,
     const uint32_t *__restrict__ voxel_of_first, int64_t n, uint32_t cap, int num_features, int max_points,
     int max_voxels, float *voxels, int32_t *coors, int32_t *num_points_per_voxel, int32_t *voxel_num) {
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -225,8 +227,9 @@ __global__ __launch_bounds__(kBlock) void voxAssign(
     *voxel_num = cells < (uint32_t)max_voxels ? (int32_t)cells : max_voxels;
   }
   const bool live = p < n;
-  const uint32_t s = live ? slot_sorted[p] : cap;
-  const uint32_t before = (live && p > 0) ? slot_sorted[p - 1] : cap;
+  const unsigned long long mine = live ? sorted[p] : (unsigned long long)cap;
+  const uint32_t s = (uint32_t)mine;
+  const uint32_t before = (live && p > 0) ? (uint32_t)sorted[p - 1] : cap;
   const bool starts = live && s != cap && (p == 0 || before != s);
   // nearest run start at or below this lane, inside the wave (-1: none)
   long long head = starts ? (long long)p : -1;
@@ -236,13 +239,13 @@ __global__ __launch_bounds__(kBlock) void voxAssign(
     if (lane >= d && up > head) head = up;
   }
   if (!live || s == cap) return;
-  if (head < 0) head = headBefore(slot_sorted, p - lane, s);  // (position p - lane holds slot s too)
+  if (head < 0) head = headBefore(sorted, p - lane, s);  // (position p - lane holds slot s too)
   const int64_t r = p - head;
   if (r >= max_points) return;
-  const uint32_t f = point_sorted[head];
+  const uint32_t f = (uint32_t)(sorted[head] >> 32);
   const uint32_t v = voxel_of_first[f];  // first points in front of f
   if (v >= (uint32_t)max_voxels) return;
-  const uint32_t i = point_sorted[p];
+  const uint32_t i = (uint32_t)(mine >> 32);
   const float *src = points + (size_t)i * num_features;
   float *dst = voxels + ((size_t)v * max_points + r) * num_features;
   for (int k = 0; k < num_features; ++k) dst[k] = src[k];
@@ -256,7 +259,8 @@ __global__ __launch_bounds__(kBlock) void voxAssign(
 }
 
 struct Workspace {
-  uint32_t *slot_of, *point_of, *slot_sorted, *point_sorted, *is_first, *voxel_of_first;
+  unsigned long long *pairs_a, *pairs_b;  // table slot | point index << 32
+  uint32_t *is_first, *voxel_of_first;
   unsigned long long *keys;
   void *library;
   size_t total;
@@ -276,10 +280,8 @@ Workspace carve(void *base, const VoxelizeShape &s, size_t library_bytes) {
     return q;
   };
   Workspace w;
-  w.slot_of = reinterpret_cast<uint32_t *>(take(4 * n));
-  w.point_of = reinterpret_cast<uint32_t *>(take(4 * n));
-  w.slot_sorted = reinterpret_cast<uint32_t *>(take(4 * n));
-  w.point_sorted = reinterpret_cast<uint32_t *>(take(4 * n));
+  w.pairs_a = reinterpret_cast<unsigned long long *>(take(8 * n));
+  w.pairs_b = reinterpret_cast<unsigned long long *>(take(8 * n));
   w.is_first = reinterpret_cast<uint32_t *>(take(4 * n));
   w.voxel_of_first = reinterpret_cast<uint32_t *>(take(4 * n));
   w.keys = reinterpret_cast<unsigned long long *>(take(8 * (size_t)cap));
@@ -339,22 +341,21 @@ hipError_t launchVoxelize(const LaunchCtx &lc, const VoxelizeShape &s, const flo
   const int blocks = gridFor((size_t)n);
   lc.begin("voxCellSlots");
   voxCellSlots<<<blocks, kBlock, 0, lc.stream>>>(points, voxel_size, coors_range, n,
-                                                  s.num_features, w.keys, cap, w.slot_of, w.point_of);
+                                                  s.num_features, w.keys, cap, w.pairs_a);
   lc.end();
   if ((e = hipGetLastError()) != hipSuccess) return e;
 
   // points grouped by table slot, the points of a slot in their input order
   lc.begin("radixSortPairs");
   bool in_b = false;
-  e = device_sort::sortPairs<uint32_t>(lc.stream, w.library, w.slot_of, w.slot_sorted, w.point_of,
-                                       w.point_sorted, (size_t)n, bitsFor(cap), &in_b);
+  e = device_sort::sortKeys<unsigned long long>(lc.stream, w.library, w.pairs_a, w.pairs_b, (size_t)n,
+                                                bitsFor(cap), &in_b);
   lc.end();
   if (e != hipSuccess) return e;
-  const uint32_t *slot_sorted = in_b ? w.slot_sorted : w.slot_of;
-  const uint32_t *point_sorted = in_b ? w.point_sorted : w.point_of;
+  const unsigned long long *sorted = in_b ? w.pairs_b : w.pairs_a;
 
   lc.begin("voxMarkFirst");
-  voxMarkFirst<<<blocks, kBlock, 0, lc.stream>>>(slot_sorted, point_sorted, n, cap, w.is_first);
+  voxMarkFirst<<<blocks, kBlock, 0, lc.stream>>>(sorted, n, cap, w.is_first);
   lc.end();
   if ((e = hipGetLastError()) != hipSuccess) return e;
 
@@ -365,8 +366,7 @@ hipError_t launchVoxelize(const LaunchCtx &lc, const VoxelizeShape &s, const flo
   if (e != hipSuccess) return e;
 
   lc.begin("voxAssign");
-  voxAssign<<<blocks, kBlock, 0, lc.stream>>>(points, voxel_size, coors_range, slot_sorted, point_sorted,
-                                               w.is_first, w.voxel_of_first, n, cap, s.num_features,
+  voxAssign<<<blocks, kBlock, 0, lc.stream>>>(points, voxel_size, coors_range, sorted, w.is_first, w.voxel_of_first, n, cap, s.num_features,
                                                s.max_points, s.max_voxels, voxels, coors,
                                                num_points_per_voxel, voxel_num);
   lc.end();
