@@ -1248,7 +1248,7 @@ constexpr int kPlaceMaxChunks = 8;
 static int placeChunksPerGroup(int n_wave, int K) {
   const long chunks = (n_wave + kPlaceWaves - 1) / kPlaceWaves;
   int m = 1;
-  while (m < kPlaceMaxChunks && chunks * K / m > 16384) m *= 2;
+  while (m < kPlaceMaxChunks && chunks * K / m > 8192) m *= 2;
   return m;
 }
 // A thread takes the t-th staged pair of the chunk, whichever wave of rows staged it (most
