@@ -1809,7 +1809,12 @@ struct SliceTable {
 
 constexpr int kFilterStepPairs = 64;     // pairs multiplied per barrier
 constexpr int kFilterIndexChunk = 1024;  // pair indices resident in LDS at once
-constexpr int kFilterMaxSlices = 768;    // about three workgroups per CU
+constexpr int kFilterMaxSlices = 1024;   // about four workgroups per CU
+// Many offsets with short lists (5 x 5 x 5) are cut into fewer slices: every slice costs a
+// Ci x Co fp32 tile written and summed again (config 5a, 125 offsets: 137 us at 768 slices,
+// 149 at 1024; the 27-offset network layers: 183 -> 165 us at 128 channels, 89 -> 77 at 64).
+constexpr int kFilterMaxSlicesManyOffsets = 768;
+constexpr int kFilterFewOffsets = 32;
 
 // The order in which the workgroups take the slices: by the share of its offset's list that
 // lies in front of a slice, so that the workgroups running at one time are at about the same
@@ -2870,12 +2875,13 @@ bool filterMfmaShapeOk(const ConvProblem &p) {
   return ok(p.Ci) && ok(p.Co) && p.K <= kMaxInlineK;
 }
 
-// Slices the MFMA kernels cut the pair lists into at most: kFilterMaxSlices, or what a capped
-// workspace leaves beside one tile per offset.
+// Slices the MFMA kernels cut the pair lists into at most: kFilterMaxSlices (fewer for many
+// offsets), or what a capped workspace leaves beside one tile per offset.
 int filterMaxSlices(const ConvProblem &p) {
-  if (p.max_partial_tiles <= 0) return kFilterMaxSlices;
+  const int most = p.K <= kFilterFewOffsets ? kFilterMaxSlices : kFilterMaxSlicesManyOffsets;
+  if (p.max_partial_tiles <= 0) return most;
   const int room = p.max_partial_tiles - p.K;
-  return room < 1 ? 1 : (room > kFilterMaxSlices ? kFilterMaxSlices : room);
+  return room < 1 ? 1 : (room > most ? most : room);
 }
 
 int filterGradSplits(const ConvProblem &p) {
@@ -2997,7 +3003,12 @@ void launchFilterMfma(const LaunchCtx &lc, const ConvProblem &p, const FilterGra
     SliceTable tab;
     long long total = 0;
     for (int k = 0; k < p.K; ++k) total += inl.n[k];
-    const int max_slices = filterMaxSlices(p);
+    // (the larger number of slices only where they stay long: a fourth workgroup a CU does not
+    // fit, and a second round of short slices costs more than it spreads; config 3, 404 000
+    // pairs: 24 us at 701 slices, 31 us at 789)
+    int max_slices = filterMaxSlices(p);
+    if (total < (long long)kFilterMaxSlices * 2048 && max_slices > kFilterMaxSlicesManyOffsets)
+      max_slices = kFilterMaxSlicesManyOffsets;
     int slice_len = (int)((total + max_slices - 1) / max_slices);
     slice_len = (slice_len + kFilterStepPairs - 1) / kFilterStepPairs * kFilterStepPairs;
     // A slice has fixed costs (the first rows' round trip, a Ci x Co fp32 tile written and summed
