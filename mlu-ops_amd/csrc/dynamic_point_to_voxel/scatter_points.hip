@@ -160,9 +160,11 @@ __global__ __launch_bounds__(kBlock) void dpvHeads(const int32_t *__restrict__ c
 }
 
 // (`points` holds the sorted point indices `stride` words apart: 1, or 2 where they are the
-// high halves of sorted records)
+// high halves of sorted records; with records, a voxel's coordinates are unpacked from the
+// key half, bits1 and bits2 wide for the last two axes, instead of gathered from its first point)
 __global__ __launch_bounds__(kBlock) void dpvEmit(const int32_t *__restrict__ coors,
                                                   const uint32_t *__restrict__ points, int stride,
+                                                  bool keys_beside_points, int bits1, int bits2,
                                                   const uint32_t *__restrict__ head,
                                                   const uint32_t *__restrict__ triple_count, int n,
                                                   int rows, int32_t *point2voxel_map,
@@ -178,9 +180,16 @@ __global__ __launch_bounds__(kBlock) void dpvEmit(const int32_t *__restrict__ co
   if (head[p] && v >= 0 && v <= rows) {
     first_pos[v] = p;  // one past the last stored voxel included: it ends that voxel
     if (v < rows) {
-      voxel_coors[3 * (size_t)v] = coors[3 * (size_t)i];
-      voxel_coors[3 * (size_t)v + 1] = coors[3 * (size_t)i + 1];
-      voxel_coors[3 * (size_t)v + 2] = coors[3 * (size_t)i + 2];
+      if (keys_beside_points) {
+        const uint32_t key = points[(size_t)p * stride - 1];  // the low half of the record
+        voxel_coors[3 * (size_t)v] = (int32_t)(key >> (bits1 + bits2)) - 1;
+        voxel_coors[3 * (size_t)v + 1] = (int32_t)((key >> bits2) & ((1u << bits1) - 1u)) - 1;
+        voxel_coors[3 * (size_t)v + 2] = (int32_t)(key & ((1u << bits2) - 1u)) - 1;
+      } else {
+        voxel_coors[3 * (size_t)v] = coors[3 * (size_t)i];
+        voxel_coors[3 * (size_t)v + 1] = coors[3 * (size_t)i + 1];
+        voxel_coors[3 * (size_t)v + 2] = coors[3 * (size_t)i + 2];
+      }
     }
   }
   if (p == n - 1) *voxel_num = v + 1;
@@ -416,7 +425,8 @@ hipError_t launchScatterPoints(const LaunchCtx &lc, const ScatterShape &s, const
   if (e != hipSuccess) return e;
 
   lc.begin("dpvEmit");
-  dpvEmit<<<blocks, kBlock, 0, lc.stream>>>(coors, sorted_points, point_stride, w.head, w.triple_count, n,
+  dpvEmit<<<blocks, kBlock, 0, lc.stream>>>(coors, sorted_points, point_stride, record_points != nullptr,
+                                             bits[1], bits[2], w.head, w.triple_count, n,
                                              s.voxel_rows, point2voxel_map, voxel_coors,
                                              w.first_pos, voxel_num);
   lc.end();
